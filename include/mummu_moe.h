@@ -1,0 +1,193 @@
+/*
+ * mummu_moe.h - C ABI of the MI355X (gfx950) sparse mixture-of-experts block.
+ *
+ * One handle owns the device copy of a model's MoE blocks (router + expert banks of every
+ * layer) and a pre-sized workspace.  Every entry point returns an int status (0 = ok);
+ * mummu_moe_last_error() gives the message.  Nothing throws or aborts across this
+ * boundary.  Host-pointer entry points borrow the caller's buffers for the call only;
+ * *_device entry points take device pointers and only enqueue work on the given stream.
+ *
+ * Each declaration names the reference interface (physics515/Mummu, paths under
+ * crates/mummu/src/) that a binding would route here.
+ *
+ * Weight layout at this boundary is the GGUF payload, unchanged: expert-major, row-major,
+ * whole blocks per row - gate/up ne=[hidden, inter, E], down ne=[inter, hidden, E]
+ * (nn/moe.rs:22-30, models/qwen4exp/experts.rs:122-136); the router is row-major
+ * [E, hidden] (GGUF ffn_gate_inp, models/olmoe.rs:338-339).
+ */
+#ifndef MUMMU_MOE_H
+#define MUMMU_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MUMMU_API __attribute__((visibility("default")))
+
+/* ggml tensor type ids (gguf.rs:298-324).  Expert banks: F32, F16, BF16, Q8_0, Q4_K.
+ * Router: F32, F16, BF16. */
+enum mummu_ggml_type {
+    MUMMU_F32 = 0,
+    MUMMU_F16 = 1,
+    MUMMU_Q8_0 = 8,
+    MUMMU_Q4_K = 12,
+    MUMMU_BF16 = 30
+};
+
+enum mummu_status {
+    MUMMU_OK = 0,
+    MUMMU_ERR_CONFIG = 1,     /* nn/moe.rs:62-76, models/olmoe.rs:210-215: E<2, k outside 1..=E, zero sizes */
+    MUMMU_ERR_TYPE = 2,       /* tensor type this build has no kernel for */
+    MUMMU_ERR_BLOCKS = 3,     /* a row is not whole blocks (experts.rs:150-154) / bytes not whole blocks (gguf.rs:1411-1416) */
+    MUMMU_ERR_TOPK = 4,       /* top_k outside 1..=num_experts (nn/moe.rs:119-122, experts.rs:542-544) */
+    MUMMU_ERR_SHAPE = 5,      /* hidden width / row count mismatch (nn/moe.rs:123-126, experts.rs:380-385) */
+    MUMMU_ERR_NONFINITE = 6,  /* a router logit is inf or NaN (experts.rs:546-553) */
+    MUMMU_ERR_RANGE = 7,      /* layer or expert id out of range (experts.rs:996-1007, 1112-1117) */
+    MUMMU_ERR_NOT_LOADED = 8, /* the layer has no weights yet */
+    MUMMU_ERR_TOKENS = 9,     /* more tokens than the workspace was sized for */
+    MUMMU_ERR_DEVICE = 10,    /* no HIP device / a HIP call failed */
+    MUMMU_ERR_ARG = 11        /* null pointer or otherwise unusable argument */
+};
+
+/* Router arithmetic.  0: SparseMoe / SparseMoePerExpert (nn/moe.rs:144-150: f32 softmax,
+ * top-k, weights renormalised iff norm_topk_prob).  1: qwen4exp `route`
+ * (experts.rs:502-582: f64 normaliser, always renormalised with the 2^-14 floor). */
+enum mummu_router_flavour { MUMMU_ROUTER_SPARSE_MOE = 0, MUMMU_ROUTER_QWEN4EXP = 1 };
+
+/* SparseMoeConfig (nn/moe.rs:42-50) + the OlmoeConfig fields the block reads
+ * (models/olmoe.rs:52-66: num_experts, num_experts_per_tok, norm_topk_prob, rms_norm_eps). */
+typedef struct mummu_moe_config {
+    int32_t hidden_size;
+    int32_t expert_intermediate_size;
+    int32_t num_experts;
+    int32_t num_experts_per_tok; /* default top_k; entry points take top_k per call as the reference does */
+    int32_t norm_topk_prob;
+    int32_t router_flavour;      /* enum mummu_router_flavour */
+    int32_t num_layers;          /* MoE blocks held by this handle (>= 1) */
+    int32_t max_tokens;          /* largest b*t a call may pass; sizes the workspace */
+    float rms_norm_eps;          /* used only by mummu_moe_stack_forward* */
+} mummu_moe_config;
+
+typedef struct mummu_moe mummu_moe;
+
+/* Number of HIP devices visible to this process (0 when there is none). */
+MUMMU_API int mummu_device_count(void);
+
+/* Message of the last failure on this handle (or, for h == NULL, of the last failed call
+ * that had no handle, on this thread).  Never NULL. */
+MUMMU_API const char *mummu_moe_last_error(const mummu_moe *h);
+
+/* SparseMoeConfig::init (nn/moe.rs:61-99) minus the random weights: validates the config
+ * exactly as the reference asserts, then allocates the workspace on HIP device 0. */
+MUMMU_API int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out);
+MUMMU_API void mummu_moe_destroy(mummu_moe *h);
+
+/* The checked load of one block's tensors: `mlp.gate.weight` and
+ * `mlp.experts.{gate,up,down}` <- GGUF `ffn_gate_inp`, `ffn_{gate,up,down}_exps`
+ * (models/olmoe.rs:338-345; byte geometry ExpertBank::geometry, experts.rs:140-161).
+ * Host pointers, GGUF payload bytes.  rms_gamma (float[hidden], may be NULL) is the
+ * block's pre-norm weight (post_attention_layernorm, models/olmoe.rs:569). */
+MUMMU_API int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router_type, const void *gate,
+                                   int gate_type, const void *up, int up_type, const void *down, int down_type,
+                                   const float *rms_gamma);
+
+/* Bytes resident on the device for weights (ExpertExec::resident_bytes, nn/moe.rs:352). */
+MUMMU_API uint64_t mummu_moe_resident_bytes(const mummu_moe *h);
+
+/* SparseMoe::forward / SparseMoePerExpert::forward (nn/moe.rs:116, 214):
+ * x [n_tokens, hidden] f32 -> out [n_tokens, hidden] f32. */
+MUMMU_API int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n_tokens, int top_k,
+                                int norm_topk_prob, float *out);
+
+/* SparseMoePerExpert::route (nn/moe.rs:247-290): ids/weights [n_tokens, top_k] in slot
+ * (descending probability) order; logits [n_tokens, E] optional (may be NULL). */
+MUMMU_API int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n_tokens, int top_k,
+                              int norm_topk_prob, int32_t *ids, float *weights, float *logits);
+
+/* qwen4exp `route` on caller-supplied logits (experts.rs:541-582) or the SparseMoe router
+ * on them, per `flavour`.  No weights involved; n_experts is free. */
+MUMMU_API int mummu_route_logits(mummu_moe *h, const float *logits, int64_t n_tokens, int n_experts, int top_k,
+                                 int flavour, int norm_topk_prob, int32_t *ids, float *weights);
+
+/* RoutedExperts::routed_moe (experts.rs:1066-1076): route these logits (qwen4exp flavour),
+ * run the routed experts of `layer`, weighted sum in ascending expert id. */
+MUMMU_API int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const float *xs, int64_t n,
+                               int top_k, float *out);
+
+/* RoutedExperts::apply_routing (experts.rs:1092-1150) == SparseMoePerExpert::run_local
+ * (nn/moe.rs:296-328) == ExpertPool::run_layer (nn/moe.rs:1545-1607) for a given routing. */
+MUMMU_API int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const float *weights,
+                                      const float *xs, int64_t n, int top_k, float *out);
+
+/* ExpertExec::run (nn/moe.rs:357) / RoutedExperts::expert_ffn (experts.rs:1015-1057):
+ * SwiGLU of one expert on rows x hidden f32, row-major in and out. */
+MUMMU_API int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden,
+                               float *out);
+
+/* ExpertPool::take_hits (nn/moe.rs:1562-1564, 857-874): rows served per expert since the
+ * last take; hits is uint64[num_experts] and the counters reset. */
+MUMMU_API int mummu_moe_take_hits(mummu_moe *h, int layer, uint64_t *hits);
+
+/* The decoder layer's MoE half for every layer of the handle, models/olmoe.rs:566-572:
+ * x <- x + MoE_l(RmsNorm_l(x)), l = 0..num_layers-1.  x [n_tokens, hidden] f32 in,
+ * out the final residual stream.  ids (optional) receives [num_layers, n_tokens, top_k]. */
+MUMMU_API int mummu_moe_stack_forward(mummu_moe *h, const float *x, int64_t n_tokens, int top_k, int norm_topk_prob,
+                                      float *out, int32_t *ids);
+
+/* gguf::dequantize (gguf.rs:1403-1463) on the device: bytes -> f32, bit-exact.  Host
+ * buffers; out holds nbytes / block_bytes * block_size floats. */
+MUMMU_API int mummu_dequantize(int type, const void *bytes, size_t nbytes, float *out);
+
+/* Dequantize one expert's matrix FROM THE DEVICE COPY held by the handle (proves the
+ * resident bytes are the loaded bytes): which = 0 gate, 1 up, 2 down; out is
+ * [out_dim * in_dim] f32 on the host. */
+MUMMU_API int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, int expert, float *out);
+
+/* ---- device-pointer entry points (no host copies, no synchronisation) ------------------
+ * stream is a hipStream_t (NULL = the null stream).  Safe to capture into a HIP graph:
+ * no allocation, no memset node, no host readback.  A non-finite router logit cannot be
+ * reported synchronously here; mummu_moe_check() reads the flag back. */
+MUMMU_API int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_t n_tokens, int top_k,
+                                       int norm_topk_prob, float *out_dev, void *stream);
+MUMMU_API int mummu_moe_stack_forward_device(mummu_moe *h, const float *x_dev, int64_t n_tokens, int top_k,
+                                             int norm_topk_prob, float *out_dev, void *stream);
+/* Synchronises the stream and returns MUMMU_ERR_NONFINITE if any call since the last check
+ * saw a non-finite router logit, MUMMU_ERR_DEVICE on a HIP error, else MUMMU_OK. */
+MUMMU_API int mummu_moe_check(mummu_moe *h, void *stream);
+/* Device copies of the last call's routing: ids int32 [n, k], weights f32 [n, k]. */
+MUMMU_API int mummu_moe_last_routing(mummu_moe *h, int64_t n_tokens, int top_k, int32_t *ids, float *weights);
+
+/* ---- plumbing for harnesses that do not link HIP themselves -----------------------------*/
+MUMMU_API void *mummu_device_alloc(size_t bytes);
+MUMMU_API void mummu_device_free(void *p);
+MUMMU_API int mummu_copy_to_device(void *dst_dev, const void *src_host, size_t bytes);
+MUMMU_API int mummu_copy_to_host(void *dst_host, const void *src_dev, size_t bytes);
+MUMMU_API int mummu_device_synchronize(void);
+MUMMU_API int mummu_device_name(char *buf, size_t len);
+
+/* HIP-graph capture of whatever *_device calls are issued between begin and end on the
+ * handle's own stream; launch replays it there. */
+MUMMU_API void *mummu_moe_stream(mummu_moe *h);
+MUMMU_API int mummu_graph_begin(mummu_moe *h);
+MUMMU_API int mummu_graph_end(mummu_moe *h, void **graph_exec);
+MUMMU_API int mummu_graph_launch(mummu_moe *h, void *graph_exec);
+MUMMU_API void mummu_graph_destroy(void *graph_exec);
+
+/* HIP-event stopwatch on the handle's stream: elapsed milliseconds between start and stop. */
+MUMMU_API int mummu_timer_start(mummu_moe *h);
+MUMMU_API int mummu_timer_stop(mummu_moe *h, float *ms);
+
+/* Per-kernel timing: when enabled, every kernel launched by the *_device entry points on
+ * the handle's stream is bracketed by HIP events.  mummu_moe_kernel_times() synchronises and
+ * returns, per kernel slot, the summed milliseconds and the launch count since the last
+ * call; names[i] points at a static string.  Returns the number of slots written. */
+MUMMU_API int mummu_moe_kernel_timing(mummu_moe *h, int enable);
+MUMMU_API int mummu_moe_kernel_times(mummu_moe *h, const char **names, double *total_ms, int64_t *launches, int max_slots);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MUMMU_MOE_H */

@@ -1,0 +1,94 @@
+"""ctypes loader of ``lib/libmummu_moe.so`` (the HIP library behind include/mummu_moe.h).
+
+The library is built in-tree by ``python -m mummu_amd.build``.  Loading fails loudly when it
+is missing: there is no CPU fallback anywhere in this package.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmummu_moe.so")
+
+F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
+ROUTER_SPARSE_MOE, ROUTER_QWEN4EXP = 0, 1
+
+(OK, ERR_CONFIG, ERR_TYPE, ERR_BLOCKS, ERR_TOPK, ERR_SHAPE, ERR_NONFINITE, ERR_RANGE, ERR_NOT_LOADED, ERR_TOKENS,
+ ERR_DEVICE, ERR_ARG) = range(12)
+
+STATUS_NAMES = ["ok", "config", "type", "blocks", "topk", "shape", "nonfinite", "range", "not_loaded", "tokens",
+                "device", "arg"]
+
+
+class Config(C.Structure):
+    """mummu_moe_config."""
+    _fields_ = [
+        ("hidden_size", C.c_int32), ("expert_intermediate_size", C.c_int32), ("num_experts", C.c_int32),
+        ("num_experts_per_tok", C.c_int32), ("norm_topk_prob", C.c_int32), ("router_flavour", C.c_int32),
+        ("num_layers", C.c_int32), ("max_tokens", C.c_int32), ("rms_norm_eps", C.c_float),
+    ]
+
+
+# name -> (restype, argtypes); the list the header declares, checked against the .so by the tests
+_P, _I, _I64, _SZ = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
+SIGNATURES = {
+    "mummu_device_count": (_I, []),
+    "mummu_moe_last_error": (C.c_char_p, [_P]),
+    "mummu_moe_create": (_I, [C.POINTER(Config), C.POINTER(_P)]),
+    "mummu_moe_destroy": (None, [_P]),
+    "mummu_moe_load_layer": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P]),
+    "mummu_moe_resident_bytes": (C.c_uint64, [_P]),
+    "mummu_moe_forward": (_I, [_P, _I, _P, _I64, _I, _I, _P]),
+    "mummu_moe_route": (_I, [_P, _I, _P, _I64, _I, _I, _P, _P, _P]),
+    "mummu_route_logits": (_I, [_P, _P, _I64, _I, _I, _I, _I, _P, _P]),
+    "mummu_moe_routed": (_I, [_P, _I, _P, _P, _I64, _I, _P]),
+    "mummu_moe_apply_routing": (_I, [_P, _I, _P, _P, _P, _I64, _I, _P]),
+    "mummu_expert_run": (_I, [_P, _I, _I, _P, _I64, _I, _P]),
+    "mummu_moe_take_hits": (_I, [_P, _I, _P]),
+    "mummu_moe_stack_forward": (_I, [_P, _P, _I64, _I, _I, _P, _P]),
+    "mummu_dequantize": (_I, [_I, _P, _SZ, _P]),
+    "mummu_moe_dequantize_expert": (_I, [_P, _I, _I, _I, _P]),
+    "mummu_moe_forward_device": (_I, [_P, _I, _P, _I64, _I, _I, _P, _P]),
+    "mummu_moe_stack_forward_device": (_I, [_P, _P, _I64, _I, _I, _P, _P]),
+    "mummu_moe_check": (_I, [_P, _P]),
+    "mummu_moe_last_routing": (_I, [_P, _I64, _I, _P, _P]),
+    "mummu_device_alloc": (_P, [_SZ]),
+    "mummu_device_free": (None, [_P]),
+    "mummu_copy_to_device": (_I, [_P, _P, _SZ]),
+    "mummu_copy_to_host": (_I, [_P, _P, _SZ]),
+    "mummu_device_synchronize": (_I, []),
+    "mummu_device_name": (_I, [C.c_char_p, _SZ]),
+    "mummu_moe_stream": (_P, [_P]),
+    "mummu_graph_begin": (_I, [_P]),
+    "mummu_graph_end": (_I, [_P, C.POINTER(_P)]),
+    "mummu_graph_launch": (_I, [_P, _P]),
+    "mummu_graph_destroy": (None, [_P]),
+    "mummu_timer_start": (_I, [_P]),
+    "mummu_timer_stop": (_I, [_P, C.POINTER(C.c_float)]),
+    "mummu_moe_kernel_timing": (_I, [_P, _I]),
+    "mummu_moe_kernel_times": (_I, [_P, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(C.c_int64), _I]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """The HIP library, loaded once.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build the HIP library first (python -m mummu_amd.build). "
+                "This package has no CPU path.")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def device_count() -> int:
+    return load().mummu_device_count()

@@ -1,0 +1,770 @@
+// C ABI of the sparse MoE block (include/mummu_moe.h): handle, weight residency, workspace,
+// and the launch sequences.  Host logic only; the arithmetic lives in the kernel files.
+#include "../../include/mummu_moe.h"
+
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "device_utils.h"
+#include "kernels.h"
+
+using namespace mummu;
+
+namespace {
+
+thread_local std::string g_error;  // failures of calls that have no handle
+
+enum KernelSlot { K_ROUTER_LOGITS, K_ROUTE_TOPK, K_GATE_UP, K_DOWN, K_COMBINE, K_RMSNORM, K_SLOTS };
+const char *const kSlotNames[K_SLOTS] = {"router_logits", "route_topk", "gate_up", "down", "combine", "rmsnorm"};
+
+struct Layer {
+    void *router = nullptr;
+    int router_type = 0;
+    uint8_t *gate = nullptr, *up = nullptr, *down = nullptr;
+    int gate_type = 0, up_type = 0, down_type = 0;
+    float *gamma = nullptr;
+    unsigned long long *hits = nullptr;
+    size_t bytes = 0;
+    bool loaded = false;
+};
+
+struct TimedLaunch {
+    hipEvent_t start, stop;
+    int slot;
+};
+
+}  // namespace
+
+struct mummu_moe {
+    mummu_moe_config cfg{};
+    std::vector<Layer> layers;
+    hipStream_t stream = nullptr;
+    std::mutex mu;
+    mutable std::string err;
+
+    // workspace (device)
+    int64_t ws_tokens = 0, ws_assign = 0;
+    int ws_experts = 0;
+    float *logits = nullptr, *weights = nullptr, *act = nullptr, *y = nullptr;
+    int32_t *ids = nullptr, *flags = nullptr;
+    float *xin = nullptr, *xout = nullptr, *h2 = nullptr, *resid[2] = {nullptr, nullptr};
+
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    bool timing = false;
+    std::vector<TimedLaunch> timed;
+    std::vector<hipEvent_t> event_pool;
+};
+
+namespace {
+
+int fail(mummu_moe *h, int code, const std::string &msg) {
+    if (h) h->err = msg;
+    else g_error = msg;
+    return code;
+}
+
+#define HIPCHK(h, call)                                                                                    \
+    do {                                                                                                   \
+        hipError_t e_ = (call);                                                                            \
+        if (e_ != hipSuccess)                                                                              \
+            return fail(h, MUMMU_ERR_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_));            \
+    } while (0)
+
+bool bank_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16 || t == T_Q8_0 || t == T_Q4_K; }
+bool router_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16; }
+size_t row_bytes_of(int t, int in_dim) { return (size_t)(in_dim / block_elems(t)) * (size_t)block_bytes(t); }
+
+void free_ws(mummu_moe *h) {
+    void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1]};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    h->logits = h->weights = h->act = h->y = h->xin = h->xout = h->h2 = h->resid[0] = h->resid[1] = nullptr;
+    h->ids = nullptr;
+    h->ws_tokens = h->ws_assign = 0;
+    h->ws_experts = 0;
+}
+
+// Grow the workspace to hold n tokens and n_assign (token, expert) pairs.  Host entry points
+// only: synchronises and reallocates.
+int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
+    if (n_experts < h->cfg.num_experts) n_experts = h->cfg.num_experts;
+    if (n <= h->ws_tokens && n_assign <= h->ws_assign && n_experts <= h->ws_experts) return MUMMU_OK;
+    HIPCHK(h, hipDeviceSynchronize());
+    int64_t nt = n > h->ws_tokens ? n : h->ws_tokens;
+    int64_t na = n_assign > h->ws_assign ? n_assign : h->ws_assign;
+    if (n_experts < h->ws_experts) n_experts = h->ws_experts;
+    free_ws(h);
+    const size_t H = (size_t)h->cfg.hidden_size, I = (size_t)h->cfg.expert_intermediate_size;
+    const size_t E = (size_t)n_experts;
+    HIPCHK(h, hipMalloc(&h->logits, sizeof(float) * (size_t)nt * E));
+    HIPCHK(h, hipMalloc(&h->ids, sizeof(int32_t) * (size_t)na));
+    HIPCHK(h, hipMalloc(&h->weights, sizeof(float) * (size_t)na));
+    HIPCHK(h, hipMalloc(&h->act, sizeof(float) * (size_t)na * I));
+    HIPCHK(h, hipMalloc(&h->y, sizeof(float) * (size_t)na * H));
+    HIPCHK(h, hipMalloc(&h->xin, sizeof(float) * (size_t)nt * H));
+    HIPCHK(h, hipMalloc(&h->xout, sizeof(float) * (size_t)nt * H));
+    HIPCHK(h, hipMalloc(&h->h2, sizeof(float) * (size_t)nt * H));
+    HIPCHK(h, hipMalloc(&h->resid[0], sizeof(float) * (size_t)nt * H));
+    HIPCHK(h, hipMalloc(&h->resid[1], sizeof(float) * (size_t)nt * H));
+    h->ws_tokens = nt;
+    h->ws_assign = na;
+    h->ws_experts = n_experts;
+    return MUMMU_OK;
+}
+
+int reset_flags(mummu_moe *h) {
+    const int32_t init[4] = {0, INT_MAX, 0, 0};
+    HIPCHK(h, hipMemcpy(h->flags, init, sizeof(init), hipMemcpyHostToDevice));
+    return MUMMU_OK;
+}
+
+// Synchronise and translate the device error flags.
+int check_flags(mummu_moe *h, hipStream_t s) {
+    HIPCHK(h, hipStreamSynchronize(s));
+    int32_t f[4];
+    HIPCHK(h, hipMemcpy(f, h->flags, sizeof(f), hipMemcpyDeviceToHost));
+    if (f[FLAG_NONFINITE] == 0 && f[FLAG_BAD_ID] == 0) return MUMMU_OK;
+    int rc = reset_flags(h);
+    if (rc != MUMMU_OK) return rc;
+    if (f[FLAG_NONFINITE]) {
+        const int E = h->cfg.num_experts;
+        char buf[160];
+        snprintf(buf, sizeof(buf), "router logit for token %d expert %d is not finite", f[FLAG_NONFINITE_INDEX] / E,
+                 f[FLAG_NONFINITE_INDEX] % E);
+        return fail(h, MUMMU_ERR_NONFINITE, buf);
+    }
+    return fail(h, MUMMU_ERR_RANGE, "a routed expert id is out of range");
+}
+
+struct ScopedTimer {
+    mummu_moe *h;
+    hipStream_t s;
+    hipEvent_t stop = nullptr;
+    ScopedTimer(mummu_moe *h_, hipStream_t s_, int slot) : h(h_), s(s_) {
+        if (!h->timing) return;
+        hipEvent_t ev[2];
+        for (auto &e : ev) {
+            if (!h->event_pool.empty()) {
+                e = h->event_pool.back();
+                h->event_pool.pop_back();
+            } else if (hipEventCreate(&e) != hipSuccess) {
+                return;
+            }
+        }
+        (void)hipEventRecord(ev[0], s);
+        stop = ev[1];
+        h->timed.push_back({ev[0], ev[1], slot});
+    }
+    ~ScopedTimer() {
+        if (stop) (void)hipEventRecord(stop, s);
+    }
+};
+
+#define LAUNCH(h, slot, s, call)                                                                 \
+    do {                                                                                         \
+        hipError_t e_;                                                                           \
+        {                                                                                        \
+            ScopedTimer timer_(h, s, slot);                                                      \
+            e_ = (call);                                                                         \
+        }                                                                                        \
+        if (e_ != hipSuccess)                                                                    \
+            return fail(h, MUMMU_ERR_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_));  \
+    } while (0)
+
+ExpertBanks banks_of(const mummu_moe *h, const Layer &L) {
+    ExpertBanks b;
+    b.gate = L.gate;
+    b.up = L.up;
+    b.down = L.down;
+    b.gate_type = L.gate_type;
+    b.up_type = L.up_type;
+    b.down_type = L.down_type;
+    b.hidden = h->cfg.hidden_size;
+    b.inter = h->cfg.expert_intermediate_size;
+    b.n_experts = h->cfg.num_experts;
+    return b;
+}
+
+int check_layer(mummu_moe *h, int layer) {
+    if (layer < 0 || layer >= (int)h->layers.size())
+        return fail(h, MUMMU_ERR_RANGE, "layer " + std::to_string(layer) + " out of range (" + std::to_string(h->layers.size()) + ")");
+    if (!h->layers[layer].loaded) return fail(h, MUMMU_ERR_NOT_LOADED, "layer " + std::to_string(layer) + " has no weights");
+    return MUMMU_OK;
+}
+
+int check_topk(mummu_moe *h, int top_k, int n_experts) {
+    if (top_k < 1 || top_k > n_experts)
+        return fail(h, MUMMU_ERR_TOPK, "MoE forward: top_k (" + std::to_string(top_k) + ") must be in 1..=num_experts (" +
+                                           std::to_string(n_experts) + ")");
+    return MUMMU_OK;
+}
+
+// experts of an already-made routing: gate/up -> down -> combine
+int run_experts(mummu_moe *h, const Layer &L, const float *x, int64_t n, int k, const float *residual, float *out,
+                hipStream_t s) {
+    ExpertBanks b = banks_of(h, L);
+    const int na = (int)(n * k);
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x, h->ids, na, k, -1, h->act, h->flags, s));
+    LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->ids, na, -1, h->y, s));
+    LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, (int)n, k, b.hidden, residual, out, s));
+    return MUMMU_OK;
+}
+
+int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
+                 hipStream_t s) {
+    const Layer &L = h->layers[layer];
+    const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
+    LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, s));
+    LAUNCH(h, K_ROUTE_TOPK, s,
+           launch_route_topk(h->logits, (int)n, E, k, h->cfg.router_flavour, norm, h->ids, h->weights, L.hits, h->flags, s));
+    return run_experts(h, L, x, n, k, residual, out, s);
+}
+
+int check_device_call(mummu_moe *h, int64_t n, int k, const void *a, const void *b) {
+    if (!a || !b) return fail(h, MUMMU_ERR_ARG, "null device pointer");
+    if (((uintptr_t)a & 15) || ((uintptr_t)b & 15)) return fail(h, MUMMU_ERR_ARG, "device buffers must be 16-byte aligned");
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n > h->ws_tokens || n * k > h->ws_assign)
+        return fail(h, MUMMU_ERR_TOKENS, std::to_string(n) + " tokens x top_k " + std::to_string(k) +
+                                             " exceeds the workspace (max_tokens " + std::to_string(h->ws_tokens) + ", pairs " +
+                                             std::to_string(h->ws_assign) + ")");
+    return MUMMU_OK;
+}
+
+int stack_impl(mummu_moe *h, const float *x, int64_t n, int k, int norm, float *out, hipStream_t s, int32_t *ids_host) {
+    const int nl = (int)h->layers.size(), H = h->cfg.hidden_size;
+    for (int l = 0; l < nl; l++) {
+        int rc = check_layer(h, l);
+        if (rc) return rc;
+        if (!h->layers[l].gamma) return fail(h, MUMMU_ERR_NOT_LOADED, "layer " + std::to_string(l) + " has no RmsNorm weight");
+    }
+    for (int l = 0; l < nl; l++) {
+        const float *src = l == 0 ? x : h->resid[(l - 1) & 1];
+        float *dst = l == nl - 1 ? out : h->resid[l & 1];
+        LAUNCH(h, K_RMSNORM, s, launch_rmsnorm(src, h->layers[l].gamma, h->cfg.rms_norm_eps, (int)n, H, h->h2, s));
+        int rc = forward_impl(h, l, h->h2, n, k, norm, src, dst, s);
+        if (rc) return rc;
+        if (ids_host) {
+            HIPCHK(h, hipStreamSynchronize(s));
+            HIPCHK(h, hipMemcpy(ids_host + (size_t)l * n * k, h->ids, sizeof(int32_t) * (size_t)(n * k), hipMemcpyDeviceToHost));
+        }
+    }
+    return MUMMU_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mummu_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+const char *mummu_moe_last_error(const mummu_moe *h) { return h ? h->err.c_str() : g_error.c_str(); }
+
+int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
+    if (!cfg || !out) return fail(nullptr, MUMMU_ERR_ARG, "null config or output pointer");
+    *out = nullptr;
+    // nn/moe.rs:62-76
+    if (cfg->num_experts < 2)
+        return fail(nullptr, MUMMU_ERR_CONFIG,
+                    "MoE: num_experts must be >= 2 (got " + std::to_string(cfg->num_experts) + "); use SwiGluMlp for a dense FFN");
+    if (cfg->num_experts_per_tok < 1 || cfg->num_experts_per_tok > cfg->num_experts)
+        return fail(nullptr, MUMMU_ERR_CONFIG, "MoE: num_experts_per_tok (" + std::to_string(cfg->num_experts_per_tok) +
+                                                   ") must be in 1..=num_experts (" + std::to_string(cfg->num_experts) + ")");
+    if (cfg->hidden_size < 1 || cfg->expert_intermediate_size < 1)
+        return fail(nullptr, MUMMU_ERR_CONFIG, "MoE: hidden_size and expert_intermediate_size must be >= 1");
+    if (cfg->num_experts > 512) return fail(nullptr, MUMMU_ERR_CONFIG, "MoE: this build routes over at most 512 experts");
+    if (cfg->num_layers < 1 || cfg->max_tokens < 1) return fail(nullptr, MUMMU_ERR_CONFIG, "MoE: num_layers and max_tokens must be >= 1");
+    if (cfg->router_flavour != MUMMU_ROUTER_SPARSE_MOE && cfg->router_flavour != MUMMU_ROUTER_QWEN4EXP)
+        return fail(nullptr, MUMMU_ERR_CONFIG, "MoE: unknown router_flavour");
+    if (mummu_device_count() < 1) return fail(nullptr, MUMMU_ERR_DEVICE, "no HIP device visible to this process");
+
+    mummu_moe *h = new mummu_moe();
+    h->cfg = *cfg;
+    h->layers.resize((size_t)cfg->num_layers);
+    auto bail = [&](int rc) {
+        g_error = h->err;
+        mummu_moe_destroy(h);
+        return rc;
+    };
+    if (hipSetDevice(0) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipSetDevice(0) failed"));
+    if (hipStreamCreate(&h->stream) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipStreamCreate failed"));
+    if (hipEventCreate(&h->t0) != hipSuccess || hipEventCreate(&h->t1) != hipSuccess)
+        return bail(fail(h, MUMMU_ERR_DEVICE, "hipEventCreate failed"));
+    if (hipMalloc(&h->flags, sizeof(int32_t) * 4) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(flags) failed"));
+    int rc = reset_flags(h);
+    if (rc) return bail(rc);
+    rc = ensure_ws(h, cfg->max_tokens, (int64_t)cfg->max_tokens * cfg->num_experts_per_tok, cfg->num_experts);
+    if (rc) return bail(rc);
+    *out = h;
+    return MUMMU_OK;
+}
+
+void mummu_moe_destroy(mummu_moe *h) {
+    if (!h) return;
+    (void)hipDeviceSynchronize();
+    for (Layer &L : h->layers) {
+        void *ptrs[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits};
+        for (void *p : ptrs)
+            if (p) (void)hipFree(p);
+    }
+    free_ws(h);
+    if (h->flags) (void)hipFree(h->flags);
+    for (auto &t : h->timed) {
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
+    for (auto e : h->event_pool) (void)hipEventDestroy(e);
+    if (h->t0) (void)hipEventDestroy(h->t0);
+    if (h->t1) (void)hipEventDestroy(h->t1);
+    if (h->stream) (void)hipStreamDestroy(h->stream);
+    delete h;
+}
+
+int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router_type, const void *gate, int gate_type,
+                         const void *up, int up_type, const void *down, int down_type, const float *rms_gamma) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    if (layer < 0 || layer >= (int)h->layers.size())
+        return fail(h, MUMMU_ERR_RANGE, "layer " + std::to_string(layer) + " out of range (" + std::to_string(h->layers.size()) + ")");
+    if (!router || !gate || !up || !down) return fail(h, MUMMU_ERR_ARG, "null weight pointer");
+    if (!router_type_ok(router_type)) return fail(h, MUMMU_ERR_TYPE, "router must be F32, F16 or BF16 (got ggml type " + std::to_string(router_type) + ")");
+    for (int t : {gate_type, up_type, down_type})
+        if (!bank_type_ok(t)) return fail(h, MUMMU_ERR_TYPE, "no expert kernel for ggml type " + std::to_string(t));
+    if (gate_type != up_type) return fail(h, MUMMU_ERR_TYPE, "gate and up banks must share one type");
+    const int H = h->cfg.hidden_size, I = h->cfg.expert_intermediate_size, E = h->cfg.num_experts;
+    // experts.rs:150-154: a row that is not whole blocks cannot be sliced out of the bank
+    if (H % block_elems(gate_type))
+        return fail(h, MUMMU_ERR_BLOCKS, "row width " + std::to_string(H) + " is not whole blocks of " + std::to_string(block_elems(gate_type)));
+    if (I % block_elems(down_type))
+        return fail(h, MUMMU_ERR_BLOCKS, "row width " + std::to_string(I) + " is not whole blocks of " + std::to_string(block_elems(down_type)));
+    if ((gate_type == T_Q4_K || gate_type == T_Q8_0) && H / 32 > 256)
+        return fail(h, MUMMU_ERR_CONFIG, "quantized rows wider than 8192 are not supported");
+    if ((down_type == T_Q4_K || down_type == T_Q8_0) && I / 32 > 256)
+        return fail(h, MUMMU_ERR_CONFIG, "quantized rows wider than 8192 are not supported");
+
+    Layer &L = h->layers[layer];
+    HIPCHK(h, hipDeviceSynchronize());
+    void *old[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits};
+    for (void *p : old)
+        if (p) (void)hipFree(p);
+    L = Layer();
+    const size_t rb = (size_t)E * (size_t)H * (size_t)block_bytes(router_type);
+    const size_t gb = (size_t)E * (size_t)I * row_bytes_of(gate_type, H);
+    const size_t ub = (size_t)E * (size_t)I * row_bytes_of(up_type, H);
+    const size_t db = (size_t)E * (size_t)H * row_bytes_of(down_type, I);
+    HIPCHK(h, hipMalloc(&L.router, rb));
+    HIPCHK(h, hipMalloc(&L.gate, gb));
+    HIPCHK(h, hipMalloc(&L.up, ub));
+    HIPCHK(h, hipMalloc(&L.down, db));
+    HIPCHK(h, hipMalloc(&L.hits, sizeof(unsigned long long) * (size_t)E));
+    HIPCHK(h, hipMemcpy(L.router, router, rb, hipMemcpyHostToDevice));
+    HIPCHK(h, hipMemcpy(L.gate, gate, gb, hipMemcpyHostToDevice));
+    HIPCHK(h, hipMemcpy(L.up, up, ub, hipMemcpyHostToDevice));
+    HIPCHK(h, hipMemcpy(L.down, down, db, hipMemcpyHostToDevice));
+    HIPCHK(h, hipMemset(L.hits, 0, sizeof(unsigned long long) * (size_t)E));
+    if (rms_gamma) {
+        HIPCHK(h, hipMalloc(&L.gamma, sizeof(float) * (size_t)H));
+        HIPCHK(h, hipMemcpy(L.gamma, rms_gamma, sizeof(float) * (size_t)H, hipMemcpyHostToDevice));
+    }
+    L.router_type = router_type;
+    L.gate_type = gate_type;
+    L.up_type = up_type;
+    L.down_type = down_type;
+    L.bytes = rb + gb + ub + db + (rms_gamma ? sizeof(float) * (size_t)H : 0);
+    L.loaded = true;
+    return MUMMU_OK;
+}
+
+uint64_t mummu_moe_resident_bytes(const mummu_moe *h) {
+    if (!h) return 0;
+    uint64_t total = 0;
+    for (const Layer &L : h->layers) total += L.bytes;
+    return total;
+}
+
+int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n, int top_k, int norm, float *out) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (!x || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
+    const size_t bytes = sizeof(float) * (size_t)n * (size_t)h->cfg.hidden_size;
+    HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, h->stream));
+    if ((rc = forward_impl(h, layer, h->xin, n, top_k, norm, nullptr, h->xout, h->stream))) return rc;
+    if ((rc = check_flags(h, h->stream))) return rc;
+    HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_k, int norm, int32_t *ids, float *weights,
+                    float *logits) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (!x || !ids || !weights) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
+    const Layer &L = h->layers[layer];
+    const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
+    hipStream_t s = h->stream;
+    HIPCHK(h, hipMemcpyAsync(h->xin, x, sizeof(float) * (size_t)n * H, hipMemcpyHostToDevice, s));
+    LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(h->xin, L.router, L.router_type, h->logits, (int)n, H, E, s));
+    LAUNCH(h, K_ROUTE_TOPK, s,
+           launch_route_topk(h->logits, (int)n, E, top_k, h->cfg.router_flavour, norm, h->ids, h->weights, nullptr, h->flags, s));
+    if (logits) HIPCHK(h, hipMemcpyAsync(logits, h->logits, sizeof(float) * (size_t)n * E, hipMemcpyDeviceToHost, s));
+    if ((rc = check_flags(h, s))) return rc;
+    HIPCHK(h, hipMemcpy(ids, h->ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    HIPCHK(h, hipMemcpy(weights, h->weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_route_logits(mummu_moe *h, const float *logits, int64_t n, int n_experts, int top_k, int flavour, int norm,
+                       int32_t *ids, float *weights) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    // experts.rs:542-544
+    if (n_experts <= 0 || top_k <= 0 || top_k > n_experts)
+        return fail(h, MUMMU_ERR_TOPK, "top-" + std::to_string(top_k) + " of " + std::to_string(n_experts) + " experts is not a routing");
+    if (n_experts > 512) return fail(h, MUMMU_ERR_CONFIG, "this build routes over at most 512 experts");
+    if (flavour != MUMMU_ROUTER_SPARSE_MOE && flavour != MUMMU_ROUTER_QWEN4EXP) return fail(h, MUMMU_ERR_CONFIG, "unknown router flavour");
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (!logits || !ids || !weights) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    int rc = ensure_ws(h, n, n * top_k, n_experts);
+    if (rc) return rc;
+    hipStream_t s = h->stream;
+    HIPCHK(h, hipMemcpyAsync(h->logits, logits, sizeof(float) * (size_t)n * n_experts, hipMemcpyHostToDevice, s));
+    LAUNCH(h, K_ROUTE_TOPK, s, launch_route_topk(h->logits, (int)n, n_experts, top_k, flavour, norm, h->ids, h->weights, nullptr, h->flags, s));
+    HIPCHK(h, hipStreamSynchronize(s));
+    int32_t f[4];
+    HIPCHK(h, hipMemcpy(f, h->flags, sizeof(f), hipMemcpyDeviceToHost));
+    if (f[FLAG_NONFINITE]) {
+        if ((rc = reset_flags(h))) return rc;
+        char buf[160];
+        snprintf(buf, sizeof(buf), "router logit for token %d expert %d is not finite", f[FLAG_NONFINITE_INDEX] / n_experts,
+                 f[FLAG_NONFINITE_INDEX] % n_experts);
+        return fail(h, MUMMU_ERR_NONFINITE, buf);
+    }
+    HIPCHK(h, hipMemcpy(ids, h->ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    HIPCHK(h, hipMemcpy(weights, h->weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const float *weights, const float *xs, int64_t n,
+                            int top_k, float *out) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (!ids || !weights || !xs || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    // experts.rs:1111-1117
+    for (int64_t i = 0; i < n * top_k; i++)
+        if (ids[i] < 0 || ids[i] >= h->cfg.num_experts)
+            return fail(h, MUMMU_ERR_RANGE, "routed expert " + std::to_string(ids[i]) + " out of range (" + std::to_string(h->cfg.num_experts) + ")");
+    if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
+    hipStream_t s = h->stream;
+    const size_t bytes = sizeof(float) * (size_t)n * (size_t)h->cfg.hidden_size;
+    HIPCHK(h, hipMemcpyAsync(h->xin, xs, bytes, hipMemcpyHostToDevice, s));
+    HIPCHK(h, hipMemcpyAsync(h->ids, ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyHostToDevice, s));
+    HIPCHK(h, hipMemcpyAsync(h->weights, weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyHostToDevice, s));
+    Layer &L = h->layers[layer];
+    // hit counters, nn/moe.rs:1562-1564 (the routing came from the host, so count here)
+    {
+        std::vector<unsigned long long> add((size_t)h->cfg.num_experts, 0), cur((size_t)h->cfg.num_experts);
+        for (int64_t i = 0; i < n * top_k; i++) add[(size_t)ids[i]]++;
+        HIPCHK(h, hipStreamSynchronize(s));
+        HIPCHK(h, hipMemcpy(cur.data(), L.hits, sizeof(unsigned long long) * cur.size(), hipMemcpyDeviceToHost));
+        for (size_t e = 0; e < cur.size(); e++) cur[e] += add[e];
+        HIPCHK(h, hipMemcpy(L.hits, cur.data(), sizeof(unsigned long long) * cur.size(), hipMemcpyHostToDevice));
+    }
+    if ((rc = run_experts(h, L, h->xin, n, top_k, nullptr, h->xout, s))) return rc;
+    if ((rc = check_flags(h, s))) return rc;
+    HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const float *xs, int64_t n, int top_k, float *out) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    int rc;
+    {
+        std::lock_guard<std::mutex> lock(h->mu);
+        if ((rc = check_layer(h, layer))) return rc;
+    }
+    if (n <= 0) return n < 0 ? fail(h, MUMMU_ERR_SHAPE, "negative token count") : MUMMU_OK;
+    if (top_k < 1 || top_k > h->cfg.num_experts) return check_topk(h, top_k, h->cfg.num_experts);
+    std::vector<int32_t> ids((size_t)(n * top_k));
+    std::vector<float> w((size_t)(n * top_k));
+    if ((rc = mummu_route_logits(h, router_logits, n, h->cfg.num_experts, top_k, MUMMU_ROUTER_QWEN4EXP, 1, ids.data(), w.data()))) return rc;
+    return mummu_moe_apply_routing(h, layer, ids.data(), w.data(), xs, n, top_k, out);
+}
+
+int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden, float *out) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if (expert < 0 || expert >= h->cfg.num_experts)
+        return fail(h, MUMMU_ERR_RANGE, "expert " + std::to_string(expert) + " out of range (" + std::to_string(h->cfg.num_experts) + ")");
+    if (hidden != h->cfg.hidden_size)
+        return fail(h, MUMMU_ERR_SHAPE, "input hidden " + std::to_string(hidden) + " does not match expert hidden " + std::to_string(h->cfg.hidden_size));
+    if (rows < 0) return fail(h, MUMMU_ERR_SHAPE, "negative row count");
+    if (rows == 0) return MUMMU_OK;
+    if (!x || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if ((rc = ensure_ws(h, rows, rows, 0))) return rc;
+    hipStream_t s = h->stream;
+    const size_t bytes = sizeof(float) * (size_t)rows * (size_t)hidden;
+    HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, s));
+    ExpertBanks b = banks_of(h, h->layers[layer]);
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, h->xin, nullptr, (int)rows, 1, expert, h->act, h->flags, s));
+    LAUNCH(h, K_DOWN, s, launch_down(b, h->act, nullptr, (int)rows, expert, h->y, s));
+    HIPCHK(h, hipStreamSynchronize(s));
+    HIPCHK(h, hipMemcpy(out, h->y, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_moe_take_hits(mummu_moe *h, int layer, uint64_t *hits) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if (!hits) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    Layer &L = h->layers[layer];
+    HIPCHK(h, hipDeviceSynchronize());
+    HIPCHK(h, hipMemcpy(hits, L.hits, sizeof(uint64_t) * (size_t)h->cfg.num_experts, hipMemcpyDeviceToHost));
+    HIPCHK(h, hipMemset(L.hits, 0, sizeof(uint64_t) * (size_t)h->cfg.num_experts));
+    return MUMMU_OK;
+}
+
+int mummu_moe_stack_forward(mummu_moe *h, const float *x, int64_t n, int top_k, int norm, float *out, int32_t *ids) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_topk(h, top_k, h->cfg.num_experts);
+    if (rc) return rc;
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (!x || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
+    const size_t bytes = sizeof(float) * (size_t)n * (size_t)h->cfg.hidden_size;
+    HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, h->stream));
+    if ((rc = stack_impl(h, h->xin, n, top_k, norm, h->xout, h->stream, ids))) return rc;
+    if ((rc = check_flags(h, h->stream))) return rc;
+    HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_dequantize(int type, const void *bytes, size_t nbytes, float *out) {
+    if (!bank_type_ok(type)) return fail(nullptr, MUMMU_ERR_TYPE, "dequant for ggml type " + std::to_string(type) + " is not implemented");
+    const size_t bpb = (size_t)block_bytes(type);
+    // gguf.rs:1411-1416
+    if (nbytes == 0 || nbytes % bpb != 0)
+        return fail(nullptr, MUMMU_ERR_BLOCKS, std::to_string(nbytes) + " bytes is not whole blocks of " + std::to_string(bpb));
+    if (!bytes || !out) return fail(nullptr, MUMMU_ERR_ARG, "null buffer");
+    if (mummu_device_count() < 1) return fail(nullptr, MUMMU_ERR_DEVICE, "no HIP device visible to this process");
+    const size_t blocks = nbytes / bpb, n = blocks * (size_t)block_elems(type);
+    uint8_t *d_in = nullptr;
+    float *d_out = nullptr;
+    mummu_moe *h = nullptr;
+    HIPCHK(h, hipMalloc(&d_in, nbytes));
+    if (hipMalloc(&d_out, n * sizeof(float)) != hipSuccess) {
+        (void)hipFree(d_in);
+        return fail(nullptr, MUMMU_ERR_DEVICE, "hipMalloc failed");
+    }
+    hipError_t e = hipMemcpy(d_in, bytes, nbytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = launch_dequantize(type, d_in, blocks, d_out, nullptr);
+    if (e == hipSuccess) e = hipMemcpy(out, d_out, n * sizeof(float), hipMemcpyDeviceToHost);
+    (void)hipFree(d_in);
+    (void)hipFree(d_out);
+    if (e != hipSuccess) return fail(nullptr, MUMMU_ERR_DEVICE, std::string("dequantize: ") + hipGetErrorString(e));
+    return MUMMU_OK;
+}
+
+int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, int expert, float *out) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if (expert < 0 || expert >= h->cfg.num_experts) return fail(h, MUMMU_ERR_RANGE, "expert out of range");
+    if (which < 0 || which > 2 || !out) return fail(h, MUMMU_ERR_ARG, "which must be 0 (gate), 1 (up) or 2 (down)");
+    const Layer &L = h->layers[layer];
+    const int H = h->cfg.hidden_size, I = h->cfg.expert_intermediate_size;
+    const int type = which == 0 ? L.gate_type : (which == 1 ? L.up_type : L.down_type);
+    const int in_dim = which == 2 ? I : H, out_dim = which == 2 ? H : I;
+    const uint8_t *base = which == 0 ? L.gate : (which == 1 ? L.up : L.down);
+    const size_t rb = row_bytes_of(type, in_dim);
+    const size_t n = (size_t)in_dim * (size_t)out_dim;
+    float *d_out = nullptr;
+    HIPCHK(h, hipMalloc(&d_out, n * sizeof(float)));
+    hipError_t e = launch_dequantize(type, base + (size_t)expert * (size_t)out_dim * rb, n / (size_t)block_elems(type), d_out, h->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
+    if (e == hipSuccess) e = hipMemcpy(out, d_out, n * sizeof(float), hipMemcpyDeviceToHost);
+    (void)hipFree(d_out);
+    if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("dequantize_expert: ") + hipGetErrorString(e));
+    return MUMMU_OK;
+}
+
+int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_t n, int top_k, int norm, float *out_dev,
+                             void *stream) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if ((rc = check_device_call(h, n, top_k, x_dev, out_dev))) return rc;
+    if (n == 0) return MUMMU_OK;
+    return forward_impl(h, layer, x_dev, n, top_k, norm, nullptr, out_dev, (hipStream_t)stream);
+}
+
+int mummu_moe_stack_forward_device(mummu_moe *h, const float *x_dev, int64_t n, int top_k, int norm, float *out_dev, void *stream) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    int rc = check_topk(h, top_k, h->cfg.num_experts);
+    if (rc) return rc;
+    if ((rc = check_device_call(h, n, top_k, x_dev, out_dev))) return rc;
+    if (n == 0) return MUMMU_OK;
+    return stack_impl(h, x_dev, n, top_k, norm, out_dev, (hipStream_t)stream, nullptr);
+}
+
+int mummu_moe_check(mummu_moe *h, void *stream) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    return check_flags(h, (hipStream_t)stream);
+}
+
+int mummu_moe_last_routing(mummu_moe *h, int64_t n, int top_k, int32_t *ids, float *weights) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    if (n * top_k > h->ws_assign || n < 0 || top_k < 1) return fail(h, MUMMU_ERR_SHAPE, "routing larger than the workspace");
+    HIPCHK(h, hipDeviceSynchronize());
+    if (ids) HIPCHK(h, hipMemcpy(ids, h->ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    if (weights) HIPCHK(h, hipMemcpy(weights, h->weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+void *mummu_device_alloc(size_t bytes) {
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) return nullptr;
+    return p;
+}
+
+void mummu_device_free(void *p) {
+    if (p) (void)hipFree(p);
+}
+
+int mummu_copy_to_device(void *dst, const void *src, size_t bytes) {
+    mummu_moe *h = nullptr;
+    HIPCHK(h, hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return MUMMU_OK;
+}
+
+int mummu_copy_to_host(void *dst, const void *src, size_t bytes) {
+    mummu_moe *h = nullptr;
+    HIPCHK(h, hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int mummu_device_synchronize(void) {
+    mummu_moe *h = nullptr;
+    HIPCHK(h, hipDeviceSynchronize());
+    return MUMMU_OK;
+}
+
+int mummu_device_name(char *buf, size_t len) {
+    mummu_moe *h = nullptr;
+    if (!buf || len == 0) return fail(nullptr, MUMMU_ERR_ARG, "null buffer");
+    hipDeviceProp_t p;
+    HIPCHK(h, hipGetDeviceProperties(&p, 0));
+    snprintf(buf, len, "%s (%s, %d CUs)", p.name, p.gcnArchName, p.multiProcessorCount);
+    return MUMMU_OK;
+}
+
+void *mummu_moe_stream(mummu_moe *h) { return h ? (void *)h->stream : nullptr; }
+
+int mummu_graph_begin(mummu_moe *h) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    if (h->timing) return fail(h, MUMMU_ERR_ARG, "kernel timing records events; disable it before capturing a graph");
+    HIPCHK(h, hipStreamBeginCapture(h->stream, hipStreamCaptureModeThreadLocal));
+    return MUMMU_OK;
+}
+
+int mummu_graph_end(mummu_moe *h, void **graph_exec) {
+    if (!h || !graph_exec) return fail(h, MUMMU_ERR_ARG, "null argument");
+    hipGraph_t g = nullptr;
+    HIPCHK(h, hipStreamEndCapture(h->stream, &g));
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
+    *graph_exec = (void *)ex;
+    return MUMMU_OK;
+}
+
+int mummu_graph_launch(mummu_moe *h, void *graph_exec) {
+    if (!h || !graph_exec) return fail(h, MUMMU_ERR_ARG, "null argument");
+    HIPCHK(h, hipGraphLaunch((hipGraphExec_t)graph_exec, h->stream));
+    return MUMMU_OK;
+}
+
+void mummu_graph_destroy(void *graph_exec) {
+    if (graph_exec) (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+}
+
+int mummu_timer_start(mummu_moe *h) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    HIPCHK(h, hipEventRecord(h->t0, h->stream));
+    return MUMMU_OK;
+}
+
+int mummu_timer_stop(mummu_moe *h, float *ms) {
+    if (!h || !ms) return fail(h, MUMMU_ERR_ARG, "null argument");
+    HIPCHK(h, hipEventRecord(h->t1, h->stream));
+    HIPCHK(h, hipEventSynchronize(h->t1));
+    HIPCHK(h, hipEventElapsedTime(ms, h->t0, h->t1));
+    return MUMMU_OK;
+}
+
+int mummu_moe_kernel_timing(mummu_moe *h, int enable) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    h->timing = enable != 0;
+    return MUMMU_OK;
+}
+
+int mummu_moe_kernel_times(mummu_moe *h, const char **names, double *total_ms, int64_t *launches, int max_slots) {
+    if (!h || !names || !total_ms || !launches) return -1;
+    if (hipDeviceSynchronize() != hipSuccess) return -1;
+    const int n = max_slots < K_SLOTS ? max_slots : (int)K_SLOTS;
+    for (int i = 0; i < n; i++) {
+        names[i] = kSlotNames[i];
+        total_ms[i] = 0.0;
+        launches[i] = 0;
+    }
+    for (auto &t : h->timed) {
+        float ms = 0.0f;
+        if (t.slot < n && hipEventElapsedTime(&ms, t.start, t.stop) == hipSuccess) {
+            total_ms[t.slot] += ms;
+            launches[t.slot]++;
+        }
+        h->event_pool.push_back(t.start);
+        h->event_pool.push_back(t.stop);
+    }
+    h->timed.clear();
+    return n;
+}
+
+}  // extern "C"

@@ -1,0 +1,323 @@
+// Router of the sparse MoE block: logits GEMV, fused softmax / top-k / renormalise, and the
+// pre-norm + residual helpers of the layer wrapper.
+//
+// Reference semantics: nn/moe.rs:139-150 (Linear, f32 softmax over all experts, top-k,
+// optional renorm), models/qwen4exp/experts.rs:502-582 (the ggml-flavoured router),
+// models/olmoe.rs:566-572 (x + MoE(RmsNorm(x))).
+//
+// Summation orders are fixed so the routing indices are reproducible bit for bit:
+//   * a logit is 512 strided partial sums (element i -> partial i mod 512, one fma per
+//     element in ascending i).  Lane l of the wave owns partials 8l..8l+7, folds them as
+//     ((a0+a4)+(a1+a5))+((a2+a6)+(a3+a7)), and the 64 lane sums fold by the xor butterfly
+//     32,16,...,1.
+//   * softmax normaliser and top-k renorm sums run sequentially in ascending expert /
+//     slot order (f32, or f64 for the qwen4exp flavour), as the reference spells them out.
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace mummu {
+
+constexpr int kRouterTokensPerBlock = 4;
+constexpr int kMaxExpertsPerLane = 8;  // num_experts <= 512
+
+template <int WT>
+__device__ inline float load_w(const void *w, size_t i) {
+    if constexpr (WT == T_F32) return ((const float *)w)[i];
+    else if constexpr (WT == T_F16) return half_bits_to_float(((const uint16_t *)w)[i]);
+    else return bf16_bits_to_float(((const uint16_t *)w)[i]);
+}
+
+// 8 consecutive weights starting at element i (i % 8 == 0, 16-byte aligned rows).
+template <int WT>
+__device__ inline void load_w8(const void *w, size_t i, float (&o)[8]) {
+    if constexpr (WT == T_F32) {
+        const float4 *p = (const float4 *)((const float *)w + i);
+        float4 a = p[0], b = p[1];
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    } else {
+        uint4 v = *(const uint4 *)((const uint16_t *)w + i);
+        uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint16_t lo = (uint16_t)(u[j] & 0xFFFFu), hi = (uint16_t)(u[j] >> 16);
+            if constexpr (WT == T_F16) {
+                o[2 * j] = half_bits_to_float(lo);
+                o[2 * j + 1] = half_bits_to_float(hi);
+            } else {
+                o[2 * j] = bf16_bits_to_float(lo);
+                o[2 * j + 1] = bf16_bits_to_float(hi);
+            }
+        }
+    }
+}
+
+// One wave per expert row; the wave walks the row in chunks of 512 elements and serves
+// kRouterTokensPerBlock tokens from each loaded weight chunk.
+template <int WT, bool VEC>
+__global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x, const void *__restrict__ w,
+                                                            float *__restrict__ logits, int n, int hidden,
+                                                            int n_experts) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int e = blockIdx.y * (blockDim.x >> 6) + wave;
+    const int t0 = blockIdx.x * kRouterTokensPerBlock;
+    if (e >= n_experts) return;
+    float acc[kRouterTokensPerBlock][8];
+#pragma unroll
+    for (int t = 0; t < kRouterTokensPerBlock; t++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[t][j] = 0.0f;
+
+    const size_t wrow = (size_t)e * (size_t)hidden;
+    for (int base = lane * 8; base < hidden; base += 512) {
+        float wv[8];
+        int cnt = hidden - base < 8 ? hidden - base : 8;
+        if (VEC) {
+            load_w8<WT>(w, wrow + (size_t)base, wv);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) wv[j] = j < cnt ? load_w<WT>(w, wrow + (size_t)(base + j)) : 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < kRouterTokensPerBlock; t++) {
+            if (t0 + t >= n) break;
+            const float *xr = x + (size_t)(t0 + t) * (size_t)hidden + base;
+            float xv[8];
+            if (VEC) {
+                float4 a = ((const float4 *)xr)[0], b = ((const float4 *)xr)[1];
+                xv[0] = a.x; xv[1] = a.y; xv[2] = a.z; xv[3] = a.w; xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) xv[j] = j < cnt ? xr[j] : 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (VEC || j < cnt) acc[t][j] = __builtin_fmaf(xv[j], wv[j], acc[t][j]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < kRouterTokensPerBlock; t++) {
+        if (t0 + t >= n) break;
+        const float *a = acc[t];
+        float s = __fadd_rn(__fadd_rn(__fadd_rn(a[0], a[4]), __fadd_rn(a[1], a[5])),
+                            __fadd_rn(__fadd_rn(a[2], a[6]), __fadd_rn(a[3], a[7])));
+        s = wave_sum(s);
+        if (lane == 0) logits[(size_t)(t0 + t) * (size_t)n_experts + (size_t)e] = s;
+    }
+}
+
+hipError_t launch_router_logits(const float *x, const void *w, int wtype, float *logits, int n, int hidden,
+                                int n_experts, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
+    // few tokens: one wave per workgroup so the expert rows spread over as many CUs as possible
+    const int waves = n <= 8 ? 1 : 4;
+    dim3 block(64 * waves);
+    dim3 grid((n + kRouterTokensPerBlock - 1) / kRouterTokensPerBlock, (n_experts + waves - 1) / waves);
+#define MUMMU_LAUNCH_ROUTER(WT)                                                                          \
+    do {                                                                                                 \
+        if (vec) router_logits_kernel<WT, true><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts);  \
+        else router_logits_kernel<WT, false><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts);     \
+    } while (0)
+    switch (wtype) {
+    case T_F32: MUMMU_LAUNCH_ROUTER(T_F32); break;
+    case T_F16: MUMMU_LAUNCH_ROUTER(T_F16); break;
+    case T_BF16: MUMMU_LAUNCH_ROUTER(T_BF16); break;
+    default: return hipErrorInvalidValue;
+    }
+#undef MUMMU_LAUNCH_ROUTER
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------
+// softmax -> top-k -> renormalise, one wave per token.  Lane l holds experts l, l+64, ...
+// Ties: strictly-greater wins, so the lower expert id keeps a tie and equal slots ascend
+// by id (experts.rs:557-573; the stable descending sort of nn/moe.rs:2143-2144).
+// ---------------------------------------------------------------------------------------
+constexpr int kTopkWavesPerBlock = 4;
+constexpr int kMaxExperts = 64 * kMaxExpertsPerLane;
+
+__device__ inline float lane_bcast(float v, int src) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+
+__global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
+    const float *__restrict__ logits, int n, int n_experts, int k, int flavour, int norm, int32_t *__restrict__ ids,
+    float *__restrict__ weights, unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
+    __shared__ float s_w[kTopkWavesPerBlock][kMaxExperts];
+    __shared__ int s_id[kTopkWavesPerBlock][kMaxExperts];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * kTopkWavesPerBlock + wave;
+    if (t >= n) return;
+    const float *row = logits + (size_t)t * (size_t)n_experts;
+
+    float p[kMaxExpertsPerLane];
+    bool bad = false;
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int j = 0; j < kMaxExpertsPerLane; j++) {
+        int e = lane + 64 * j;
+        if (e < n_experts) {
+            float l = row[e];
+            p[j] = l;
+            if (!(fabsf(l) <= 3.402823466e38f)) {  // inf or NaN
+                bad = true;
+                atomicMin(&flags[FLAG_NONFINITE_INDEX], t * n_experts + e);
+            }
+            mx = fmaxf(mx, l);
+        } else {
+            p[j] = -__builtin_inff();
+        }
+    }
+    const bool any_bad = __any(bad);
+    if (any_bad) {
+        // Refused like experts.rs:546-553: flag it and emit a harmless, in-range routing so
+        // the kernels downstream stay inside their buffers; the host reports the error.
+        if (lane == 0) atomicAdd(&flags[FLAG_NONFINITE], 1);
+        for (int s = lane; s < k; s += 64) {
+            ids[(size_t)t * k + s] = s;
+            weights[(size_t)t * k + s] = 0.0f;
+        }
+        return;
+    }
+    mx = wave_max(mx);
+#pragma unroll
+    for (int j = 0; j < kMaxExpertsPerLane; j++) p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(p[j], mx)) : 0.0f;
+
+    // normaliser: sequential over ascending expert id
+    if (flavour == 0) {
+        float total = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; j++) {
+            int lim = n_experts - 64 * j;
+            lim = lim > 64 ? 64 : lim;
+            for (int src = 0; src < lim; src++) total = __fadd_rn(total, lane_bcast(p[j], src));
+        }
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; j++) p[j] = __fdiv_rn(p[j], total);
+    } else {
+        double total = 0.0;
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; j++) {
+            int lim = n_experts - 64 * j;
+            lim = lim > 64 ? 64 : lim;
+            for (int src = 0; src < lim; src++) total = __dadd_rn(total, (double)lane_bcast(p[j], src));
+        }
+        float scale = (float)__ddiv_rn(1.0, total);
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; j++) p[j] = __fmul_rn(p[j], scale);
+    }
+
+    // k rounds of wave-wide arg-max with (prob desc, id asc) order
+    unsigned taken = 0;
+    for (int s = 0; s < k; s++) {
+        float bp = -1.0f;
+        int bid = 0x7FFFFFFF;
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; j++) {
+            int e = lane + 64 * j;
+            if (e < n_experts && !(taken & (1u << j)) && p[j] > bp) {
+                bp = p[j];
+                bid = e;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            float op = __shfl_xor(bp, off, kWave);
+            int oid = __shfl_xor(bid, off, kWave);
+            if (op > bp || (op == bp && oid < bid)) {
+                bp = op;
+                bid = oid;
+            }
+        }
+        if ((bid & 63) == lane) taken |= 1u << (bid >> 6);
+        if (lane == 0) {
+            s_w[wave][s] = bp;
+            s_id[wave][s] = bid;
+        }
+    }
+    // lane 0's LDS writes above are read by every lane of this same wave below
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    float denom = 1.0f;
+    if (flavour == 0) {
+        if (norm) {
+            float d = 0.0f;
+            for (int s = 0; s < k; s++) d = __fadd_rn(d, s_w[wave][s]);
+            denom = d;
+        }
+    } else {
+        double d = 0.0;
+        for (int s = 0; s < k; s++) d = __dadd_rn(d, (double)s_w[wave][s]);
+        float fs = (float)d;
+        const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
+        denom = fs > floor_v ? fs : floor_v;
+    }
+    const bool divide = flavour != 0 || norm;
+    for (int s = lane; s < k; s += 64) {
+        float wv = s_w[wave][s];
+        int id = s_id[wave][s];
+        if (divide) wv = __fdiv_rn(wv, denom);
+        ids[(size_t)t * k + s] = id;
+        weights[(size_t)t * k + s] = wv;
+        if (hits) atomicAdd(&hits[id], 1ULL);
+    }
+}
+
+hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, int flavour, int norm, int32_t *ids,
+                             float *weights, unsigned long long *hits, int32_t *flags, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (n_experts > kMaxExperts || k > n_experts || k < 1) return hipErrorInvalidValue;
+    dim3 block(64 * kTopkWavesPerBlock), grid((n + kTopkWavesPerBlock - 1) / kTopkWavesPerBlock);
+    route_topk_kernel<<<grid, block, 0, s>>>(logits, n, n_experts, k, flavour, norm, ids, weights, hits, flags);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------
+// RmsNorm, one wave per token: sum of squares in the router's 512-partial order, then
+// (x * (1/sqrt(mean + eps))) * gamma with every step rounded separately.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                      float eps, int n, int hidden, float *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (t >= n) return;
+    const float *row = x + (size_t)t * (size_t)hidden;
+    float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int base = lane * 8; base < hidden; base += 512) {
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (base + j < hidden) {
+                float v = row[base + j];
+                a[j] = __builtin_fmaf(v, v, a[j]);
+            }
+    }
+    float ss = __fadd_rn(__fadd_rn(__fadd_rn(a[0], a[4]), __fadd_rn(a[1], a[5])),
+                         __fadd_rn(__fadd_rn(a[2], a[6]), __fadd_rn(a[3], a[7])));
+    ss = wave_sum(ss);
+    float mean = __fdiv_rn(ss, (float)hidden);
+    float r = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, eps)));
+    for (int i = lane; i < hidden; i += 64) out[(size_t)t * hidden + i] = __fmul_rn(__fmul_rn(row[i], r), gamma[i]);
+}
+
+hipError_t launch_rmsnorm(const float *x, const float *gamma, float eps, int n, int hidden, float *out, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    dim3 block(256), grid((n + 3) / 4);
+    rmsnorm_kernel<<<grid, block, 0, s>>>(x, gamma, eps, n, hidden, out);
+    return hipGetLastError();
+}
+
+__global__ void add_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = __fadd_rn(a[i], b[i]);
+}
+
+hipError_t launch_add(const float *a, const float *b, float *dst, size_t n, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    add_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(a, b, dst, n);
+    return hipGetLastError();
+}
+
+}  // namespace mummu

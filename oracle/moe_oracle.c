@@ -25,7 +25,8 @@
  *   orc_route_olmoe    - softmax/top-k/renorm as the reference's scalar restatement of its
  *                        tensor path does it (nn/moe.rs:2138-2152).  Tie order and last-ulp
  *                        softmax rounding of burn itself are PARITY UNPINNED.
- *   orc_rmsnorm        - x * rsqrt(mean(x^2) + eps) * gamma with an f32 sequential mean.
+ *   orc_rmsnorm        - x * rsqrt(mean(x^2) + eps) * gamma, sum of squares in the router's
+ *                        512-partial order.
  *                        PARITY UNPINNED (burn RmsNorm is third-party).
  *
  * Everything else (GGUF dequantizers, f16 conversion, the 8-lane dot, silu, the
@@ -771,18 +772,14 @@ ORC_API int orc_moe_forward_dense_mask(const orc_banks *b, const void *router_w,
 /* ------------------------------------------------------------------------------------
  * Layer wrapper, models/olmoe.rs:566-572 and 1742-1755: h2 = RmsNorm(x; gamma, eps),
  * x = x + MoE(h2).  burn's RmsNorm is x * rsqrt(mean(x^2) + eps) * gamma; its rounding is
- * third-party (PARITY UNPINNED).  Fixed here: f32 sequential sum of squares (each square
- * rounded, then added), mean = sum / H, r = 1/sqrt(mean + eps) (correctly rounded sqrt
- * and divide), y = (x * r) * gamma.
+ * third-party (PARITY UNPINNED).  Fixed here: the sum of squares in the same 512-partial
+ * fma order as the router logits (orc_router_dot of the row with itself), mean = sum / H,
+ * r = 1/sqrt(mean + eps) (correctly rounded sqrt and divide), y = (x * r) * gamma.
  * ---------------------------------------------------------------------------------- */
 ORC_API void orc_rmsnorm(const float *x, const float *gamma, float eps, size_t n, size_t hidden, float *out) {
     for (size_t t = 0; t < n; t++) {
         const float *row = x + t * hidden;
-        float ss = 0.0f;
-        for (size_t i = 0; i < hidden; i++) {
-            float sq = row[i] * row[i];
-            ss = ss + sq;
-        }
+        float ss = orc_router_dot(row, row, ORC_F32, 0, hidden);
         float mean = ss / (float)hidden;
         float r = 1.0f / sqrtf(mean + eps);
         for (size_t i = 0; i < hidden; i++) {
