@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse MoE block on one MI355X.
+
+Default workload: the Q4_K OLMoE-shaped layer at decode batch 1 (hidden 2048, 64 experts,
+top-8, SwiGLU intermediate 1024, f16 router, norm_topk_prob=false) - the configuration the
+headline metric is quoted on.  A "step" is one forward of one MoE layer over one batch of
+tokens, inputs and weights already resident in HBM.  Steps rotate over `--layers` distinct
+layer banks (16 x 226.5 MB) and over a pool of distinct tokens, so that no step finds its
+expert weights in the 256 MB Infinity Cache from an earlier step: a layer is revisited only
+after the other 15 have streamed >= 425 MB through the cache.
+
+The whole rotation is captured once in a HIP graph and replayed (the serving-loop form);
+--no-graph times eager launches instead.
+
+Prints ONE JSON line (the contract the round driver reads), including
+  roofline      the dominant kernel (gate_up) against the 8 TB/s HBM peak, its duration
+                measured live with HIP events on the library's stream,
+  cpu_baseline  the CPU oracle (a C restatement of the reference's routed CPU path) timed on
+                this host on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (hidden, inter, experts, top_k, norm, bank type, router type)
+    "olmoe_q4k_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q4_K", router="F16"),
+    "olmoe_q8_0_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q8_0", router="F16"),
+    "olmoe_f16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F16", router="F16"),
+    "qwen3_a3b_q4k": dict(hidden=2048, inter=768, experts=128, top_k=8, norm=True, bank="Q4_K", router="F16"),
+}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--workload", default="olmoe_q4k_decode", choices=sorted(WORKLOADS))
+    ap.add_argument("--tokens", type=int, default=1, help="tokens per step (decode batch)")
+    ap.add_argument("--layers", type=int, default=16, help="distinct layer banks the steps rotate over")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
+              "(expert-parallel sharding over several GPUs is described in DESIGN.md, not built).", file=sys.stderr)
+        return 2
+
+    from mummu_amd import _lib, moe as M, synth
+
+    if _lib.device_count() < 1:
+        print("bench.py: no HIP device", file=sys.stderr)
+        return 3
+
+    w = WORKLOADS[args.workload]
+    H, I, E, k, norm = w["hidden"], w["inter"], w["experts"], w["top_k"], w["norm"]
+    bank_t = {"Q4_K": M.Q4_K, "Q8_0": M.Q8_0, "F16": M.F16}[w["bank"]]
+    router_t = M.F16
+    n = args.tokens
+    L = args.layers
+
+    def bank_bytes(in_dim, out_dim):
+        return E * out_dim * synth.row_bytes(bank_t, in_dim)
+
+    g = np.random.Generator(np.random.PCG64(args.seed))
+
+    def make_bank(in_dim, out_dim, seed):
+        if bank_t in (M.Q4_K, M.Q8_0):
+            return synth.random_bank_fast(bank_t, [in_dim, out_dim, E], seed)
+        gg = np.random.Generator(np.random.PCG64(seed))
+        return (gg.standard_normal(E * out_dim * in_dim, dtype=np.float32) * np.float32(0.02)).astype(np.float16).view(np.uint8)
+
+    t_setup = time.time()
+    moe = M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=max(n, 8), norm_topk_prob=norm)
+    routers = []
+    keep_layer0 = None
+    for l in range(L):
+        router = (g.standard_normal((E, H), dtype=np.float32) * np.float32(0.02)).astype(np.float16)
+        gate = make_bank(H, I, args.seed * 1000 + 3 * l)
+        up = make_bank(H, I, args.seed * 1000 + 3 * l + 1)
+        down = make_bank(I, H, args.seed * 1000 + 3 * l + 2)
+        moe.load_layer(l, router, router_t, gate, bank_t, up, bank_t, down, bank_t)
+        routers.append(router)
+        if l == 0:
+            keep_layer0 = (router, gate, up, down)
+    # a pool of distinct token batches: routing differs from step to step
+    pool = 64
+    xs = g.standard_normal((pool, n, H), dtype=np.float32)
+    x_dev = [M.DeviceBuffer.from_array(xs[i]) for i in range(pool)]
+    out_dev = M.DeviceBuffer(n * H * 4)
+    setup_s = time.time() - t_setup
+
+    expert_bytes = 2 * I * synth.row_bytes(bank_t, H) + H * synth.row_bytes(bank_t, I)
+    gate_up_expert_bytes = 2 * I * synth.row_bytes(bank_t, H)
+    router_bytes = E * H * 2
+
+    # distinct experts per step, from the actual routing of every (layer, token batch) pair used
+    period = int(L * pool // np.gcd(L, pool))
+    distinct = {}
+    for s in range(min(period, L * pool)):
+        l, p = s % L, s % pool
+        if (l, p) in distinct:
+            continue
+        r = moe.route(xs[p], k, norm, layer=l)
+        distinct[(l, p)] = len(np.unique(r.ids))
+    mean_distinct = float(np.mean(list(distinct.values())))
+
+    def step(s):
+        moe.forward_device(s % L, x_dev[s % pool], n, k, norm, out_dev)
+
+    use_graph = not args.no_graph
+    graph = None
+    steps_per_launch = 1
+    if use_graph:
+        steps_per_launch = period if period <= 1024 else L
+        moe.graph_begin()
+        for s in range(steps_per_launch):
+            step(s)
+        graph = moe.graph_end()
+
+    def run(nsteps, s0=0):
+        if graph is not None:
+            for _ in range(nsteps // steps_per_launch):
+                graph.launch()
+            for s in range(nsteps % steps_per_launch):
+                step(s)
+        else:
+            for s in range(nsteps):
+                step(s0 + s)
+
+    run(args.warmup)
+    M.synchronize()
+    moe.check()
+    moe.timer_start()
+    t0 = time.perf_counter()
+    run(args.steps)
+    ev_ms = moe.timer_stop()
+    M.synchronize()
+    wall = time.perf_counter() - t0
+    moe.check()
+
+    ms_per_step = wall * 1e3 / args.steps
+    value = n * args.steps / wall
+
+    # per-kernel durations: eager launches bracketed by HIP events on the library's stream
+    moe.kernel_timing(True)
+    probe_steps = min(args.steps, 800)
+    for s in range(probe_steps):
+        step(s)
+    kt = moe.kernel_times()
+    moe.kernel_timing(False)
+    per_kernel_us = {name: (tot / cnt * 1e3 if cnt else None) for name, (tot, cnt) in kt.items()}
+    gu_us = per_kernel_us.get("gate_up")
+    gu_bytes = mean_distinct * gate_up_expert_bytes
+    achieved = gu_bytes / (gu_us * 1e-6) / 1e9 if gu_us else None
+
+    layer_bytes = mean_distinct * expert_bytes + router_bytes + n * H * 8
+    layer_gbs = layer_bytes / (ms_per_step * 1e-3) / 1e9
+
+    out = {
+        "metric": "MoE-layer tokens/s + achieved HBM GB/s (Q4_K, OLMoE shape, 1 GPU)",
+        "value": round(value, 1),
+        "unit": "layer-tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"Q4_K": "u4*i16->i32 (v_dot4_i32_i8), f32 scales", "Q8_0": "i8*i16->i32 (v_dot4_i32_i8), f32 scales",
+                  "F16": "f32"}[w["bank"]],
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts, "
+                               f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
+                   "tokens_per_step": n, "layers": L, "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
+                   "mean_distinct_experts_per_step": round(mean_distinct, 3)},
+        "us_per_layer": round(ms_per_step * 1e3, 3),
+        "event_ms_per_step": round(ev_ms / args.steps, 6),
+        "layer_algorithmic_bytes": int(layer_bytes),
+        "layer_hbm_gbs": round(layer_gbs, 1),
+        "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4),
+        "kernel_us": {k_: (round(v, 3) if v is not None else None) for k_, v in per_kernel_us.items()},
+        "roofline": {"bound": "hbm", "kernel": "gate_up", "achieved": round(achieved, 1) if achieved else None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None, "traffic": None,
+                     "algorithmic_bytes_per_launch": int(gu_bytes), "avg_launch_us": round(gu_us, 3) if gu_us else None},
+        "device": M.device_name(),
+        "setup_s": round(setup_s, 1),
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(keep_layer0, w, bank_t, xs, n, args.cpu_seconds)
+    print(json.dumps(out))
+    return 0
+
+
+def cpu_baseline(layer0, w, bank_t, xs, n, budget_s):
+    """The oracle's routed path (the reference's qwen4exp algorithm: per hit expert, dequantize
+    row chunks and dot them in the fixed 8-lane order; OpenMP over rows where the reference
+    uses rayon) on layer 0 of the same banks, same token batches, for about budget_s seconds."""
+    from oracle import binding as orc
+    router, gate, up, down = layer0
+    H, I, E, k, norm = w["hidden"], w["inter"], w["experts"], w["top_k"], w["norm"]
+    t = {"Q4_K": orc.Q4_K, "Q8_0": orc.Q8_0, "F16": orc.F16}[w["bank"]]
+    banks = orc.LayerBanks(H, I, E, gate, up, down, t)
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    orc.moe_forward(banks, router, orc.F16, xs[0], k, norm)  # warm
+    done, t0, best = 0, time.perf_counter(), None
+    while time.perf_counter() - t0 < budget_s:
+        t1 = time.perf_counter()
+        orc.moe_forward(banks, router, orc.F16, xs[done % xs.shape[0]], k, norm)
+        dt = time.perf_counter() - t1
+        best = dt if best is None else min(best, dt)
+        done += 1
+    total = time.perf_counter() - t0
+    return {"value": round(n * done / total, 2), "unit": "layer-tokens/s", "cores": threads, "kind": "port",
+            "sample": f"{done} steps of the same workload on layer 0 ({n} token(s)/step), mean over {total:.1f} s; "
+                      f"best step {best * 1e3:.1f} ms",
+            "cpu": _cpu_model()}
+
+
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+if __name__ == "__main__":
+    sys.exit(main())

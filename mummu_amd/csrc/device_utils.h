@@ -98,6 +98,77 @@ __device__ inline float group_sum(float v, int width) {
     return v;
 }
 
+// ---- cross-lane sums at VALU speed (DPP inside a 16-lane row, gfx950 lane swaps across rows) ----
+template <int CTRL>
+__device__ inline float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+
+// Sum over aligned groups of `width` lanes inside a 16-lane row (width in {1,2,4,8,16}); every
+// lane of a group ends with the group's sum.  Steps: xor 1, xor 2 (quad permutes), then the
+// half-row and row mirrors, which pair lanes of the two already-uniform halves.
+__device__ inline float row_group_sum(float v, int width) {
+    if (width >= 2) v = __fadd_rn(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    if (width >= 4) v = __fadd_rn(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    if (width >= 8) v = __fadd_rn(v, dpp_move<0x141>(v));  // row_half_mirror
+    if (width >= 16) v = __fadd_rn(v, dpp_move<0x140>(v)); // row_mirror
+    return v;
+}
+
+// v_permlane32_swap: lanes 0-31 receive a[l] + a[l+32], lanes 32-63 receive b[l-32] + b[l].
+// With a == b this is the xor-32 butterfly step; with two values it also halves the work.
+__device__ inline float swap32_add(float a, float b) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_int(a), __float_as_int(b), false, false);
+    return __fadd_rn(__int_as_float(r[0]), __int_as_float(r[1]));
+}
+
+// v_permlane16_swap: even 16-lane rows receive a[row] + a[row+1], odd rows b[row-1] + b[row].
+__device__ inline float swap16_add(float a, float b) {
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_int(a), __float_as_int(b), false, false);
+    return __fadd_rn(__int_as_float(r[0]), __int_as_float(r[1]));
+}
+
+// Reduce NV per-lane partials, each over aligned groups of `group` lanes (power of two), and
+// leave `count` finished sums in v[0..count): the value with original index offset + j sits
+// in v[j].  Crossing 32- and 16-lane boundaries halves the number of values a lane carries
+// (the two halves of the group finish different values), so the expensive steps are shared.
+template <int NV>
+__device__ inline void reduce_partials(float (&v)[NV], int group, int lane, int &count, int &offset) {
+    count = NV;
+    offset = 0;
+    if (group == 64) {
+        if constexpr (NV >= 4) {
+#pragma unroll
+            for (int j = 0; j < NV / 2; j++) v[j] = swap32_add(v[j], v[j + NV / 2]);
+#pragma unroll
+            for (int j = 0; j < NV / 4; j++) v[j] = swap16_add(v[j], v[j + NV / 4]);
+            count = NV / 4;
+            offset = ((lane >> 5) & 1) * (NV / 2) + ((lane >> 4) & 1) * (NV / 4);
+        } else if constexpr (NV == 2) {
+            v[0] = swap32_add(v[0], v[1]);
+            v[0] = swap16_add(v[0], v[0]);
+            count = 1;
+            offset = (lane >> 5) & 1;
+        } else {
+            v[0] = swap32_add(v[0], v[0]);
+            v[0] = swap16_add(v[0], v[0]);
+        }
+    } else if (group == 32) {
+        if constexpr (NV >= 2) {
+#pragma unroll
+            for (int j = 0; j < NV / 2; j++) v[j] = swap16_add(v[j], v[j + NV / 2]);
+            count = NV / 2;
+            offset = ((lane >> 4) & 1) * (NV / 2);
+        } else {
+            v[0] = swap16_add(v[0], v[0]);
+        }
+    }
+    const int width = group < 16 ? group : 16;
+#pragma unroll
+    for (int j = 0; j < NV; j++)
+        if (j < count) v[j] = row_group_sum(v[j], width);
+}
+
 __device__ inline float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));

@@ -11,15 +11,17 @@
 // block; float types: consecutive elements), so every global load is a contiguous run.
 //
 // Arithmetic of the quantized types (Q4_K, Q8_0): the activation row is quantized ONCE per
-// wave, in registers, to 16-bit integers with one f32 scale per 32 elements
-// (xq = rint(x * 32512/amax)), split into two signed bytes xq = 256*hi + lo.  Weight codes
-// and activation bytes meet in v_dot4_i32_i8, so the per-block sums  sum(q * xq)  are exact
-// integers; only the scale products are floating point:
-//     Q8_0 block :  d * (s * float(sum q*xq))
-//     Q4_K half-sub-block pair:  (d*sc)*(s*float(sum q*xq)) - (dmin*m)*(s*float(sum xq))
+// wave, in registers, to 16-bit integers xq = rint(x * 32512/amax) with one f32 scale
+// s = amax/32512 per activation block (64 elements under Q4_K - one low/high nibble chunk -
+// and 32 under Q8_0), split into two signed bytes xq = 256*hi + lo.  Weight codes and
+// activation bytes meet in v_dot4_i32_i8, so the block sums  sum(q * xq)  are exact integers;
+// only the scale products are floating point:
+//     Q8_0 block :              d * (s * float(sum q*xq))
+//     Q4_K sub-block pair:  (d*s) * float(sc0*sum(q0*xq0) + sc1*sum(q1*xq1))
+//                         - (dmin*s) * float(m0*sum(xq0) + m1*sum(xq1))
 // A 16-bit activation is ~2^-15 of the block maximum - about 100x finer than the int8
-// activations llama.cpp multiplies these formats with - and keeps the result independent
-// of how many tokens share the call.
+// activations llama.cpp multiplies these formats with - and, being a function of the token's
+// own row only, keeps the result independent of how many tokens share the call.
 // Float weight types (F32/F16/BF16) run an f32 fma chain per lane on the exact f32 value of
 // each weight.
 #include "device_utils.h"
@@ -52,8 +54,8 @@ template <int UPL>
 struct LaneAct {
     int xh[UPL][8];  // hi bytes of the lane's 32 activations, 4 per word
     int xl[UPL][8];  // lo bytes
-    float s[UPL][2];   // block scale of the first / second 16 elements
-    float fx[UPL][2];  // s * sum(xq) over the first / second 16 elements (Q4_K min term)
+    float s[UPL];    // scale of the activation block the lane's 32 elements belong to
+    int sx[UPL][2];  // sum(xq) over the first / second 16 elements (Q4_K min term)
 };
 
 // Start elements of the two 16-element halves unit u of a row covers.
@@ -69,10 +71,8 @@ __device__ inline void unit_halves(int u, int &e0, int &e1) {
     }
 }
 
-__device__ inline void quantize16(const float (&v)[16], float amax, int *xh, int *xl, float &s, float &fx) {
-    float inv = amax > 0.0f ? __fdiv_rn(32512.0f, amax) : 0.0f;
-    s = amax > 0.0f ? __fdiv_rn(amax, 32512.0f) : 0.0f;
-    int sum = 0;
+__device__ inline void quantize16(const float (&v)[16], float inv, int *xh, int *xl, int &sum) {
+    sum = 0;
 #pragma unroll
     for (int w = 0; w < 4; w++) {
         uint32_t hw = 0, lw = 0;
@@ -89,10 +89,11 @@ __device__ inline void quantize16(const float (&v)[16], float amax, int *xh, int
         xh[w] = (int)hw;
         xl[w] = (int)lw;
     }
-    fx = __fmul_rn(s, (float)sum);
 }
 
-// Quantize the lane's share of activation row `xrow` (f32, in_dim wide).
+// Quantize the lane's share of activation row `xrow` (f32, in_dim wide).  The activation
+// block (one scale) is the 64-element chunk for Q4_K - the lane's two halves plus those of the
+// neighbouring unit, lane ^ 1 - and the 32-element block for Q8_0.
 template <int WT, int UPL>
 __device__ inline void load_lane_act(const float *__restrict__ xrow, int unit0, int units, LaneAct<UPL> &a) {
 #pragma unroll
@@ -110,69 +111,103 @@ __device__ inline void load_lane_act(const float *__restrict__ xrow, int unit0, 
             v0[4 * j] = a0.x; v0[4 * j + 1] = a0.y; v0[4 * j + 2] = a0.z; v0[4 * j + 3] = a0.w;
             v1[4 * j] = a1.x; v1[4 * j + 1] = a1.y; v1[4 * j + 2] = a1.z; v1[4 * j + 3] = a1.w;
         }
-        float m0 = 0.0f, m1 = 0.0f;
+        float m = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            m0 = fmaxf(m0, fabsf(v0[j]));
-            m1 = fmaxf(m1, fabsf(v1[j]));
-        }
-        if (!on) m0 = m1 = 0.0f;
-        if constexpr (WT == T_Q4_K) {
-            // each 32-element activation block is shared with the neighbouring unit (lane ^ 1)
-            m0 = fmaxf(m0, __shfl_xor(m0, 1, kWave));
-            m1 = fmaxf(m1, __shfl_xor(m1, 1, kWave));
-        } else {
-            m0 = m1 = fmaxf(m0, m1);
-        }
-        quantize16(v0, m0, &a.xh[i][0], &a.xl[i][0], a.s[i][0], a.fx[i][0]);
-        quantize16(v1, m1, &a.xh[i][4], &a.xl[i][4], a.s[i][1], a.fx[i][1]);
+        for (int j = 0; j < 16; j++) m = fmaxf(m, fmaxf(fabsf(v0[j]), fabsf(v1[j])));
+        if (!on) m = 0.0f;
+        if constexpr (WT == T_Q4_K) m = fmaxf(m, dpp_move<0xB1>(m));  // lane ^ 1 holds the rest of the chunk
+        const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
+        a.s[i] = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
+        quantize16(v0, inv, &a.xh[i][0], &a.xl[i][0], a.sx[i][0]);
+        quantize16(v1, inv, &a.xh[i][4], &a.xl[i][4], a.sx[i][1]);
         if (!on) {
 #pragma unroll
             for (int w = 0; w < 8; w++) a.xh[i][w] = a.xl[i][w] = 0;
-            a.s[i][0] = a.s[i][1] = a.fx[i][0] = a.fx[i][1] = 0.0f;
+            a.s[i] = 0.0f;
+            a.sx[i][0] = a.sx[i][1] = 0;
         }
     }
 }
 
-__device__ inline uint32_t scale_byte(uint32_t s0, uint32_t s1, uint32_t s2, int k) {
-    uint32_t w = k < 4 ? s0 : (k < 8 ? s1 : s2);
-    return (w >> (8 * (k & 3))) & 0xFFu;
-}
-
-// 6-bit (scale, min) of sub-block j from the 12 packed bytes (ggml get_scale_min_k4).
-__device__ inline void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j, float &sc, float &mn) {
-    uint32_t a, b;
-    if (j < 4) {
-        a = scale_byte(s0, s1, s2, j) & 63u;
-        b = scale_byte(s0, s1, s2, j + 4) & 63u;
-    } else {
-        uint32_t hi = scale_byte(s0, s1, s2, j + 4);
-        a = (hi & 0x0Fu) | ((scale_byte(s0, s1, s2, j - 4) >> 6) << 4);
-        b = (hi >> 4) | ((scale_byte(s0, s1, s2, j) >> 6) << 4);
-    }
-    sc = (float)a;
-    mn = (float)b;
-}
-
-// The lane's partial of <row, activation> for a quantized row.
+// The lane's raw share of one quantized weight row, as loaded (nothing decoded yet), so that a
+// wave can put the loads of several rows in flight before it touches any of them.
 template <int WT, int UPL>
-__device__ inline float row_partial_q(const uint8_t *__restrict__ rowp, int unit0, int units, const LaneAct<UPL> &a) {
+struct RawRow;
+template <int UPL>
+struct RawRow<T_Q4_K, UPL> {
+    uint4 hdr[UPL];  // f16 d, f16 dmin, 12 B of 6-bit scales/mins
+    uint4 q[UPL];    // the lane's 16 bytes of nibbles
+};
+template <int UPL>
+struct RawRow<T_Q8_0, UPL> {
+    uint32_t d[UPL];     // f16 scale bits
+    uint32_t q[UPL][8];  // 32 int8 codes
+};
+
+template <int WT, int UPL>
+__device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int units, bool ok, RawRow<WT, UPL> &r) {
+#pragma unroll
+    for (int i = 0; i < UPL; i++) {
+        const int u = unit0 + 64 * i;
+        const bool on = ok && u < units;
+        if constexpr (WT == T_Q4_K) {
+            r.hdr[i] = make_uint4(0, 0, 0, 0);
+            r.q[i] = make_uint4(0, 0, 0, 0);
+            if (on) {
+                const uint8_t *blk = rowp + (size_t)(u >> 3) * 144;
+                r.hdr[i] = *(const uint4 *)blk;
+                r.q[i] = *(const uint4 *)(blk + 16 + (u & 7) * 16);
+            }
+        } else {
+            r.d[i] = 0;
+#pragma unroll
+            for (int w = 0; w < 8; w++) r.q[i][w] = 0;
+            if (on) {
+                const uint8_t *blk = rowp + (size_t)u * 34;
+                uint16_t db;
+                __builtin_memcpy(&db, blk, 2);
+                r.d[i] = db;
+#pragma unroll
+                for (int w = 0; w < 8; w++) __builtin_memcpy(&r.q[i][w], blk + 2 + 4 * w, 4);  // 2-byte aligned
+            }
+        }
+    }
+}
+
+// The lane's partial of <row, activation>.  A lane that loaded nothing holds zero scales and
+// contributes exactly 0.
+//   Q4_K: with q the 4-bit codes, xq the 16-bit activations of the lane's two 16-element halves
+//   (sub-blocks 2c and 2c+1 of one super-block, one activation scale s),
+//       (d*s) * float(sc0*sum(q0*xq0) + sc1*sum(q1*xq1)) - (dmin*s) * float(m0*sum(xq0) + m1*sum(xq1))
+//   where every sum and both 6-bit-weighted combinations are exact integers.
+//   Q8_0: d * (s * float(sum(q*xq))).
+template <int WT, int UPL>
+__device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneAct<UPL> &a) {
     float acc = 0.0f;
 #pragma unroll
     for (int i = 0; i < UPL; i++) {
-        int u = unit0 + 64 * i;
-        if (u >= units) break;
         if constexpr (WT == T_Q4_K) {
-            const uint8_t *blk = rowp + (size_t)(u >> 3) * 144;
-            uint4 hdr = *(const uint4 *)blk;
-            uint4 qv = *(const uint4 *)(blk + 16 + (u & 7) * 16);
-            float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFFu));
-            float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
-            int c = (u & 7) >> 1;
-            float sc0, mn0, sc1, mn1;
-            q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc0, mn0);
-            q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc1, mn1);
-            uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+            const int u = unit0 + 64 * i;
+            const uint4 hdr = r.hdr[i];
+            const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFFu));
+            const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
+            // 6-bit (scale, min) of sub-blocks 2c, 2c+1 (ggml get_scale_min_k4), c fixed per lane
+            const int c = (u & 7) >> 1;
+            const int sh = 16 * (c & 1);
+            int sc0, sc1, mn0, mn1;
+            if (c < 2) {
+                sc0 = (int)((hdr.y >> sh) & 63u);
+                sc1 = (int)((hdr.y >> (sh + 8)) & 63u);
+                mn0 = (int)((hdr.z >> sh) & 63u);
+                mn1 = (int)((hdr.z >> (sh + 8)) & 63u);
+            } else {
+                const uint32_t lo = hdr.w >> sh;
+                sc0 = (int)((lo & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4));
+                mn0 = (int)(((lo >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4));
+                sc1 = (int)(((lo >> 8) & 0xFu) | (((hdr.y >> (sh + 14)) & 3u) << 4));
+                mn1 = (int)(((lo >> 12) & 0xFu) | (((hdr.z >> (sh + 14)) & 3u) << 4));
+            }
+            const uint32_t q[4] = {r.q[i].x, r.q[i].y, r.q[i].z, r.q[i].w};
             int lh = 0, ll = 0, hh = 0, hl = 0;
 #pragma unroll
             for (int w = 0; w < 4; w++) {
@@ -183,26 +218,20 @@ __device__ inline float row_partial_q(const uint8_t *__restrict__ rowp, int unit
                 hh = __builtin_amdgcn_sdot4(hi, a.xh[i][4 + w], hh, false);
                 hl = __builtin_amdgcn_sdot4(hi, a.xl[i][4 + w], hl, false);
             }
-            float t0 = __fmul_rn((float)(lh * 256 + ll), a.s[i][0]);
-            float t1 = __fmul_rn((float)(hh * 256 + hl), a.s[i][1]);
-            float pos = __builtin_fmaf(__fmul_rn(d, sc0), t0, __fmul_rn(__fmul_rn(d, sc1), t1));
-            float neg = __builtin_fmaf(__fmul_rn(dmin, mn0), a.fx[i][0], __fmul_rn(__fmul_rn(dmin, mn1), a.fx[i][1]));
-            acc = __fadd_rn(acc, __fsub_rn(pos, neg));
+            // |sum(q*xq)| <= 15*32512*16 < 2^23 and |sum(xq)| <= 16*32512: 24-bit multiplies are exact
+            const int pos = __mul24(sc0, lh * 256 + ll) + __mul24(sc1, hh * 256 + hl);
+            const int neg = __mul24(mn0, a.sx[i][0]) + __mul24(mn1, a.sx[i][1]);
+            const float t = __fmul_rn(__fmul_rn(d, a.s[i]), (float)pos);
+            acc = __fadd_rn(acc, __builtin_fmaf(-__fmul_rn(dmin, a.s[i]), (float)neg, t));
         } else {  // Q8_0
-            const uint8_t *blk = rowp + (size_t)u * 34;
-            uint16_t db;
-            __builtin_memcpy(&db, blk, 2);
-            float d = half_bits_to_float(db);
+            float d = half_bits_to_float((uint16_t)r.d[i]);
             int sh = 0, sl = 0;
 #pragma unroll
             for (int w = 0; w < 8; w++) {
-                int qw;
-                __builtin_memcpy(&qw, blk + 2 + 4 * w, 4);
-                sh = __builtin_amdgcn_sdot4(qw, a.xh[i][w], sh, false);
-                sl = __builtin_amdgcn_sdot4(qw, a.xl[i][w], sl, false);
+                sh = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xh[i][w], sh, false);
+                sl = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xl[i][w], sl, false);
             }
-            // both halves of a Q8_0 block share one activation scale
-            float t = __fmul_rn((float)(sh * 256 + sl), a.s[i][0]);
+            float t = __fmul_rn((float)(sh * 256 + sl), a.s[i]);
             acc = __builtin_fmaf(d, t, acc);
         }
     }
@@ -254,7 +283,7 @@ __host__ __device__ inline size_t type_row_bytes(int type, int in_dim) {
 // ------------------------------------------------------------------------------------------
 // gate/up: act[a, j] = silu(<gate_e[j], x_t>) * <up_e[j], x_t>
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int VEC>
+template <int WT, int UPL, int VEC, int NIT>
 __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_kernel(
     const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, const float *__restrict__ x,
     const int32_t *__restrict__ ids, int k, int fixed_expert, int hidden, int inter, int n_experts,
@@ -275,21 +304,37 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_kernel(
     const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
 
     if constexpr (WT == T_Q4_K || WT == T_Q8_0) {
+        // rows_per_wave == NIT * rows_per_it: every weight load of the wave is issued before
+        // the first one is consumed
         const RowSplit rs = row_split(WT, hidden);
         const int sub = lane / rs.group, unit0 = lane % rs.group;
         LaneAct<UPL> la;
         load_lane_act<WT, UPL>(xrow, unit0, rs.units, la);
-        for (int r = 0; r < rows_per_wave; r += rs.rows_per_it) {
-            const int row = row0 + r + sub;
-            const bool ok = row < inter && r + sub < rows_per_wave;
-            float pg = 0.0f, pu = 0.0f;
-            if (ok) {
-                pg = row_partial_q<WT, UPL>(ge + (size_t)row * row_bytes, unit0, rs.units, la);
-                pu = row_partial_q<WT, UPL>(ue + (size_t)row * row_bytes, unit0, rs.units, la);
+        RawRow<WT, UPL> rg[NIT], ru[NIT];
+#pragma unroll
+        for (int i = 0; i < NIT; i++) {
+            const int row = row0 + i * rs.rows_per_it + sub;
+            const bool ok = row < inter;
+            load_row<WT, UPL>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
+            load_row<WT, UPL>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
+        }
+        float part[2 * NIT];
+#pragma unroll
+        for (int i = 0; i < NIT; i++) {
+            part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
+            part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
+        }
+        int count, offset;
+        reduce_partials<2 * NIT>(part, rs.group, lane, count, offset);
+        const int width = rs.group < 16 ? rs.group : 16;
+        if ((lane & (width - 1)) == 0) {
+#pragma unroll
+            for (int j = 0; j < 2 * NIT; j += 2) {
+                if (j < count) {
+                    const int row = row0 + ((offset + j) >> 1) * rs.rows_per_it + sub;
+                    if (row < inter) arow[row] = __fmul_rn(det_silu(part[j]), part[j + 1]);
+                }
             }
-            pg = group_sum(pg, rs.group);
-            pu = group_sum(pu, rs.group);
-            if (ok && unit0 == 0) arow[row] = __fmul_rn(det_silu(pg), pu);
         }
     } else {
         for (int r = 0; r < rows_per_wave; r++) {
@@ -307,7 +352,7 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_kernel(
 // ------------------------------------------------------------------------------------------
 // down: y[a, c] = <down_e[c], act[a]>
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int VEC>
+template <int WT, int UPL, int VEC, int NIT>
 __global__ __launch_bounds__(64 * kGemvWaves) void down_kernel(const uint8_t *__restrict__ down,
                                                                const float *__restrict__ act,
                                                                const int32_t *__restrict__ ids, int fixed_expert,
@@ -326,15 +371,29 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_kernel(const uint8_t *__
     if constexpr (WT == T_Q4_K || WT == T_Q8_0) {
         const RowSplit rs = row_split(WT, inter);
         const int sub = lane / rs.group, unit0 = lane % rs.group;
+        RawRow<WT, UPL> rd[NIT];
+#pragma unroll
+        for (int i = 0; i < NIT; i++) {
+            const int row = row0 + i * rs.rows_per_it + sub;
+            const bool ok = row < hidden;
+            load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i]);
+        }
         LaneAct<UPL> la;
         load_lane_act<WT, UPL>(arow, unit0, rs.units, la);
-        for (int r = 0; r < rows_per_wave; r += rs.rows_per_it) {
-            const int row = row0 + r + sub;
-            const bool ok = row < hidden && r + sub < rows_per_wave;
-            float p = 0.0f;
-            if (ok) p = row_partial_q<WT, UPL>(de + (size_t)row * row_bytes, unit0, rs.units, la);
-            p = group_sum(p, rs.group);
-            if (ok && unit0 == 0) yrow[row] = p;
+        float part[NIT];
+#pragma unroll
+        for (int i = 0; i < NIT; i++) part[i] = dot_row<WT, UPL>(rd[i], unit0, la);
+        int count, offset;
+        reduce_partials<NIT>(part, rs.group, lane, count, offset);
+        const int width = rs.group < 16 ? rs.group : 16;
+        if ((lane & (width - 1)) == 0) {
+#pragma unroll
+            for (int j = 0; j < NIT; j++) {
+                if (j < count) {
+                    const int row = row0 + (offset + j) * rs.rows_per_it + sub;
+                    if (row < hidden) yrow[row] = part[j];
+                }
+            }
         }
     } else {
         for (int r = 0; r < rows_per_wave; r++) {
@@ -347,39 +406,39 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_kernel(const uint8_t *__
     }
 }
 
-// Rows per wave so that a launch has a few thousand waves without making tiles tiny.
-static int pick_rows_per_wave(int out_dim, int n_assign, int rows_per_it) {
-    int rpw = rows_per_it;
-    // grow while the launch would still have >= 4096 waves
+// Float rows: rows per wave so that a launch has a few thousand waves without tiny tiles.
+static int pick_rows_per_wave(int out_dim, int n_assign) {
+    int rpw = 1;
     while ((long)((out_dim + rpw * 2 - 1) / (rpw * 2)) * n_assign >= 4096 && rpw < 64) rpw *= 2;
-    if (rpw < 4 && rows_per_it <= 4) rpw = 4 > rows_per_it ? 4 : rows_per_it;
-    return rpw;
+    return rpw < 4 ? 4 : rpw;
 }
 
+// Quantized rows: NIT iterations of rows_per_it rows per wave, all loads in flight at once.
+// NIT shrinks as units-per-lane grows so the raw rows stay in registers.
 template <int WT>
 static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, const int32_t *ids, int n_assign, int k,
                                    int fixed_expert, float *act, int32_t *flags, hipStream_t s) {
     constexpr bool quant = WT == T_Q4_K || WT == T_Q8_0;
-    int rows_per_it = 1, upl = 1;
-    if (quant) {
-        RowSplit rs = row_split(WT, b.hidden);
-        rows_per_it = rs.rows_per_it;
-        upl = (rs.units + 63) / 64;
-    }
-    const int rpw = pick_rows_per_wave(b.inter, n_assign, rows_per_it);
-    dim3 block(64 * kGemvWaves), grid(n_assign, (b.inter + rpw * kGemvWaves - 1) / (rpw * kGemvWaves));
-#define MUMMU_GU(UPL, VEC)                                                                                     \
-    gate_up_kernel<WT, UPL, VEC><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter, \
-                                                        b.n_experts, rpw, act, flags)
-    if (quant) {
-        if (upl == 1) MUMMU_GU(1, 1);
-        else if (upl == 2) MUMMU_GU(2, 1);
-        else if (upl <= 4) MUMMU_GU(4, 1);
+    dim3 block(64 * kGemvWaves);
+#define MUMMU_GU(UPL, VEC, NIT, RPW)                                                                                \
+    do {                                                                                                            \
+        const int rpw_ = (RPW);                                                                                     \
+        dim3 grid(n_assign, (b.inter + rpw_ * kGemvWaves - 1) / (rpw_ * kGemvWaves));                               \
+        gate_up_kernel<WT, UPL, VEC, NIT><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden,   \
+                                                                 b.inter, b.n_experts, rpw_, act, flags);           \
+    } while (0)
+    if constexpr (quant) {
+        const RowSplit rs = row_split(WT, b.hidden);
+        const int upl = (rs.units + 63) / 64;
+        if (upl == 1) MUMMU_GU(1, 1, 4, 4 * rs.rows_per_it);
+        else if (upl == 2) MUMMU_GU(2, 1, 2, 2 * rs.rows_per_it);
+        else if (upl <= 4) MUMMU_GU(4, 1, 1, rs.rows_per_it);
         else return hipErrorInvalidValue;
     } else {
+        const int rpw = pick_rows_per_wave(b.inter, n_assign);
         const bool vec = b.hidden % 4 == 0 && (((uintptr_t)x & 15) == 0);
-        if (vec) MUMMU_GU(1, 4);
-        else MUMMU_GU(1, 1);
+        if (vec) MUMMU_GU(1, 4, 1, rpw);
+        else MUMMU_GU(1, 1, 1, rpw);
     }
 #undef MUMMU_GU
     return hipGetLastError();
@@ -403,25 +462,25 @@ template <int WT>
 static hipError_t launch_down_t(const ExpertBanks &b, const float *act, const int32_t *ids, int n_assign,
                                 int fixed_expert, float *y, hipStream_t s) {
     constexpr bool quant = WT == T_Q4_K || WT == T_Q8_0;
-    int rows_per_it = 1, upl = 1;
-    if (quant) {
-        RowSplit rs = row_split(WT, b.inter);
-        rows_per_it = rs.rows_per_it;
-        upl = (rs.units + 63) / 64;
-    }
-    const int rpw = pick_rows_per_wave(b.hidden, n_assign, rows_per_it);
-    dim3 block(64 * kGemvWaves), grid(n_assign, (b.hidden + rpw * kGemvWaves - 1) / (rpw * kGemvWaves));
-#define MUMMU_DN(UPL, VEC)                                                                                        \
-    down_kernel<WT, UPL, VEC><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, \
-                                                     rpw, y)
-    if (quant) {
-        if (upl == 1) MUMMU_DN(1, 1);
-        else if (upl == 2) MUMMU_DN(2, 1);
-        else if (upl <= 4) MUMMU_DN(4, 1);
+    dim3 block(64 * kGemvWaves);
+#define MUMMU_DN(UPL, VEC, NIT, RPW)                                                                                \
+    do {                                                                                                            \
+        const int rpw_ = (RPW);                                                                                     \
+        dim3 grid(n_assign, (b.hidden + rpw_ * kGemvWaves - 1) / (rpw_ * kGemvWaves));                              \
+        down_kernel<WT, UPL, VEC, NIT><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter,    \
+                                                              b.n_experts, rpw_, y);                                \
+    } while (0)
+    if constexpr (quant) {
+        const RowSplit rs = row_split(WT, b.inter);
+        const int upl = (rs.units + 63) / 64;
+        if (upl == 1) MUMMU_DN(1, 1, 4, 4 * rs.rows_per_it);
+        else if (upl == 2) MUMMU_DN(2, 1, 2, 2 * rs.rows_per_it);
+        else if (upl <= 4) MUMMU_DN(4, 1, 1, rs.rows_per_it);
         else return hipErrorInvalidValue;
     } else {
-        if (b.inter % 4 == 0) MUMMU_DN(1, 4);
-        else MUMMU_DN(1, 1);
+        const int rpw = pick_rows_per_wave(b.hidden, n_assign);
+        if (b.inter % 4 == 0) MUMMU_DN(1, 4, 1, rpw);
+        else MUMMU_DN(1, 1, 1, rpw);
     }
 #undef MUMMU_DN
     return hipGetLastError();

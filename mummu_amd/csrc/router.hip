@@ -141,22 +141,24 @@ __device__ inline float lane_bcast(float v, int src) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
 }
 
+// JN = experts held per lane (num_experts <= 64 * JN).
+template <int JN>
 __global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
     const float *__restrict__ logits, int n, int n_experts, int k, int flavour, int norm, int32_t *__restrict__ ids,
     float *__restrict__ weights, unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
-    __shared__ float s_w[kTopkWavesPerBlock][kMaxExperts];
-    __shared__ int s_id[kTopkWavesPerBlock][kMaxExperts];
+    __shared__ float s_w[kTopkWavesPerBlock][64 * JN];
+    __shared__ int s_id[kTopkWavesPerBlock][64 * JN];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int t = blockIdx.x * kTopkWavesPerBlock + wave;
     if (t >= n) return;
     const float *row = logits + (size_t)t * (size_t)n_experts;
 
-    float p[kMaxExpertsPerLane];
+    float p[JN];
     bool bad = false;
     float mx = -__builtin_inff();
 #pragma unroll
-    for (int j = 0; j < kMaxExpertsPerLane; j++) {
+    for (int j = 0; j < JN; j++) {
         int e = lane + 64 * j;
         if (e < n_experts) {
             float l = row[e];
@@ -170,8 +172,7 @@ __global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
             p[j] = -__builtin_inff();
         }
     }
-    const bool any_bad = __any(bad);
-    if (any_bad) {
+    if (__any(bad)) {
         // Refused like experts.rs:546-553: flag it and emit a harmless, in-range routing so
         // the kernels downstream stay inside their buffers; the host reports the error.
         if (lane == 0) atomicAdd(&flags[FLAG_NONFINITE], 1);
@@ -183,61 +184,56 @@ __global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
     }
     mx = wave_max(mx);
 #pragma unroll
-    for (int j = 0; j < kMaxExpertsPerLane; j++) p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(p[j], mx)) : 0.0f;
+    for (int j = 0; j < JN; j++) p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(p[j], mx)) : 0.0f;
 
-    // normaliser: sequential over ascending expert id
+    // normaliser: sequential over ascending expert id (every lane computes the same sum).
+    // Experts past n_experts hold p = +0, which leaves the running sum unchanged bit for bit,
+    // so the loops run over all 64*JN slots and unroll without branches.
     if (flavour == 0) {
         float total = 0.0f;
 #pragma unroll
-        for (int j = 0; j < kMaxExpertsPerLane; j++) {
-            int lim = n_experts - 64 * j;
-            lim = lim > 64 ? 64 : lim;
-            for (int src = 0; src < lim; src++) total = __fadd_rn(total, lane_bcast(p[j], src));
+        for (int j = 0; j < JN; j++) {
+#pragma unroll
+            for (int src = 0; src < 64; src++) total = __fadd_rn(total, lane_bcast(p[j], src));
         }
 #pragma unroll
-        for (int j = 0; j < kMaxExpertsPerLane; j++) p[j] = __fdiv_rn(p[j], total);
+        for (int j = 0; j < JN; j++) p[j] = __fdiv_rn(p[j], total);
     } else {
         double total = 0.0;
 #pragma unroll
-        for (int j = 0; j < kMaxExpertsPerLane; j++) {
-            int lim = n_experts - 64 * j;
-            lim = lim > 64 ? 64 : lim;
-            for (int src = 0; src < lim; src++) total = __dadd_rn(total, (double)lane_bcast(p[j], src));
+        for (int j = 0; j < JN; j++) {
+#pragma unroll
+            for (int src = 0; src < 64; src++) total = __dadd_rn(total, (double)lane_bcast(p[j], src));
         }
         float scale = (float)__ddiv_rn(1.0, total);
 #pragma unroll
-        for (int j = 0; j < kMaxExpertsPerLane; j++) p[j] = __fmul_rn(p[j], scale);
+        for (int j = 0; j < JN; j++) p[j] = __fmul_rn(p[j], scale);
     }
 
-    // k rounds of wave-wide arg-max with (prob desc, id asc) order
-    unsigned taken = 0;
-    for (int s = 0; s < k; s++) {
-        float bp = -1.0f;
-        int bid = 0x7FFFFFFF;
+    // rank of each expert under (probability descending, id ascending); rank < k is its slot.
+    // A padding slot (p = 0, id >= n_experts) never outranks a real expert: it is not greater,
+    // and on a tie at 0 its id is higher.
+    int rank[JN];
 #pragma unroll
-        for (int j = 0; j < kMaxExpertsPerLane; j++) {
-            int e = lane + 64 * j;
-            if (e < n_experts && !(taken & (1u << j)) && p[j] > bp) {
-                bp = p[j];
-                bid = e;
-            }
-        }
+    for (int j = 0; j < JN; j++) rank[j] = 0;
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            float op = __shfl_xor(bp, off, kWave);
-            int oid = __shfl_xor(bid, off, kWave);
-            if (op > bp || (op == bp && oid < bid)) {
-                bp = op;
-                bid = oid;
-            }
-        }
-        if ((bid & 63) == lane) taken |= 1u << (bid >> 6);
-        if (lane == 0) {
-            s_w[wave][s] = bp;
-            s_id[wave][s] = bid;
+    for (int js = 0; js < JN; js++) {
+#pragma unroll
+        for (int src = 0; src < 64; src++) {
+            const float q = lane_bcast(p[js], src);
+            const int eq = 64 * js + src;
+#pragma unroll
+            for (int j = 0; j < JN; j++) rank[j] += (q > p[j]) || (q == p[j] && eq < lane + 64 * j);
         }
     }
-    // lane 0's LDS writes above are read by every lane of this same wave below
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        if (lane + 64 * j < n_experts && rank[j] < k) {
+            s_w[wave][rank[j]] = p[j];
+            s_id[wave][rank[j]] = lane + 64 * j;
+        }
+    }
+    // the slots written above are read by every lane of this same wave below
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
@@ -271,7 +267,13 @@ hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, i
     if (n <= 0) return hipSuccess;
     if (n_experts > kMaxExperts || k > n_experts || k < 1) return hipErrorInvalidValue;
     dim3 block(64 * kTopkWavesPerBlock), grid((n + kTopkWavesPerBlock - 1) / kTopkWavesPerBlock);
-    route_topk_kernel<<<grid, block, 0, s>>>(logits, n, n_experts, k, flavour, norm, ids, weights, hits, flags);
+#define MUMMU_TOPK(JN) \
+    route_topk_kernel<JN><<<grid, block, 0, s>>>(logits, n, n_experts, k, flavour, norm, ids, weights, hits, flags)
+    if (n_experts <= 64) MUMMU_TOPK(1);
+    else if (n_experts <= 128) MUMMU_TOPK(2);
+    else if (n_experts <= 256) MUMMU_TOPK(4);
+    else MUMMU_TOPK(8);
+#undef MUMMU_TOPK
     return hipGetLastError();
 }
 
