@@ -7,9 +7,31 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace mummu {
 
 constexpr int kWave = 64;
+
+// Phase marks for kernel timing studies.  A normal build compiles them away; with
+// -DMUMMU_TRACE every wave stores the shader clock at each mark into a caller-provided buffer
+// (8 slots per wave), set per translation unit through mummu_trace_set_<unit>().
+#ifdef MUMMU_TRACE
+static __device__ long long *g_trace_buf = nullptr;
+#define MUMMU_PHASE(ph)                                                                                           \
+    do {                                                                                                          \
+        if (g_trace_buf && (threadIdx.x & 63) == 0)                                                               \
+            g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + \
+                        (ph)] = clock64();                                                                        \
+    } while (0)
+#define MUMMU_TRACE_UNIT(name)                                                                      \
+    extern "C" __attribute__((visibility("default"))) int mummu_trace_set_##name(void *p) {         \
+        return (int)hipMemcpyToSymbol(HIP_SYMBOL(mummu::g_trace_buf), &p, sizeof(p));                \
+    }
+#else
+#define MUMMU_PHASE(ph) do { } while (0)
+#define MUMMU_TRACE_UNIT(name)
+#endif
 
 // ggml tensor type ids (the values stored in GGUF tensor tables).
 enum : int { T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_BF16 = 30 };
@@ -104,14 +126,15 @@ __device__ inline float dpp_move(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
 }
 
-// Sum over aligned groups of `width` lanes inside a 16-lane row (width in {1,2,4,8,16}); every
+// Sum over aligned groups of WIDTH lanes inside a 16-lane row (WIDTH in {1,2,4,8,16}); every
 // lane of a group ends with the group's sum.  Steps: xor 1, xor 2 (quad permutes), then the
 // half-row and row mirrors, which pair lanes of the two already-uniform halves.
-__device__ inline float row_group_sum(float v, int width) {
-    if (width >= 2) v = __fadd_rn(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
-    if (width >= 4) v = __fadd_rn(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
-    if (width >= 8) v = __fadd_rn(v, dpp_move<0x141>(v));  // row_half_mirror
-    if (width >= 16) v = __fadd_rn(v, dpp_move<0x140>(v)); // row_mirror
+template <int WIDTH>
+__device__ inline float row_group_sum(float v) {
+    if constexpr (WIDTH >= 2) v = __fadd_rn(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    if constexpr (WIDTH >= 4) v = __fadd_rn(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    if constexpr (WIDTH >= 8) v = __fadd_rn(v, dpp_move<0x141>(v));  // row_half_mirror
+    if constexpr (WIDTH >= 16) v = __fadd_rn(v, dpp_move<0x140>(v)); // row_mirror
     return v;
 }
 
@@ -128,51 +151,78 @@ __device__ inline float swap16_add(float a, float b) {
     return __fadd_rn(__int_as_float(r[0]), __int_as_float(r[1]));
 }
 
-// Reduce NV per-lane partials, each over aligned groups of `group` lanes (power of two), and
-// leave `count` finished sums in v[0..count): the value with original index offset + j sits
-// in v[j].  Crossing 32- and 16-lane boundaries halves the number of values a lane carries
-// (the two halves of the group finish different values), so the expensive steps are shared.
-template <int NV>
-__device__ inline void reduce_partials(float (&v)[NV], int group, int lane, int &count, int &offset) {
-    count = NV;
-    offset = 0;
-    if (group == 64) {
+// Number of finished sums a lane holds after reduce_partials<NV, GROUP>.
+template <int NV, int GROUP>
+__host__ __device__ constexpr int reduced_count() {
+    if (GROUP == 64) return NV >= 4 ? NV / 4 : 1;
+    if (GROUP == 32) return NV >= 2 ? NV / 2 : 1;
+    return NV;
+}
+
+// Reduce NV per-lane partials, each over aligned groups of GROUP lanes (power of two), and
+// leave reduced_count<NV, GROUP>() finished sums in v[0..count): the value with original index
+// (returned offset) + j sits in v[j].  Crossing the 32- and 16-lane boundaries halves the number
+// of values a lane carries (the two halves of the group finish different values), so those
+// steps are shared between values.
+template <int NV, int GROUP>
+__device__ inline int reduce_partials(float (&v)[NV], int lane) {
+    int offset = 0;
+    if constexpr (GROUP == 64) {
         if constexpr (NV >= 4) {
 #pragma unroll
             for (int j = 0; j < NV / 2; j++) v[j] = swap32_add(v[j], v[j + NV / 2]);
 #pragma unroll
             for (int j = 0; j < NV / 4; j++) v[j] = swap16_add(v[j], v[j + NV / 4]);
-            count = NV / 4;
             offset = ((lane >> 5) & 1) * (NV / 2) + ((lane >> 4) & 1) * (NV / 4);
         } else if constexpr (NV == 2) {
             v[0] = swap32_add(v[0], v[1]);
             v[0] = swap16_add(v[0], v[0]);
-            count = 1;
             offset = (lane >> 5) & 1;
         } else {
             v[0] = swap32_add(v[0], v[0]);
             v[0] = swap16_add(v[0], v[0]);
         }
-    } else if (group == 32) {
+    } else if constexpr (GROUP == 32) {
         if constexpr (NV >= 2) {
 #pragma unroll
             for (int j = 0; j < NV / 2; j++) v[j] = swap16_add(v[j], v[j + NV / 2]);
-            count = NV / 2;
             offset = ((lane >> 4) & 1) * (NV / 2);
         } else {
             v[0] = swap16_add(v[0], v[0]);
         }
     }
-    const int width = group < 16 ? group : 16;
+    constexpr int count = reduced_count<NV, GROUP>();
+    constexpr int width = GROUP < 16 ? GROUP : 16;
 #pragma unroll
-    for (int j = 0; j < NV; j++)
-        if (j < count) v[j] = row_group_sum(v[j], width);
+    for (int j = 0; j < count; j++) v[j] = row_group_sum<width>(v[j]);
+    return offset;
 }
 
+// Calls f(std::integral_constant<int, G>{}) with G the lane-group size g in {64, 32, ..., 1}.
+template <typename F>
+__device__ inline void dispatch_group(int g, F &&f) {
+    switch (g) {
+    case 64: f(std::integral_constant<int, 64>{}); break;
+    case 32: f(std::integral_constant<int, 32>{}); break;
+    case 16: f(std::integral_constant<int, 16>{}); break;
+    case 8: f(std::integral_constant<int, 8>{}); break;
+    case 4: f(std::integral_constant<int, 4>{}); break;
+    case 2: f(std::integral_constant<int, 2>{}); break;
+    default: f(std::integral_constant<int, 1>{}); break;
+    }
+}
+
+// Maximum over the wave, every lane gets it: four DPP steps inside each 16-lane row, then the
+// two lane swaps across rows.
 __device__ inline float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_int(v), __float_as_int(v), false, false);
+    v = fmaxf(__int_as_float(a[0]), __int_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_int(v), __float_as_int(v), false, false);
+    return fmaxf(__int_as_float(b[0]), __int_as_float(b[1]));
 }
 
 }  // namespace mummu

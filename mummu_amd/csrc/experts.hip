@@ -1,62 +1,58 @@
 // SwiGLU expert products for small batches (decode): packed GEMV straight off the GGUF bytes
-// resident in HBM, plus the weighted combine.
+// resident in HBM, and the weighted combine.
 //
 // Reference semantics: down(silu(gate.x) * (up.x)) per routed (token, expert) pair
 // (nn/moe.rs:312-316, models/qwen4exp/experts.rs:781-845), results scatter-added in
 // ascending expert id with two roundings (nn/moe.rs:1590-1601, experts.rs:1137-1148).
 //
-// Work decomposition: blockIdx.x = one (token, expert) assignment a = t*k + s, blockIdx.y = a
-// tile of output rows.  A wave walks its rows; the lanes of a wave split one weight row in
-// 16-byte units (Q4_K: one 16-byte slice of a super-block's nibbles; Q8_0: one 34-byte
-// block; float types: consecutive elements), so every global load is a contiguous run.
+// Work decomposition: blockIdx.x = one (token, expert) assignment a = t*k + s (or one token for
+// the fused down+combine), blockIdx.y = a tile of output rows.  The lanes of a wave split one
+// weight row in 16-byte units (Q4_K: one 16-byte slice of a super-block's nibbles; Q8_0: one
+// 34-byte block; float types: consecutive elements), so every global load is a contiguous
+// run, and a wave puts the loads of ALL its rows in flight before it consumes the first.
 //
-// Arithmetic of the quantized types (Q4_K, Q8_0): the activation row is quantized ONCE per
-// wave, in registers, to 16-bit integers xq = rint(x * 32512/amax) with one f32 scale
-// s = amax/32512 per activation block (64 elements under Q4_K - one low/high nibble chunk -
-// and 32 under Q8_0), split into two signed bytes xq = 256*hi + lo.  Weight codes and
-// activation bytes meet in v_dot4_i32_i8, so the block sums  sum(q * xq)  are exact integers;
-// only the scale products are floating point:
-//     Q8_0 block :              d * (s * float(sum q*xq))
-//     Q4_K sub-block pair:  (d*s) * float(sc0*sum(q0*xq0) + sc1*sum(q1*xq1))
-//                         - (dmin*s) * float(m0*sum(xq0) + m1*sum(xq1))
-// A 16-bit activation is ~2^-15 of the block maximum - about 100x finer than the int8
+// Arithmetic of the quantized types (Q4_K, Q8_0): activations arrive quantized to 16-bit
+// integers xq = rint(x * 32512/amax) with one f32 scale s = amax/32512 per 16 elements, split
+// into two signed bytes xq = 256*hi + lo (struct QAct).  Weight codes and activation bytes
+// meet in v_dot4_i32_i8, so every sum(q * xq) over 16 elements is an exact integer; only the
+// scale products are floating point:
+//     Q8_0 block (two halves):  d * (s0*float(sum q*xq|0) + s1*float(sum q*xq|1))
+//     Q4_K sub-block pair:      d * (s0*float(sc0*sum q0*xq0) + s1*float(sc1*sum q1*xq1))
+//                            - dmin * (s0*float(m0*sum xq0) + s1*float(m1*sum xq1))
+// A 16-bit activation is ~2^-15 of its block maximum - about 100x finer than the int8
 // activations llama.cpp multiplies these formats with - and, being a function of the token's
 // own row only, keeps the result independent of how many tokens share the call.
 // Float weight types (F32/F16/BF16) run an f32 fma chain per lane on the exact f32 value of
-// each weight.
+// each weight and the f32 activation.
 #include "device_utils.h"
 #include "kernels.h"
 
+MUMMU_TRACE_UNIT(experts)
+
 namespace mummu {
 
-constexpr int kGemvWaves = 4;  // waves per workgroup
+constexpr int kGemvWaves = 4;  // waves per workgroup of the float kernels
 
 // ------------------------------------------------------------------------------------------
-// Lane geometry of one weight row split in "units" (see file comment).
+// Lane geometry of one quantized weight row split in 32-element "units".
 // ------------------------------------------------------------------------------------------
 struct RowSplit {
-    int units;        // units per row
+    int units;        // units per row (in_dim / 32)
     int group;        // lanes that share a row (power of two, <= 64)
+    int group_log2;
     int rows_per_it;  // rows a wave handles per iteration = 64 / group
 };
 
-__host__ __device__ inline RowSplit row_split(int type, int in_dim) {
+__host__ __device__ inline RowSplit row_split(int in_dim) {
     RowSplit r;
-    r.units = type == T_Q4_K ? in_dim / 32 : in_dim / 32;  // Q4_K: 8 units per 256; Q8_0: 1 per 32
-    int g = 1;
-    while (g < r.units && g < 64) g <<= 1;
-    r.group = g;
-    r.rows_per_it = 64 / g;
+    r.units = in_dim / 32;
+    int lg = 0;
+    while ((1 << lg) < r.units && lg < 6) lg++;
+    r.group_log2 = lg;
+    r.group = 1 << lg;
+    r.rows_per_it = 64 >> lg;
     return r;
 }
-
-template <int UPL>
-struct LaneAct {
-    int xh[UPL][8];  // hi bytes of the lane's 32 activations, 4 per word
-    int xl[UPL][8];  // lo bytes
-    float s[UPL];    // scale of the activation block the lane's 32 elements belong to
-    int sx[UPL][2];  // sum(xq) over the first / second 16 elements (Q4_K min term)
-};
 
 // Start elements of the two 16-element halves unit u of a row covers.
 template <int WT>
@@ -71,66 +67,41 @@ __device__ inline void unit_halves(int u, int &e0, int &e1) {
     }
 }
 
-__device__ inline void quantize16(const float (&v)[16], float inv, int *xh, int *xl, int &sum) {
-    sum = 0;
-#pragma unroll
-    for (int w = 0; w < 4; w++) {
-        uint32_t hw = 0, lw = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            int q = (int)__builtin_rintf(__fmul_rn(v[4 * w + j], inv));
-            q = q > 32512 ? 32512 : (q < -32512 ? -32512 : q);
-            int lo = ((q + 128) & 255) - 128;
-            int hi = (q - lo) >> 8;
-            sum += q;
-            hw |= ((uint32_t)hi & 0xFFu) << (8 * j);
-            lw |= ((uint32_t)lo & 0xFFu) << (8 * j);
-        }
-        xh[w] = (int)hw;
-        xl[w] = (int)lw;
-    }
-}
+// The lane's share of a quantized activation row: 32 values (two 16-element blocks).
+template <int UPL>
+struct LaneAct {
+    int xh[UPL][8];   // hi bytes, 4 per word: words 0-3 first half, 4-7 second half
+    int xl[UPL][8];   // lo bytes
+    float s[UPL][2];  // scale of each half
+    int sx[UPL][2];   // sum(xq) of each half
+};
 
-// Quantize the lane's share of activation row `xrow` (f32, in_dim wide).  The activation
-// block (one scale) is the 64-element chunk for Q4_K - the lane's two halves plus those of the
-// neighbouring unit, lane ^ 1 - and the 32-element block for Q8_0.
 template <int WT, int UPL>
-__device__ inline void load_lane_act(const float *__restrict__ xrow, int unit0, int units, LaneAct<UPL> &a) {
+__device__ inline void load_lane_act(const QAct &q, size_t row, int d, int unit0, int units, LaneAct<UPL> &a) {
+    const int8_t *hi = q.hi + row * (size_t)d;
+    const int8_t *lo = q.lo + row * (size_t)d;
+    const float *sc = q.scale + row * (size_t)(d / 16);
+    const int32_t *sm = q.sum + row * (size_t)(d / 16);
 #pragma unroll
     for (int i = 0; i < UPL; i++) {
-        int u = unit0 + 64 * i;
-        bool on = u < units;
+        const int u = unit0 + 64 * i;
+        const bool on = u < units;
         int e0, e1;
         unit_halves<WT>(on ? u : 0, e0, e1);
-        float v0[16], v1[16];
-        const float4 *p0 = (const float4 *)(xrow + e0);
-        const float4 *p1 = (const float4 *)(xrow + e1);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float4 a0 = p0[j], a1 = p1[j];
-            v0[4 * j] = a0.x; v0[4 * j + 1] = a0.y; v0[4 * j + 2] = a0.z; v0[4 * j + 3] = a0.w;
-            v1[4 * j] = a1.x; v1[4 * j + 1] = a1.y; v1[4 * j + 2] = a1.z; v1[4 * j + 3] = a1.w;
-        }
-        float m = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 16; j++) m = fmaxf(m, fmaxf(fabsf(v0[j]), fabsf(v1[j])));
-        if (!on) m = 0.0f;
-        if constexpr (WT == T_Q4_K) m = fmaxf(m, dpp_move<0xB1>(m));  // lane ^ 1 holds the rest of the chunk
-        const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
-        a.s[i] = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
-        quantize16(v0, inv, &a.xh[i][0], &a.xl[i][0], a.sx[i][0]);
-        quantize16(v1, inv, &a.xh[i][4], &a.xl[i][4], a.sx[i][1]);
-        if (!on) {
-#pragma unroll
-            for (int w = 0; w < 8; w++) a.xh[i][w] = a.xl[i][w] = 0;
-            a.s[i] = 0.0f;
-            a.sx[i][0] = a.sx[i][1] = 0;
-        }
+        const int4 h0 = *(const int4 *)(hi + e0), h1 = *(const int4 *)(hi + e1);
+        const int4 l0 = *(const int4 *)(lo + e0), l1 = *(const int4 *)(lo + e1);
+        a.xh[i][0] = h0.x; a.xh[i][1] = h0.y; a.xh[i][2] = h0.z; a.xh[i][3] = h0.w;
+        a.xh[i][4] = h1.x; a.xh[i][5] = h1.y; a.xh[i][6] = h1.z; a.xh[i][7] = h1.w;
+        a.xl[i][0] = l0.x; a.xl[i][1] = l0.y; a.xl[i][2] = l0.z; a.xl[i][3] = l0.w;
+        a.xl[i][4] = l1.x; a.xl[i][5] = l1.y; a.xl[i][6] = l1.z; a.xl[i][7] = l1.w;
+        a.s[i][0] = on ? sc[e0 >> 4] : 0.0f;
+        a.s[i][1] = on ? sc[e1 >> 4] : 0.0f;
+        a.sx[i][0] = on ? sm[e0 >> 4] : 0;
+        a.sx[i][1] = on ? sm[e1 >> 4] : 0;
     }
 }
 
-// The lane's raw share of one quantized weight row, as loaded (nothing decoded yet), so that a
-// wave can put the loads of several rows in flight before it touches any of them.
+// The lane's raw share of one quantized weight row, as loaded (nothing decoded yet).
 template <int WT, int UPL>
 struct RawRow;
 template <int UPL>
@@ -174,13 +145,8 @@ __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int
     }
 }
 
-// The lane's partial of <row, activation>.  A lane that loaded nothing holds zero scales and
-// contributes exactly 0.
-//   Q4_K: with q the 4-bit codes, xq the 16-bit activations of the lane's two 16-element halves
-//   (sub-blocks 2c and 2c+1 of one super-block, one activation scale s),
-//       (d*s) * float(sc0*sum(q0*xq0) + sc1*sum(q1*xq1)) - (dmin*s) * float(m0*sum(xq0) + m1*sum(xq1))
-//   where every sum and both 6-bit-weighted combinations are exact integers.
-//   Q8_0: d * (s * float(sum(q*xq))).
+// The lane's partial of <row, activation> (formulas in the file comment).  A lane that loaded
+// nothing holds zero scales and contributes exactly 0.
 template <int WT, int UPL>
 __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneAct<UPL> &a) {
     float acc = 0.0f;
@@ -219,19 +185,22 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
                 hl = __builtin_amdgcn_sdot4(hi, a.xl[i][4 + w], hl, false);
             }
             // |sum(q*xq)| <= 15*32512*16 < 2^23 and |sum(xq)| <= 16*32512: 24-bit multiplies are exact
-            const int pos = __mul24(sc0, lh * 256 + ll) + __mul24(sc1, hh * 256 + hl);
-            const int neg = __mul24(mn0, a.sx[i][0]) + __mul24(mn1, a.sx[i][1]);
-            const float t = __fmul_rn(__fmul_rn(d, a.s[i]), (float)pos);
-            acc = __fadd_rn(acc, __builtin_fmaf(-__fmul_rn(dmin, a.s[i]), (float)neg, t));
+            const float p0 = (float)__mul24(sc0, lh * 256 + ll), p1 = (float)__mul24(sc1, hh * 256 + hl);
+            const float n0 = (float)__mul24(mn0, a.sx[i][0]), n1 = (float)__mul24(mn1, a.sx[i][1]);
+            const float pos = __builtin_fmaf(a.s[i][0], p0, __fmul_rn(a.s[i][1], p1));
+            const float neg = __builtin_fmaf(a.s[i][0], n0, __fmul_rn(a.s[i][1], n1));
+            acc = __fadd_rn(acc, __builtin_fmaf(-dmin, neg, __fmul_rn(d, pos)));
         } else {  // Q8_0
-            float d = half_bits_to_float((uint16_t)r.d[i]);
-            int sh = 0, sl = 0;
+            const float d = half_bits_to_float((uint16_t)r.d[i]);
+            int h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
-            for (int w = 0; w < 8; w++) {
-                sh = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xh[i][w], sh, false);
-                sl = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xl[i][w], sl, false);
+            for (int w = 0; w < 4; w++) {
+                h0 = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xh[i][w], h0, false);
+                l0 = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xl[i][w], l0, false);
+                h1 = __builtin_amdgcn_sdot4((int)r.q[i][4 + w], a.xh[i][4 + w], h1, false);
+                l1 = __builtin_amdgcn_sdot4((int)r.q[i][4 + w], a.xl[i][4 + w], l1, false);
             }
-            float t = __fmul_rn((float)(sh * 256 + sl), a.s[i]);
+            const float t = __builtin_fmaf(a.s[i][0], (float)(h0 * 256 + l0), __fmul_rn(a.s[i][1], (float)(h1 * 256 + l1)));
             acc = __builtin_fmaf(d, t, acc);
         }
     }
@@ -281,17 +250,95 @@ __host__ __device__ inline size_t type_row_bytes(int type, int in_dim) {
 }
 
 // ------------------------------------------------------------------------------------------
-// gate/up: act[a, j] = silu(<gate_e[j], x_t>) * <up_e[j], x_t>
+// gate/up, quantized banks: NIT iterations of rows_per_it rows per wave; the workgroup's
+// rows_per_block = waves*NIT*rows_per_it output rows are a whole number of 16-element
+// activation blocks, quantized for the down projection in the epilogue.
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int VEC, int NIT>
-__global__ __launch_bounds__(64 * kGemvWaves) void gate_up_kernel(
+template <int WT, int UPL, int NIT, bool ACTQ>
+__global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restrict__ gate,
+                                                         const uint8_t *__restrict__ up, QAct xq,
+                                                         const int32_t *__restrict__ ids, int k, int fixed_expert,
+                                                         int hidden, int inter, int n_experts,
+                                                         float *__restrict__ act, QAct actq,
+                                                         int32_t *__restrict__ flags) {
+    extern __shared__ float s_act[];  // rows_per_block floats
+    MUMMU_PHASE(0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.z;  // grid = (slot, row tile, token)
+    const int a = t * gridDim.x + blockIdx.x;
+    const int e = fixed_expert >= 0 ? fixed_expert : ids[a];
+    if ((unsigned)e >= (unsigned)n_experts) {
+        if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
+        return;
+    }
+    const RowSplit rs = row_split(hidden);
+    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
+    const int rows_per_wave = NIT * rs.rows_per_it;
+    const int rows_per_block = rows_per_wave * (blockDim.x >> 6);
+    const int block_row0 = blockIdx.y * rows_per_block;
+    const int row0 = block_row0 + wave * rows_per_wave;
+    const size_t row_bytes = type_row_bytes(WT, hidden);
+    const uint8_t *ge = gate + (size_t)e * (size_t)inter * row_bytes;
+    const uint8_t *ue = up + (size_t)e * (size_t)inter * row_bytes;
+
+    LaneAct<UPL> la;
+    load_lane_act<WT, UPL>(xq, (size_t)t, hidden, unit0, rs.units, la);
+    RawRow<WT, UPL> rg[NIT], ru[NIT];
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int row = row0 + i * rs.rows_per_it + sub;
+        const bool ok = row < inter;
+        load_row<WT, UPL>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
+        load_row<WT, UPL>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
+    }
+    MUMMU_PHASE(1);
+    float part[2 * NIT];
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
+        part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
+    }
+    MUMMU_PHASE(2);
+    dispatch_group(rs.group, [&](auto group_tag) {
+        constexpr int GROUP = decltype(group_tag)::value;
+        const int offset = reduce_partials<2 * NIT, GROUP>(part, lane);
+        constexpr int count = reduced_count<2 * NIT, GROUP>();
+        constexpr int width = GROUP < 16 ? GROUP : 16;
+        if ((lane & (width - 1)) == 0) {
+#pragma unroll
+            for (int j = 0; j < count; j += 2) {
+                const int row = row0 + ((offset + j) >> 1) * rs.rows_per_it + sub;
+                if (row < inter) {
+                    const float v = __fmul_rn(det_silu(part[j]), part[j + 1]);
+                    if (ACTQ) s_act[row - block_row0] = v;
+                    else act[(size_t)a * (size_t)inter + row] = v;
+                }
+            }
+        }
+    });
+    MUMMU_PHASE(3);
+    if (ACTQ) {
+        __syncthreads();
+        MUMMU_PHASE(4);
+        for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
+            const int row = block_row0 + r;
+            const bool on = row < inter;  // inter % 16 == 0: a 16-lane row is all on or all off
+            quantize_store16(on ? s_act[r] : 0.0f, on, actq, (size_t)a, inter, on ? row : 0);
+        }
+    }
+    MUMMU_PHASE(5);
+}
+
+// gate/up, float banks.
+template <int WT, int VEC>
+__global__ __launch_bounds__(64 * kGemvWaves) void gate_up_f_kernel(
     const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, const float *__restrict__ x,
     const int32_t *__restrict__ ids, int k, int fixed_expert, int hidden, int inter, int n_experts,
     int rows_per_wave, float *__restrict__ act, int32_t *__restrict__ flags) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int a = blockIdx.x;
+    const int t = blockIdx.z;  // grid = (slot, row tile, token)
+    const int a = t * gridDim.x + blockIdx.x;
     const int e = fixed_expert >= 0 ? fixed_expert : ids[a];
-    const int t = fixed_expert >= 0 ? a : a / k;
     if ((unsigned)e >= (unsigned)n_experts) {
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
@@ -302,110 +349,207 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_kernel(
     const float *xrow = x + (size_t)t * (size_t)hidden;
     float *arow = act + (size_t)a * (size_t)inter;
     const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
-
-    if constexpr (WT == T_Q4_K || WT == T_Q8_0) {
-        // rows_per_wave == NIT * rows_per_it: every weight load of the wave is issued before
-        // the first one is consumed
-        const RowSplit rs = row_split(WT, hidden);
-        const int sub = lane / rs.group, unit0 = lane % rs.group;
-        LaneAct<UPL> la;
-        load_lane_act<WT, UPL>(xrow, unit0, rs.units, la);
-        RawRow<WT, UPL> rg[NIT], ru[NIT];
-#pragma unroll
-        for (int i = 0; i < NIT; i++) {
-            const int row = row0 + i * rs.rows_per_it + sub;
-            const bool ok = row < inter;
-            load_row<WT, UPL>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
-            load_row<WT, UPL>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
-        }
-        float part[2 * NIT];
-#pragma unroll
-        for (int i = 0; i < NIT; i++) {
-            part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
-            part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
-        }
-        int count, offset;
-        reduce_partials<2 * NIT>(part, rs.group, lane, count, offset);
-        const int width = rs.group < 16 ? rs.group : 16;
-        if ((lane & (width - 1)) == 0) {
-#pragma unroll
-            for (int j = 0; j < 2 * NIT; j += 2) {
-                if (j < count) {
-                    const int row = row0 + ((offset + j) >> 1) * rs.rows_per_it + sub;
-                    if (row < inter) arow[row] = __fmul_rn(det_silu(part[j]), part[j + 1]);
-                }
-            }
-        }
-    } else {
-        for (int r = 0; r < rows_per_wave; r++) {
-            const int row = row0 + r;
-            if (row >= inter) break;
-            float pg = row_partial_f<WT, VEC>(ge + (size_t)row * row_bytes, xrow, hidden, lane);
-            float pu = row_partial_f<WT, VEC>(ue + (size_t)row * row_bytes, xrow, hidden, lane);
-            pg = wave_sum(pg);
-            pu = wave_sum(pu);
-            if (lane == 0) arow[row] = __fmul_rn(det_silu(pg), pu);
-        }
+    for (int r = 0; r < rows_per_wave; r++) {
+        const int row = row0 + r;
+        if (row >= inter) break;
+        float pg = row_partial_f<WT, VEC>(ge + (size_t)row * row_bytes, xrow, hidden, lane);
+        float pu = row_partial_f<WT, VEC>(ue + (size_t)row * row_bytes, xrow, hidden, lane);
+        pg = wave_sum(pg);
+        pu = wave_sum(pu);
+        if (lane == 0) arow[row] = __fmul_rn(det_silu(pg), pu);
     }
+}
+
+// x [n, d] f32 -> QAct: one lane per element, 16-lane rows are the activation blocks.
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const float *__restrict__ x, int n, int d, QAct q) {
+    const size_t total = (size_t)n * (size_t)d;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool on = i < total;  // d % 16 == 0: whole 16-lane rows are on or off together
+    const size_t row = on ? i / (size_t)d : 0;
+    const int elem = on ? (int)(i % (size_t)d) : 0;
+    quantize_store16(on ? x[i] : 0.0f, on, q, row, d, elem);
+}
+
+hipError_t launch_quantize_rows(const float *x, int n, int d, QAct q, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (d % 16) return hipErrorInvalidValue;
+    const size_t total = (size_t)n * (size_t)d;
+    quantize_rows_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>(x, n, d, q);
+    return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------
 // down: y[a, c] = <down_e[c], act[a]>
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int VEC, int NIT>
-__global__ __launch_bounds__(64 * kGemvWaves) void down_kernel(const uint8_t *__restrict__ down,
-                                                               const float *__restrict__ act,
-                                                               const int32_t *__restrict__ ids, int fixed_expert,
-                                                               int hidden, int inter, int n_experts, int rows_per_wave,
-                                                               float *__restrict__ y) {
+template <int WT, int UPL, int NIT>
+__global__ __launch_bounds__(64 * kGemvWaves) void down_q_kernel(const uint8_t *__restrict__ down, QAct actq,
+                                                                 const int32_t *__restrict__ ids, int fixed_expert,
+                                                                 int hidden, int inter, int n_experts,
+                                                                 float *__restrict__ y) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int a = blockIdx.x;
+    const int a = blockIdx.z * gridDim.x + blockIdx.x;  // grid = (slot, row tile, token)
     const int e = fixed_expert >= 0 ? fixed_expert : ids[a];
     if ((unsigned)e >= (unsigned)n_experts) return;  // flagged by gate_up
+    const RowSplit rs = row_split(inter);
+    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
+    const int rows_per_wave = NIT * rs.rows_per_it;
+    const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
+    const size_t row_bytes = type_row_bytes(WT, inter);
+    const uint8_t *de = down + (size_t)e * (size_t)hidden * row_bytes;
+    float *yrow = y + (size_t)a * (size_t)hidden;
+
+    RawRow<WT, UPL> rd[NIT];
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int row = row0 + i * rs.rows_per_it + sub;
+        const bool ok = row < hidden;
+        load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i]);
+    }
+    LaneAct<UPL> la;
+    load_lane_act<WT, UPL>(actq, (size_t)a, inter, unit0, rs.units, la);
+    float part[NIT];
+#pragma unroll
+    for (int i = 0; i < NIT; i++) part[i] = dot_row<WT, UPL>(rd[i], unit0, la);
+    dispatch_group(rs.group, [&](auto group_tag) {
+        constexpr int GROUP = decltype(group_tag)::value;
+        const int offset = reduce_partials<NIT, GROUP>(part, lane);
+        constexpr int count = reduced_count<NIT, GROUP>();
+        constexpr int width = GROUP < 16 ? GROUP : 16;
+        if ((lane & (width - 1)) == 0) {
+#pragma unroll
+            for (int j = 0; j < count; j++) {
+                const int row = row0 + (offset + j) * rs.rows_per_it + sub;
+                if (row < hidden) yrow[row] = part[j];
+            }
+        }
+    });
+}
+
+template <int WT, int VEC>
+__global__ __launch_bounds__(64 * kGemvWaves) void down_f_kernel(const uint8_t *__restrict__ down,
+                                                                 const float *__restrict__ act,
+                                                                 const int32_t *__restrict__ ids, int fixed_expert,
+                                                                 int hidden, int inter, int n_experts, int rows_per_wave,
+                                                                 float *__restrict__ y) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int a = blockIdx.z * gridDim.x + blockIdx.x;  // grid = (slot, row tile, token)
+    const int e = fixed_expert >= 0 ? fixed_expert : ids[a];
+    if ((unsigned)e >= (unsigned)n_experts) return;
     const size_t row_bytes = type_row_bytes(WT, inter);
     const uint8_t *de = down + (size_t)e * (size_t)hidden * row_bytes;
     const float *arow = act + (size_t)a * (size_t)inter;
     float *yrow = y + (size_t)a * (size_t)hidden;
     const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
-
-    if constexpr (WT == T_Q4_K || WT == T_Q8_0) {
-        const RowSplit rs = row_split(WT, inter);
-        const int sub = lane / rs.group, unit0 = lane % rs.group;
-        RawRow<WT, UPL> rd[NIT];
-#pragma unroll
-        for (int i = 0; i < NIT; i++) {
-            const int row = row0 + i * rs.rows_per_it + sub;
-            const bool ok = row < hidden;
-            load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i]);
-        }
-        LaneAct<UPL> la;
-        load_lane_act<WT, UPL>(arow, unit0, rs.units, la);
-        float part[NIT];
-#pragma unroll
-        for (int i = 0; i < NIT; i++) part[i] = dot_row<WT, UPL>(rd[i], unit0, la);
-        int count, offset;
-        reduce_partials<NIT>(part, rs.group, lane, count, offset);
-        const int width = rs.group < 16 ? rs.group : 16;
-        if ((lane & (width - 1)) == 0) {
-#pragma unroll
-            for (int j = 0; j < NIT; j++) {
-                if (j < count) {
-                    const int row = row0 + (offset + j) * rs.rows_per_it + sub;
-                    if (row < hidden) yrow[row] = part[j];
-                }
-            }
-        }
-    } else {
-        for (int r = 0; r < rows_per_wave; r++) {
-            const int row = row0 + r;
-            if (row >= hidden) break;
-            float p = row_partial_f<WT, VEC>(de + (size_t)row * row_bytes, arow, inter, lane);
-            p = wave_sum(p);
-            if (lane == 0) yrow[row] = p;
-        }
+    for (int r = 0; r < rows_per_wave; r++) {
+        const int row = row0 + r;
+        if (row >= hidden) break;
+        float p = row_partial_f<WT, VEC>(de + (size_t)row * row_bytes, arow, inter, lane);
+        p = wave_sum(p);
+        if (lane == 0) yrow[row] = p;
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// down + combine in one launch (quantized down bank, top_k <= 4*KPW): blockIdx.x = token,
+// blockIdx.y = tile of NIT*rows_per_it output rows.  The 4 waves split the token's experts
+// in ascending-id order, KPW each; their row sums meet in LDS and are combined in that same
+// order, multiply and add rounded separately.
+// ------------------------------------------------------------------------------------------
+constexpr int kDcWaves = 4;
+
+template <int WT, int UPL, int NIT, int KPW>
+__global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
+    const uint8_t *__restrict__ down, QAct actq, const int32_t *__restrict__ ids, const float *__restrict__ weights,
+    int k, int hidden, int inter, int n_experts, const float *__restrict__ residual, float *__restrict__ out) {
+    constexpr int KMAX = kDcWaves * KPW;
+    extern __shared__ float s_mem[];  // [KMAX][rows_per_block] row sums, then [KMAX] weights
+    MUMMU_PHASE(0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x;
+    const RowSplit rs = row_split(inter);
+    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
+    const int rows_per_block = NIT * rs.rows_per_it;
+    const int row0 = blockIdx.y * rows_per_block;
+    float *s_y = s_mem;
+    float *s_w = s_mem + KMAX * rows_per_block;
+    const size_t row_bytes = type_row_bytes(WT, inter);
+
+    // rank of every slot by ascending expert id (ids of one token are distinct); lanes >= k idle
+    const int my_id = lane < k ? ids[(size_t)t * k + lane] : 0x7FFFFFFF;
+    const float my_w = lane < k ? weights[(size_t)t * k + lane] : 0.0f;
+    int rank = 0;
+#pragma unroll
+    for (int j = 0; j < KMAX; j++) {
+        const int o = __builtin_amdgcn_readlane(my_id, j);
+        rank += (j < k) && (o < my_id || (o == my_id && j < lane));
+    }
+    // this wave's positions p = wave*KPW + i in the ascending order
+    int e_p[KPW], a_p[KPW];
+    bool on_p[KPW];
+#pragma unroll
+    for (int i = 0; i < KPW; i++) {
+        const int p = wave * KPW + i;
+        const unsigned long long m = __ballot(lane < k && rank == p);
+        on_p[i] = m != 0ull;
+        const int src = on_p[i] ? (int)__builtin_ctzll(m) : 0;
+        e_p[i] = __builtin_amdgcn_readlane(my_id, src);
+        a_p[i] = t * k + src;
+        on_p[i] = on_p[i] && (unsigned)e_p[i] < (unsigned)n_experts;
+        const float wp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), src));
+        if (lane == 0) s_w[p] = on_p[i] ? wp : 0.0f;
+    }
+
+    MUMMU_PHASE(1);
+    RawRow<WT, UPL> rd[KPW][NIT];
+    LaneAct<UPL> la[KPW];
+#pragma unroll
+    for (int i = 0; i < KPW; i++) {
+        const uint8_t *de = down + (size_t)(on_p[i] ? e_p[i] : 0) * (size_t)hidden * row_bytes;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int row = row0 + it * rs.rows_per_it + sub;
+            const bool ok = on_p[i] && row < hidden;
+            load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i][it]);
+        }
+        load_lane_act<WT, UPL>(actq, (size_t)(on_p[i] ? a_p[i] : 0), inter, unit0, rs.units, la[i]);
+    }
+    float part[KPW * NIT];
+#pragma unroll
+    for (int i = 0; i < KPW; i++)
+#pragma unroll
+        for (int it = 0; it < NIT; it++) part[i * NIT + it] = dot_row<WT, UPL>(rd[i][it], unit0, la[i]);
+    MUMMU_PHASE(2);
+    dispatch_group(rs.group, [&](auto group_tag) {
+        constexpr int GROUP = decltype(group_tag)::value;
+        const int offset = reduce_partials<KPW * NIT, GROUP>(part, lane);
+        constexpr int count = reduced_count<KPW * NIT, GROUP>();
+        constexpr int width = GROUP < 16 ? GROUP : 16;
+        if ((lane & (width - 1)) == 0) {
+#pragma unroll
+            for (int j = 0; j < count; j++) {
+                const int idx = offset + j;
+                const int i = idx / NIT, it = idx % NIT;
+                s_y[(wave * KPW + i) * rows_per_block + it * rs.rows_per_it + sub] = part[j];
+            }
+        }
+    });
+    MUMMU_PHASE(3);
+    __syncthreads();
+    MUMMU_PHASE(4);
+    for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
+        const int row = row0 + r;
+        if (row >= hidden) continue;
+        float sum = 0.0f;
+        for (int p = 0; p < k; p++) sum = __fadd_rn(sum, __fmul_rn(s_w[p], s_y[p * rows_per_block + r]));
+        const size_t o = (size_t)t * (size_t)hidden + row;
+        out[o] = residual ? __fadd_rn(residual[o], sum) : sum;
+    }
+    MUMMU_PHASE(5);
+}
+
+// ------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------
 // Float rows: rows per wave so that a launch has a few thousand waves without tiny tiles.
 static int pick_rows_per_wave(int out_dim, int n_assign) {
     int rpw = 1;
@@ -413,90 +557,149 @@ static int pick_rows_per_wave(int out_dim, int n_assign) {
     return rpw < 4 ? 4 : rpw;
 }
 
-// Quantized rows: NIT iterations of rows_per_it rows per wave, all loads in flight at once.
-// NIT shrinks as units-per-lane grows so the raw rows stay in registers.
 template <int WT>
-static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, const int32_t *ids, int n_assign, int k,
-                                   int fixed_expert, float *act, int32_t *flags, hipStream_t s) {
+static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq, const int32_t *ids, int n_assign,
+                                   int k, int fixed_expert, float *act, QAct actq, int32_t *flags, hipStream_t s) {
     constexpr bool quant = WT == T_Q4_K || WT == T_Q8_0;
-    dim3 block(64 * kGemvWaves);
-#define MUMMU_GU(UPL, VEC, NIT, RPW)                                                                                \
-    do {                                                                                                            \
-        const int rpw_ = (RPW);                                                                                     \
-        dim3 grid(n_assign, (b.inter + rpw_ * kGemvWaves - 1) / (rpw_ * kGemvWaves));                               \
-        gate_up_kernel<WT, UPL, VEC, NIT><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden,   \
-                                                                 b.inter, b.n_experts, rpw_, act, flags);           \
-    } while (0)
+    const bool actq_out = is_quant_type(b.down_type);
+    const int slots = fixed_expert >= 0 ? 1 : k;  // n_assign = tokens * slots
     if constexpr (quant) {
-        const RowSplit rs = row_split(WT, b.hidden);
+        const RowSplit rs = row_split(b.hidden);
         const int upl = (rs.units + 63) / 64;
-        if (upl == 1) MUMMU_GU(1, 1, 4, 4 * rs.rows_per_it);
-        else if (upl == 2) MUMMU_GU(2, 1, 2, 2 * rs.rows_per_it);
-        else if (upl <= 4) MUMMU_GU(4, 1, 1, rs.rows_per_it);
+#define MUMMU_GUQ(UPL, NIT)                                                                                     \
+    do {                                                                                                        \
+        int waves = 4;                                                                                          \
+        while (waves * (NIT)*rs.rows_per_it < 16) waves *= 2; /* whole 16-element activation blocks */          \
+        const int rpb = waves * (NIT)*rs.rows_per_it;                                                           \
+        dim3 grid(slots, (b.inter + rpb - 1) / rpb, n_assign / slots), block(64 * waves);                                      \
+        const size_t lds = sizeof(float) * (size_t)rpb;                                                         \
+        if (actq_out)                                                                                           \
+            gate_up_q_kernel<WT, UPL, NIT, true><<<grid, block, lds, s>>>(                                      \
+                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags);      \
+        else                                                                                                    \
+            gate_up_q_kernel<WT, UPL, NIT, false><<<grid, block, lds, s>>>(                                     \
+                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags);      \
+    } while (0)
+        if (upl == 1) MUMMU_GUQ(1, 4);
+        else if (upl == 2) MUMMU_GUQ(2, 2);
+        else if (upl <= 4) MUMMU_GUQ(4, 1);
         else return hipErrorInvalidValue;
+#undef MUMMU_GUQ
     } else {
         const int rpw = pick_rows_per_wave(b.inter, n_assign);
+        dim3 block(64 * kGemvWaves), grid(slots, (b.inter + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_assign / slots);
         const bool vec = b.hidden % 4 == 0 && (((uintptr_t)x & 15) == 0);
-        if (vec) MUMMU_GU(1, 4, 1, rpw);
-        else MUMMU_GU(1, 1, 1, rpw);
+        if (vec)
+            gate_up_f_kernel<WT, 4><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
+                                                           b.n_experts, rpw, act, flags);
+        else
+            gate_up_f_kernel<WT, 1><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
+                                                           b.n_experts, rpw, act, flags);
+        if (actq_out) {  // float gate/up feeding a quantized down bank: quantize the f32 act rows
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            return launch_quantize_rows(act, n_assign, b.inter, actq, s);
+        }
     }
-#undef MUMMU_GU
     return hipGetLastError();
 }
 
-hipError_t launch_gate_up(const ExpertBanks &b, const float *x, const int32_t *ids, int n_assign, int k,
-                          int fixed_expert, float *act, int32_t *flags, hipStream_t s) {
+hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const int32_t *ids, int n_assign, int k,
+                          int fixed_expert, float *act, QAct actq, int32_t *flags, hipStream_t s) {
     if (n_assign <= 0) return hipSuccess;
     if (b.gate_type != b.up_type) return hipErrorInvalidValue;
+    if (n_assign / (fixed_expert >= 0 ? 1 : k) > 65535) return hipErrorInvalidValue;
     switch (b.gate_type) {
-    case T_F32: return launch_gate_up_t<T_F32>(b, x, ids, n_assign, k, fixed_expert, act, flags, s);
-    case T_F16: return launch_gate_up_t<T_F16>(b, x, ids, n_assign, k, fixed_expert, act, flags, s);
-    case T_BF16: return launch_gate_up_t<T_BF16>(b, x, ids, n_assign, k, fixed_expert, act, flags, s);
-    case T_Q8_0: return launch_gate_up_t<T_Q8_0>(b, x, ids, n_assign, k, fixed_expert, act, flags, s);
-    case T_Q4_K: return launch_gate_up_t<T_Q4_K>(b, x, ids, n_assign, k, fixed_expert, act, flags, s);
+    case T_F32: return launch_gate_up_t<T_F32>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
+    case T_F16: return launch_gate_up_t<T_F16>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
+    case T_BF16: return launch_gate_up_t<T_BF16>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
+    case T_Q8_0: return launch_gate_up_t<T_Q8_0>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
+    case T_Q4_K: return launch_gate_up_t<T_Q4_K>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
     default: return hipErrorInvalidValue;
     }
 }
 
 template <int WT>
-static hipError_t launch_down_t(const ExpertBanks &b, const float *act, const int32_t *ids, int n_assign,
-                                int fixed_expert, float *y, hipStream_t s) {
+static hipError_t launch_down_t(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign,
+                                int k, int fixed_expert, float *y, hipStream_t s) {
     constexpr bool quant = WT == T_Q4_K || WT == T_Q8_0;
+    const int slots = fixed_expert >= 0 ? 1 : k;  // n_assign = tokens * slots
     dim3 block(64 * kGemvWaves);
-#define MUMMU_DN(UPL, VEC, NIT, RPW)                                                                                \
-    do {                                                                                                            \
-        const int rpw_ = (RPW);                                                                                     \
-        dim3 grid(n_assign, (b.hidden + rpw_ * kGemvWaves - 1) / (rpw_ * kGemvWaves));                              \
-        down_kernel<WT, UPL, VEC, NIT><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter,    \
-                                                              b.n_experts, rpw_, y);                                \
-    } while (0)
     if constexpr (quant) {
-        const RowSplit rs = row_split(WT, b.inter);
+        const RowSplit rs = row_split(b.inter);
         const int upl = (rs.units + 63) / 64;
-        if (upl == 1) MUMMU_DN(1, 1, 4, 4 * rs.rows_per_it);
-        else if (upl == 2) MUMMU_DN(2, 1, 2, 2 * rs.rows_per_it);
-        else if (upl <= 4) MUMMU_DN(4, 1, 1, rs.rows_per_it);
+#define MUMMU_DNQ(UPL, NIT)                                                                                    \
+    do {                                                                                                       \
+        const int rpb = kGemvWaves * (NIT)*rs.rows_per_it;                                                     \
+        dim3 grid(slots, (b.hidden + rpb - 1) / rpb, n_assign / slots);                                        \
+        down_q_kernel<WT, UPL, NIT><<<grid, block, 0, s>>>(b.down, actq, ids, fixed_expert, b.hidden, b.inter, \
+                                                           b.n_experts, y);                                    \
+    } while (0)
+        if (upl == 1) MUMMU_DNQ(1, 4);
+        else if (upl == 2) MUMMU_DNQ(2, 2);
+        else if (upl <= 4) MUMMU_DNQ(4, 1);
         else return hipErrorInvalidValue;
+#undef MUMMU_DNQ
     } else {
         const int rpw = pick_rows_per_wave(b.hidden, n_assign);
-        if (b.inter % 4 == 0) MUMMU_DN(1, 4, 1, rpw);
-        else MUMMU_DN(1, 1, 1, rpw);
+        dim3 grid(slots, (b.hidden + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_assign / slots);
+        if (b.inter % 4 == 0)
+            down_f_kernel<WT, 4><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
+        else
+            down_f_kernel<WT, 1><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
     }
-#undef MUMMU_DN
     return hipGetLastError();
 }
 
-hipError_t launch_down(const ExpertBanks &b, const float *act, const int32_t *ids, int n_assign, int fixed_expert,
-                       float *y, hipStream_t s) {
+hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign, int k,
+                       int fixed_expert, float *y, hipStream_t s) {
     if (n_assign <= 0) return hipSuccess;
+    if (n_assign / (fixed_expert >= 0 ? 1 : k) > 65535) return hipErrorInvalidValue;
     switch (b.down_type) {
-    case T_F32: return launch_down_t<T_F32>(b, act, ids, n_assign, fixed_expert, y, s);
-    case T_F16: return launch_down_t<T_F16>(b, act, ids, n_assign, fixed_expert, y, s);
-    case T_BF16: return launch_down_t<T_BF16>(b, act, ids, n_assign, fixed_expert, y, s);
-    case T_Q8_0: return launch_down_t<T_Q8_0>(b, act, ids, n_assign, fixed_expert, y, s);
-    case T_Q4_K: return launch_down_t<T_Q4_K>(b, act, ids, n_assign, fixed_expert, y, s);
+    case T_F32: return launch_down_t<T_F32>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
+    case T_F16: return launch_down_t<T_F16>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
+    case T_BF16: return launch_down_t<T_BF16>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
+    case T_Q8_0: return launch_down_t<T_Q8_0>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
+    case T_Q4_K: return launch_down_t<T_Q4_K>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
     default: return hipErrorInvalidValue;
     }
+}
+
+bool down_combine_supported(const ExpertBanks &b, int k) {
+    return is_quant_type(b.down_type) && k <= 8 && (row_split(b.inter).units + 63) / 64 <= 2;
+}
+
+template <int WT>
+static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n,
+                                        int k, const float *residual, float *out, hipStream_t s) {
+    const RowSplit rs = row_split(b.inter);
+    const int upl = (rs.units + 63) / 64;
+    dim3 block(64 * kDcWaves);
+#define MUMMU_DC(UPL, NIT, KPW)                                                                                    \
+    do {                                                                                                           \
+        const int rpb = (NIT)*rs.rows_per_it;                                                                      \
+        dim3 grid(n, (b.hidden + rpb - 1) / rpb);                                                                  \
+        const size_t lds = sizeof(float) * (size_t)(kDcWaves * (KPW)) * (size_t)(rpb + 1);                         \
+        down_combine_q_kernel<WT, UPL, NIT, KPW><<<grid, block, lds, s>>>(b.down, actq, ids, weights, k, b.hidden, \
+                                                                          b.inter, b.n_experts, residual, out);    \
+    } while (0)
+    if (upl == 1) {
+        if (k <= 4) MUMMU_DC(1, 4, 1);
+        else MUMMU_DC(1, 4, 2);
+    } else {
+        if (k <= 4) MUMMU_DC(2, 2, 1);
+        else MUMMU_DC(2, 2, 2);
+    }
+#undef MUMMU_DC
+    return hipGetLastError();
+}
+
+hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,
+                               const float *residual, float *out, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (!down_combine_supported(b, k)) return hipErrorInvalidValue;
+    return b.down_type == T_Q4_K ? launch_down_combine_t<T_Q4_K>(b, actq, ids, weights, n, k, residual, out, s)
+                                 : launch_down_combine_t<T_Q8_0>(b, actq, ids, weights, n, k, residual, out, s);
 }
 
 // ------------------------------------------------------------------------------------------

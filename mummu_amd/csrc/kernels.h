@@ -1,9 +1,11 @@
 // Host-callable launchers of the MoE kernels.  Each returns hipGetLastError() after the
-// launch; shapes are validated by the caller (moe_api.cpp) before any launch.
+// launch; shapes are validated by the caller (moe_api.hip) before any launch.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include "qact.h"
 
 namespace mummu {
 
@@ -16,16 +18,23 @@ hipError_t launch_dequantize(int type, const uint8_t *bytes, size_t nblocks, flo
 
 // router.hip --------------------------------------------------------------------------
 // logits[t, e] = <x[t, :], W[e, :]> in the fixed 512-partial order.  W row-major [E, H].
+// xq.hi != nullptr: also the 16-bit quantization of x for the integer expert products.
 hipError_t launch_router_logits(const float *x, const void *w, int wtype, float *logits, int n, int hidden,
-                                int n_experts, hipStream_t s);
+                                int n_experts, QAct xq, hipStream_t s);
 // softmax -> top-k -> (re)normalise per token; one wave per token.
 //   ids/weights [n, k] in slot order; hits (nullable) [E] += rows routed; flags see above.
 hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, int flavour, int norm,
                              int32_t *ids, float *weights, unsigned long long *hits, int32_t *flags, hipStream_t s);
-// x * rsqrt(mean(x^2) + eps) * gamma, one workgroup per token.
+// Both of the above in ONE launch (num_experts <= 128), plus (xq.hi != nullptr) the 16-bit
+// quantization of x for the integer expert products.
+bool router_fused_supported(int n_experts);
+hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, int hidden, int n_experts, int k,
+                               int flavour, int norm, float *logits, int32_t *ids, float *weights,
+                               unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s);
+// x [n, D] f32 -> QAct (D % 16 == 0).
+hipError_t launch_quantize_rows(const float *x, int n, int d, QAct q, hipStream_t s);
+// x * rsqrt(mean(x^2) + eps) * gamma, one wave per token.
 hipError_t launch_rmsnorm(const float *x, const float *gamma, float eps, int n, int hidden, float *out, hipStream_t s);
-// dst = a + b (residual add), n elements.
-hipError_t launch_add(const float *a, const float *b, float *dst, size_t n, hipStream_t s);
 
 // experts.hip -------------------------------------------------------------------------
 struct ExpertBanks {
@@ -34,16 +43,24 @@ struct ExpertBanks {
     int hidden, inter, n_experts;
 };
 
+inline bool is_quant_type(int t) { return t == 8 || t == 12; }
+
 // act[a, j] = silu(<gate_e[j,:], x_t>) * <up_e[j,:], x_t>  for assignment a = t*k + s,
 // e = ids[a] (or fixed_expert >= 0 with token = a: the single-expert entry point).
-hipError_t launch_gate_up(const ExpertBanks &b, const float *x, const int32_t *ids, int n_assign, int k,
-                          int fixed_expert, float *act, int32_t *flags, hipStream_t s);
-// y[a, c] = <down_e[c,:], act[a,:]>
-hipError_t launch_down(const ExpertBanks &b, const float *act, const int32_t *ids, int n_assign, int fixed_expert,
-                       float *y, hipStream_t s);
+// Input: xq when the gate/up banks are quantized, else x.  Output: actq when the down bank
+// is quantized, else act (f32).
+hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const int32_t *ids, int n_assign, int k,
+                          int fixed_expert, float *act, QAct actq, int32_t *flags, hipStream_t s);
+// y[a, c] = <down_e[c,:], act[a,:]>   (actq for a quantized down bank, else act)
+hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign, int k,
+                       int fixed_expert, float *y, hipStream_t s);
 // out[t, c] = sum over the token's k slots in ASCENDING EXPERT ID of (w * y), two roundings.
 // residual (nullable): out = residual + that sum.
 hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, int n, int k, int hidden,
                           const float *residual, float *out, hipStream_t s);
+// down + combine in one launch (no y round trip): quantized down bank and top_k <= 8.
+bool down_combine_supported(const ExpertBanks &b, int k);
+hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,
+                               const float *residual, float *out, hipStream_t s);
 
 }  // namespace mummu

@@ -21,8 +21,9 @@ namespace {
 
 thread_local std::string g_error;  // failures of calls that have no handle
 
-enum KernelSlot { K_ROUTER_LOGITS, K_ROUTE_TOPK, K_GATE_UP, K_DOWN, K_COMBINE, K_RMSNORM, K_SLOTS };
-const char *const kSlotNames[K_SLOTS] = {"router_logits", "route_topk", "gate_up", "down", "combine", "rmsnorm"};
+enum KernelSlot { K_ROUTER, K_ROUTER_LOGITS, K_ROUTE_TOPK, K_QUANTIZE, K_GATE_UP, K_DOWN_COMBINE, K_DOWN, K_COMBINE, K_RMSNORM, K_SLOTS };
+const char *const kSlotNames[K_SLOTS] = {"router", "router_logits", "route_topk", "quantize", "gate_up", "down_combine",
+                                         "down", "combine", "rmsnorm"};
 
 struct Layer {
     void *router = nullptr;
@@ -55,6 +56,7 @@ struct mummu_moe {
     float *logits = nullptr, *weights = nullptr, *act = nullptr, *y = nullptr;
     int32_t *ids = nullptr, *flags = nullptr;
     float *xin = nullptr, *xout = nullptr, *h2 = nullptr, *resid[2] = {nullptr, nullptr};
+    QAct xq, actq;               // 16-bit activations: tokens x hidden, pairs x inter
 
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing = false;
@@ -82,11 +84,14 @@ bool router_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16; }
 size_t row_bytes_of(int t, int in_dim) { return (size_t)(in_dim / block_elems(t)) * (size_t)block_bytes(t); }
 
 void free_ws(mummu_moe *h) {
-    void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1]};
+    void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1],
+                    h->xq.hi, h->xq.lo, h->xq.scale, h->xq.sum, h->actq.hi, h->actq.lo, h->actq.scale, h->actq.sum};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     h->logits = h->weights = h->act = h->y = h->xin = h->xout = h->h2 = h->resid[0] = h->resid[1] = nullptr;
     h->ids = nullptr;
+    h->xq = QAct();
+    h->actq = QAct();
     h->ws_tokens = h->ws_assign = 0;
     h->ws_experts = 0;
 }
@@ -113,6 +118,16 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     HIPCHK(h, hipMalloc(&h->h2, sizeof(float) * (size_t)nt * H));
     HIPCHK(h, hipMalloc(&h->resid[0], sizeof(float) * (size_t)nt * H));
     HIPCHK(h, hipMalloc(&h->resid[1], sizeof(float) * (size_t)nt * H));
+    // quantized activations (element counts rounded up to whole 16-element blocks)
+    const size_t xe = (size_t)nt * ((H + 15) / 16 * 16), ae = (size_t)na * ((I + 15) / 16 * 16);
+    HIPCHK(h, hipMalloc(&h->xq.hi, xe));
+    HIPCHK(h, hipMalloc(&h->xq.lo, xe));
+    HIPCHK(h, hipMalloc(&h->xq.scale, sizeof(float) * (xe / 16)));
+    HIPCHK(h, hipMalloc(&h->xq.sum, sizeof(int32_t) * (xe / 16)));
+    HIPCHK(h, hipMalloc(&h->actq.hi, ae));
+    HIPCHK(h, hipMalloc(&h->actq.lo, ae));
+    HIPCHK(h, hipMalloc(&h->actq.scale, sizeof(float) * (ae / 16)));
+    HIPCHK(h, hipMalloc(&h->actq.sum, sizeof(int32_t) * (ae / 16)));
     h->ws_tokens = nt;
     h->ws_assign = na;
     h->ws_experts = n_experts;
@@ -206,14 +221,21 @@ int check_topk(mummu_moe *h, int top_k, int n_experts) {
     return MUMMU_OK;
 }
 
-// experts of an already-made routing: gate/up -> down -> combine
-int run_experts(mummu_moe *h, const Layer &L, const float *x, int64_t n, int k, const float *residual, float *out,
-                hipStream_t s) {
+// experts of an already-made routing: gate/up -> down -> combine.  x_quantized says h->xq
+// already holds the 16-bit form of x (the fused router produced it).
+int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, int64_t n, int k, const float *residual,
+                float *out, hipStream_t s) {
     ExpertBanks b = banks_of(h, L);
     const int na = (int)(n * k);
-    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x, h->ids, na, k, -1, h->act, h->flags, s));
-    LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->ids, na, -1, h->y, s));
-    LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, (int)n, k, b.hidden, residual, out, s));
+    if (is_quant_type(b.gate_type) && !x_quantized)
+        LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x, (int)n, b.hidden, h->xq, s));
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x, h->xq, h->ids, na, k, -1, h->act, h->actq, h->flags, s));
+    if (down_combine_supported(b, k)) {
+        LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, k, residual, out, s));
+    } else {
+        LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->actq, h->ids, na, k, -1, h->y, s));
+        LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, (int)n, k, b.hidden, residual, out, s));
+    }
     return MUMMU_OK;
 }
 
@@ -221,10 +243,21 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
                  hipStream_t s) {
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
-    LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, s));
-    LAUNCH(h, K_ROUTE_TOPK, s,
-           launch_route_topk(h->logits, (int)n, E, k, h->cfg.router_flavour, norm, h->ids, h->weights, L.hits, h->flags, s));
-    return run_experts(h, L, x, n, k, residual, out, s);
+    // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
+    const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0;
+    const QAct xq = want_xq ? h->xq : QAct();
+    if (n > 8 && router_fused_supported(E)) {
+        // many tokens: one workgroup per token tile does logits, routing and quantization
+        LAUNCH(h, K_ROUTER, s,
+               launch_router_fused(x, L.router, L.router_type, (int)n, H, E, k, h->cfg.router_flavour, norm, h->logits,
+                                   h->ids, h->weights, L.hits, h->flags, xq, s));
+    } else {
+        // few tokens: the router rows are spread over as many CUs as there are experts
+        LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s));
+        LAUNCH(h, K_ROUTE_TOPK, s,
+               launch_route_topk(h->logits, (int)n, E, k, h->cfg.router_flavour, norm, h->ids, h->weights, L.hits, h->flags, s));
+    }
+    return run_experts(h, L, x, want_xq, n, k, residual, out, s);
 }
 
 int check_device_call(mummu_moe *h, int64_t n, int k, const void *a, const void *b) {
@@ -426,7 +459,7 @@ int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     hipStream_t s = h->stream;
     HIPCHK(h, hipMemcpyAsync(h->xin, x, sizeof(float) * (size_t)n * H, hipMemcpyHostToDevice, s));
-    LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(h->xin, L.router, L.router_type, h->logits, (int)n, H, E, s));
+    LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(h->xin, L.router, L.router_type, h->logits, (int)n, H, E, QAct(), s));
     LAUNCH(h, K_ROUTE_TOPK, s,
            launch_route_topk(h->logits, (int)n, E, top_k, h->cfg.router_flavour, norm, h->ids, h->weights, nullptr, h->flags, s));
     if (logits) HIPCHK(h, hipMemcpyAsync(logits, h->logits, sizeof(float) * (size_t)n * E, hipMemcpyDeviceToHost, s));
@@ -498,7 +531,7 @@ int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const f
         for (size_t e = 0; e < cur.size(); e++) cur[e] += add[e];
         HIPCHK(h, hipMemcpy(L.hits, cur.data(), sizeof(unsigned long long) * cur.size(), hipMemcpyHostToDevice));
     }
-    if ((rc = run_experts(h, L, h->xin, n, top_k, nullptr, h->xout, s))) return rc;
+    if ((rc = run_experts(h, L, h->xin, false, n, top_k, nullptr, h->xout, s))) return rc;
     if ((rc = check_flags(h, s))) return rc;
     HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
     return MUMMU_OK;
@@ -536,8 +569,9 @@ int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_
     const size_t bytes = sizeof(float) * (size_t)rows * (size_t)hidden;
     HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, s));
     ExpertBanks b = banks_of(h, h->layers[layer]);
-    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, h->xin, nullptr, (int)rows, 1, expert, h->act, h->flags, s));
-    LAUNCH(h, K_DOWN, s, launch_down(b, h->act, nullptr, (int)rows, expert, h->y, s));
+    if (is_quant_type(b.gate_type)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(h->xin, (int)rows, hidden, h->xq, s));
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, h->xin, h->xq, nullptr, (int)rows, 1, expert, h->act, h->actq, h->flags, s));
+    LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->actq, nullptr, (int)rows, 1, expert, h->y, s));
     HIPCHK(h, hipStreamSynchronize(s));
     HIPCHK(h, hipMemcpy(out, h->y, bytes, hipMemcpyDeviceToHost));
     return MUMMU_OK;

@@ -1,0 +1,50 @@
+// 16-bit block-scaled activations for the integer expert products.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_utils.h"
+
+namespace mummu {
+
+// A matrix of activations quantized for the integer expert products: rows x D elements,
+// 16-bit values xq = 256*hi + lo with one f32 scale and one integer sum per 16 elements.
+//   hi, lo : int8  [rows][D]        scale : f32 [rows][D/16]       sum : int32 [rows][D/16]
+struct QAct {
+    int8_t *hi = nullptr;
+    int8_t *lo = nullptr;
+    float *scale = nullptr;
+    int32_t *sum = nullptr;
+};
+
+// Quantize 16 consecutive activations held one per lane in an aligned 16-lane row (an inactive
+// row holds zeros) and store them: the lanes write their hi/lo bytes, the lane of the block's
+// first element the block scale and sum.
+__device__ inline void quantize_store16(float v, bool active, const QAct &q, size_t row, int d, int elem) {
+    float m = fabsf(v);
+    m = fmaxf(m, dpp_move<0xB1>(m));
+    m = fmaxf(m, dpp_move<0x4E>(m));
+    m = fmaxf(m, dpp_move<0x141>(m));
+    m = fmaxf(m, dpp_move<0x140>(m));
+    const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
+    int xq = (int)__builtin_rintf(__fmul_rn(v, inv));
+    xq = xq > 32512 ? 32512 : (xq < -32512 ? -32512 : xq);
+    const int lo = ((xq + 128) & 255) - 128;
+    const int hi = (xq - lo) >> 8;
+    int sum = xq;
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, false);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, false);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xF, 0xF, false);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x140, 0xF, 0xF, false);
+    if (active) {
+        q.hi[row * (size_t)d + elem] = (int8_t)hi;
+        q.lo[row * (size_t)d + elem] = (int8_t)lo;
+        if ((elem & 15) == 0) {
+            q.scale[row * (size_t)(d / 16) + (elem >> 4)] = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
+            q.sum[row * (size_t)(d / 16) + (elem >> 4)] = sum;
+        }
+    }
+}
+
+}  // namespace mummu

@@ -15,6 +15,8 @@
 #include "device_utils.h"
 #include "kernels.h"
 
+MUMMU_TRACE_UNIT(router)
+
 namespace mummu {
 
 constexpr int kRouterTokensPerBlock = 4;
@@ -56,11 +58,23 @@ __device__ inline void load_w8(const void *w, size_t i, float (&o)[8]) {
 template <int WT, bool VEC>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x, const void *__restrict__ w,
                                                             float *__restrict__ logits, int n, int hidden,
-                                                            int n_experts) {
+                                                            int n_experts, QAct xq) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int e = blockIdx.y * (blockDim.x >> 6) + wave;
     const int t0 = blockIdx.x * kRouterTokensPerBlock;
+    // this wave's share of the activation quantization for the integer expert products:
+    // 64-element slices of the tile's rows, dealt round-robin over the tile's waves
+    if (xq.hi != nullptr) {
+        const int nwaves = blockDim.x >> 6;
+        const int slices_per_row = hidden / 64;  // hidden % 64 == 0 is checked by the launcher
+        const int tile_tokens = (n - t0) < kRouterTokensPerBlock ? (n - t0) : kRouterTokensPerBlock;
+        for (int sl = blockIdx.y * nwaves + wave; sl < tile_tokens * slices_per_row; sl += gridDim.y * nwaves) {
+            const int t = t0 + sl / slices_per_row;
+            const int elem = (sl % slices_per_row) * 64 + lane;
+            quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
+        }
+    }
     if (e >= n_experts) return;
     float acc[kRouterTokensPerBlock][8];
 #pragma unroll
@@ -107,8 +121,9 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
 }
 
 hipError_t launch_router_logits(const float *x, const void *w, int wtype, float *logits, int n, int hidden,
-                                int n_experts, hipStream_t s) {
+                                int n_experts, QAct xq, hipStream_t s) {
     if (n <= 0) return hipSuccess;
+    if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
     // few tokens: one wave per workgroup so the expert rows spread over as many CUs as possible
     const int waves = n <= 8 ? 1 : 4;
@@ -116,8 +131,8 @@ hipError_t launch_router_logits(const float *x, const void *w, int wtype, float 
     dim3 grid((n + kRouterTokensPerBlock - 1) / kRouterTokensPerBlock, (n_experts + waves - 1) / waves);
 #define MUMMU_LAUNCH_ROUTER(WT)                                                                          \
     do {                                                                                                 \
-        if (vec) router_logits_kernel<WT, true><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts);  \
-        else router_logits_kernel<WT, false><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts);     \
+        if (vec) router_logits_kernel<WT, true><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts, xq);  \
+        else router_logits_kernel<WT, false><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts, xq);     \
     } while (0)
     switch (wtype) {
     case T_F32: MUMMU_LAUNCH_ROUTER(T_F32); break;
@@ -133,43 +148,49 @@ hipError_t launch_router_logits(const float *x, const void *w, int wtype, float 
 // softmax -> top-k -> renormalise, one wave per token.  Lane l holds experts l, l+64, ...
 // Ties: strictly-greater wins, so the lower expert id keeps a tie and equal slots ascend
 // by id (experts.rs:557-573; the stable descending sort of nn/moe.rs:2143-2144).
+//
+// The sequential sums and the ranking read every expert's value; the wave parks them in LDS
+// and every lane streams them back with broadcast 16-byte reads, which keeps the serial
+// chains to one add (or one compare) per element instead of a cross-lane move per element.
 // ---------------------------------------------------------------------------------------
 constexpr int kTopkWavesPerBlock = 4;
 constexpr int kMaxExperts = 64 * kMaxExpertsPerLane;
 
-__device__ inline float lane_bcast(float v, int src) {
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+__device__ inline void wave_lds_sync() {
+    // LDS traffic of one wave is issued in order; this only stops the compiler from moving
+    // the reads above the writes.
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 }
 
-// JN = experts held per lane (num_experts <= 64 * JN).
+// Per-wave LDS scratch of the router.
 template <int JN>
-__global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
-    const float *__restrict__ logits, int n, int n_experts, int k, int flavour, int norm, int32_t *__restrict__ ids,
-    float *__restrict__ weights, unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
-    __shared__ float s_w[kTopkWavesPerBlock][64 * JN];
-    __shared__ int s_id[kTopkWavesPerBlock][64 * JN];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int t = blockIdx.x * kTopkWavesPerBlock + wave;
-    if (t >= n) return;
-    const float *row = logits + (size_t)t * (size_t)n_experts;
+struct RouteScratch {
+    float p[64 * JN];   // per-expert values, expert order
+    float w[64 * JN];   // selected probabilities, slot order
+    int id[64 * JN];    // selected expert ids, slot order
+};
 
+// One wave routes one token whose logits sit in l[j] (expert lane + 64*j).  JN = experts held
+// per lane (num_experts <= 64 * JN).
+template <int JN>
+__device__ inline void route_token(float (&l)[JN], int t, int n_experts, int k, int flavour, int norm,
+                                   int32_t *__restrict__ ids, float *__restrict__ weights,
+                                   unsigned long long *__restrict__ hits, int32_t *__restrict__ flags,
+                                   RouteScratch<JN> &sc) {
+    const int lane = threadIdx.x & 63;
     float p[JN];
     bool bad = false;
     float mx = -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < JN; j++) {
-        int e = lane + 64 * j;
+        const int e = lane + 64 * j;
         if (e < n_experts) {
-            float l = row[e];
-            p[j] = l;
-            if (!(fabsf(l) <= 3.402823466e38f)) {  // inf or NaN
+            if (!(fabsf(l[j]) <= 3.402823466e38f)) {  // inf or NaN
                 bad = true;
                 atomicMin(&flags[FLAG_NONFINITE_INDEX], t * n_experts + e);
             }
-            mx = fmaxf(mx, l);
-        } else {
-            p[j] = -__builtin_inff();
+            mx = fmaxf(mx, l[j]);
         }
     }
     if (__any(bad)) {
@@ -183,83 +204,140 @@ __global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
         return;
     }
     mx = wave_max(mx);
+    // experts past n_experts hold +0: it leaves a running sum unchanged bit for bit and never
+    // outranks a real expert (not greater; on a tie at 0 its id is higher)
 #pragma unroll
-    for (int j = 0; j < JN; j++) p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(p[j], mx)) : 0.0f;
+    for (int j = 0; j < JN; j++) {
+        p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(l[j], mx)) : 0.0f;
+        sc.p[lane + 64 * j] = p[j];
+    }
+    wave_lds_sync();
 
-    // normaliser: sequential over ascending expert id (every lane computes the same sum).
-    // Experts past n_experts hold p = +0, which leaves the running sum unchanged bit for bit,
-    // so the loops run over all 64*JN slots and unroll without branches.
+    // normaliser: sequential over ascending expert id (every lane computes the same sum)
+    const float4 *bp = (const float4 *)sc.p;
     if (flavour == 0) {
         float total = 0.0f;
 #pragma unroll
-        for (int j = 0; j < JN; j++) {
-#pragma unroll
-            for (int src = 0; src < 64; src++) total = __fadd_rn(total, lane_bcast(p[j], src));
+        for (int c = 0; c < 16 * JN; c++) {
+            const float4 v = bp[c];
+            total = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(total, v.x), v.y), v.z), v.w);
         }
 #pragma unroll
         for (int j = 0; j < JN; j++) p[j] = __fdiv_rn(p[j], total);
     } else {
         double total = 0.0;
 #pragma unroll
-        for (int j = 0; j < JN; j++) {
-#pragma unroll
-            for (int src = 0; src < 64; src++) total = __dadd_rn(total, (double)lane_bcast(p[j], src));
+        for (int c = 0; c < 16 * JN; c++) {
+            const float4 v = bp[c];
+            total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
         }
-        float scale = (float)__ddiv_rn(1.0, total);
+        const float scale = (float)__ddiv_rn(1.0, total);
 #pragma unroll
         for (int j = 0; j < JN; j++) p[j] = __fmul_rn(p[j], scale);
     }
 
-    // rank of each expert under (probability descending, id ascending); rank < k is its slot.
-    // A padding slot (p = 0, id >= n_experts) never outranks a real expert: it is not greater,
-    // and on a tie at 0 its id is higher.
-    int rank[JN];
+    if (k <= 16) {
+        // k rounds of "largest remaining probability, lowest id on a tie": the wave maximum,
+        // then the first lane (and, within a lane, the first expert) that holds it
+        float cand[JN];
 #pragma unroll
-    for (int j = 0; j < JN; j++) rank[j] = 0;
+        for (int j = 0; j < JN; j++) cand[j] = (lane + 64 * j < n_experts) ? p[j] : -1.0f;
+        for (int s = 0; s < k; s++) {
+            float best = cand[0];
 #pragma unroll
-    for (int js = 0; js < JN; js++) {
+            for (int j = 1; j < JN; j++) best = fmaxf(best, cand[j]);
+            best = wave_max(best);
+            // lowest expert id holding `best` (id = lane + 64*j)
+            int my = 0x7FFFFFFF;
 #pragma unroll
-        for (int src = 0; src < 64; src++) {
-            const float q = lane_bcast(p[js], src);
-            const int eq = 64 * js + src;
+            for (int j = JN - 1; j >= 0; j--)
+                if (cand[j] == best) my = lane + 64 * j;
+            int win = my;
+            if (JN == 1) {
+                const unsigned long long m = __ballot(my != 0x7FFFFFFF);
+                win = (int)__builtin_ctzll(m);
+            } else {
+                // minimum id over the wave
+                float f = -(float)win;  // ids < 2^24: exact in f32, negated so that max finds the minimum
+                f = wave_max(f);
+                win = (int)(-f);
+            }
 #pragma unroll
-            for (int j = 0; j < JN; j++) rank[j] += (q > p[j]) || (q == p[j] && eq < lane + 64 * j);
+            for (int j = 0; j < JN; j++)
+                if (lane + 64 * j == win) cand[j] = -1.0f;
+            if (lane == 0) {
+                sc.w[s] = best;
+                sc.id[s] = win;
+            }
+        }
+    } else {
+        // rank of each expert under (probability descending, id ascending); rank < k is its slot
+        wave_lds_sync();
+#pragma unroll
+        for (int j = 0; j < JN; j++) sc.p[lane + 64 * j] = p[j];
+        wave_lds_sync();
+        int rank[JN];
+#pragma unroll
+        for (int j = 0; j < JN; j++) rank[j] = 0;
+#pragma unroll
+        for (int c = 0; c < 16 * JN; c++) {
+            const float4 v = bp[c];
+            const float q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int eq = 4 * c + i;
+#pragma unroll
+                for (int j = 0; j < JN; j++) rank[j] += (q[i] > p[j]) || (q[i] == p[j] && eq < lane + 64 * j);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < JN; j++) {
+            if (lane + 64 * j < n_experts && rank[j] < k) {
+                sc.w[rank[j]] = p[j];
+                sc.id[rank[j]] = lane + 64 * j;
+            }
         }
     }
-#pragma unroll
-    for (int j = 0; j < JN; j++) {
-        if (lane + 64 * j < n_experts && rank[j] < k) {
-            s_w[wave][rank[j]] = p[j];
-            s_id[wave][rank[j]] = lane + 64 * j;
-        }
-    }
-    // the slots written above are read by every lane of this same wave below
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    wave_lds_sync();
 
     float denom = 1.0f;
     if (flavour == 0) {
         if (norm) {
             float d = 0.0f;
-            for (int s = 0; s < k; s++) d = __fadd_rn(d, s_w[wave][s]);
+            for (int s = 0; s < k; s++) d = __fadd_rn(d, sc.w[s]);
             denom = d;
         }
     } else {
         double d = 0.0;
-        for (int s = 0; s < k; s++) d = __dadd_rn(d, (double)s_w[wave][s]);
-        float fs = (float)d;
+        for (int s = 0; s < k; s++) d = __dadd_rn(d, (double)sc.w[s]);
+        const float fs = (float)d;
         const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
         denom = fs > floor_v ? fs : floor_v;
     }
     const bool divide = flavour != 0 || norm;
     for (int s = lane; s < k; s += 64) {
-        float wv = s_w[wave][s];
-        int id = s_id[wave][s];
+        float wv = sc.w[s];
+        const int id = sc.id[s];
         if (divide) wv = __fdiv_rn(wv, denom);
         ids[(size_t)t * k + s] = id;
         weights[(size_t)t * k + s] = wv;
         if (hits) atomicAdd(&hits[id], 1ULL);
     }
+}
+
+template <int JN>
+__global__ __launch_bounds__(64 * kTopkWavesPerBlock) void route_topk_kernel(
+    const float *__restrict__ logits, int n, int n_experts, int k, int flavour, int norm, int32_t *__restrict__ ids,
+    float *__restrict__ weights, unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[kTopkWavesPerBlock];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * kTopkWavesPerBlock + wave;
+    if (t >= n) return;
+    float l[JN];
+#pragma unroll
+    for (int j = 0; j < JN; j++) l[j] = (lane + 64 * j < n_experts) ? logits[(size_t)t * n_experts + lane + 64 * j] : 0.0f;
+    route_token<JN>(l, t, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[wave]);
 }
 
 hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, int flavour, int norm, int32_t *ids,
@@ -275,6 +353,149 @@ hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, i
     else MUMMU_TOPK(8);
 #undef MUMMU_TOPK
     return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------
+// The router in ONE launch: one workgroup of 16 waves per tile of TT tokens computes every
+// logit of the tile (wave w owns experts w, w+16, ...; all of a wave's weight-row loads are in
+// flight before the first is used), parks them in LDS, routes the tile's tokens (one wave
+// each) and quantizes the tile's activations for the integer expert products.  Nothing
+// crosses a workgroup, so there is no fence, ticket or second launch on the decode path.
+// ---------------------------------------------------------------------------------------
+constexpr int kRouterWaves = 16;
+
+template <int WT, bool VEC, int TT, int JN, int EPW>
+__global__ __launch_bounds__(64 * kRouterWaves) void router_block_kernel(
+    const float *__restrict__ x, const void *__restrict__ w, int n, int hidden, int n_experts, int k, int flavour,
+    int norm, float *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ weights,
+    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags, QAct xq) {
+    __shared__ float s_logits[TT][64 * JN];
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[TT];
+    MUMMU_PHASE(0);
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t0 = blockIdx.x * TT;
+    const int tile_tokens = (n - t0) < TT ? (n - t0) : TT;
+
+    // EPW experts per wave: rows e = wave + 16*i
+    float acc[EPW][TT][8];
+#pragma unroll
+    for (int i = 0; i < EPW; i++)
+#pragma unroll
+        for (int t = 0; t < TT; t++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[i][t][j] = 0.0f;
+
+    for (int base = lane * 8; base < hidden; base += 512) {
+        const int cnt = hidden - base < 8 ? hidden - base : 8;
+        float wv[EPW][8];
+#pragma unroll
+        for (int i = 0; i < EPW; i++) {
+            const int e = wave + kRouterWaves * i;
+            const size_t wrow = (size_t)(e < n_experts ? e : 0) * (size_t)hidden;
+            if (VEC) {
+                load_w8<WT>(w, wrow + (size_t)base, wv[i]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) wv[i][j] = j < cnt ? load_w<WT>(w, wrow + (size_t)(base + j)) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            if (t >= tile_tokens) break;
+            const float *xr = x + (size_t)(t0 + t) * (size_t)hidden + base;
+            float xv[8];
+            if (VEC) {
+                float4 a = ((const float4 *)xr)[0], b = ((const float4 *)xr)[1];
+                xv[0] = a.x; xv[1] = a.y; xv[2] = a.z; xv[3] = a.w; xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) xv[j] = j < cnt ? xr[j] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < EPW; i++)
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (VEC || j < cnt) acc[i][t][j] = __builtin_fmaf(xv[j], wv[i][j], acc[i][t][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < EPW; i++) {
+        const int e = wave + kRouterWaves * i;
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const float *a = acc[i][t];
+            float s = __fadd_rn(__fadd_rn(__fadd_rn(a[0], a[4]), __fadd_rn(a[1], a[5])),
+                                __fadd_rn(__fadd_rn(a[2], a[6]), __fadd_rn(a[3], a[7])));
+            s = wave_sum(s);
+            if (lane == 0 && e < n_experts && t < tile_tokens) {
+                s_logits[t][e] = s;
+                logits[(size_t)(t0 + t) * (size_t)n_experts + (size_t)e] = s;
+            }
+        }
+    }
+    MUMMU_PHASE(1);
+    // the tile's activations as 16-bit blocks: 64-element slices dealt over the waves
+    if (xq.hi != nullptr) {
+        const int slices_per_row = hidden / 64;  // hidden % 64 == 0 is checked by the launcher
+        for (int sl = wave; sl < tile_tokens * slices_per_row; sl += kRouterWaves) {
+            const int t = t0 + sl / slices_per_row;
+            const int elem = (sl % slices_per_row) * 64 + lane;
+            quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
+        }
+    }
+    __syncthreads();
+    MUMMU_PHASE(2);
+    if (wave < tile_tokens) {
+        float l[JN];
+#pragma unroll
+        for (int j = 0; j < JN; j++) l[j] = (lane + 64 * j < n_experts) ? s_logits[wave][lane + 64 * j] : 0.0f;
+        route_token<JN>(l, t0 + wave, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[wave]);
+    }
+    MUMMU_PHASE(3);
+}
+
+template <int WT, bool VEC, int TT>
+static hipError_t launch_router_block_t(const float *x, const void *w, int n, int hidden, int n_experts, int k,
+                                        int flavour, int norm, float *logits, int32_t *ids, float *weights,
+                                        unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s) {
+    dim3 block(64 * kRouterWaves), grid((n + TT - 1) / TT);
+#define MUMMU_RB(JN, EPW)                                                                                            \
+    router_block_kernel<WT, VEC, TT, JN, EPW><<<grid, block, 0, s>>>(x, w, n, hidden, n_experts, k, flavour, norm,   \
+                                                                     logits, ids, weights, hits, flags, xq)
+    if (n_experts <= 64) MUMMU_RB(1, 4);
+    else if (n_experts <= 128) MUMMU_RB(2, 8);
+    else return hipErrorInvalidValue;  // wider routers take the two-kernel path
+#undef MUMMU_RB
+    return hipGetLastError();
+}
+
+bool router_fused_supported(int n_experts) { return n_experts <= 128; }
+
+hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, int hidden, int n_experts, int k,
+                               int flavour, int norm, float *logits, int32_t *ids, float *weights,
+                               unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (n_experts > 128 || k > n_experts || k < 1) return hipErrorInvalidValue;
+    if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
+    const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
+    const bool few = n <= 64;  // few tokens: one token per workgroup
+#define MUMMU_RB2(WT)                                                                                                   \
+    do {                                                                                                                \
+        if (few) {                                                                                                      \
+            if (vec) return launch_router_block_t<WT, true, 1>(x, w, n, hidden, n_experts, k, flavour, norm, logits, ids, weights, hits, flags, xq, s); \
+            return launch_router_block_t<WT, false, 1>(x, w, n, hidden, n_experts, k, flavour, norm, logits, ids, weights, hits, flags, xq, s); \
+        }                                                                                                               \
+        if (vec) return launch_router_block_t<WT, true, 4>(x, w, n, hidden, n_experts, k, flavour, norm, logits, ids, weights, hits, flags, xq, s); \
+        return launch_router_block_t<WT, false, 4>(x, w, n, hidden, n_experts, k, flavour, norm, logits, ids, weights, hits, flags, xq, s); \
+    } while (0)
+    switch (wtype) {
+    case T_F32: MUMMU_RB2(T_F32);
+    case T_F16: MUMMU_RB2(T_F16);
+    case T_BF16: MUMMU_RB2(T_BF16);
+    default: return hipErrorInvalidValue;
+    }
+#undef MUMMU_RB2
 }
 
 // ---------------------------------------------------------------------------------------
@@ -308,17 +529,6 @@ hipError_t launch_rmsnorm(const float *x, const float *gamma, float eps, int n, 
     if (n <= 0) return hipSuccess;
     dim3 block(256), grid((n + 3) / 4);
     rmsnorm_kernel<<<grid, block, 0, s>>>(x, gamma, eps, n, hidden, out);
-    return hipGetLastError();
-}
-
-__global__ void add_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst, size_t n) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) dst[i] = __fadd_rn(a[i], b[i]);
-}
-
-hipError_t launch_add(const float *a, const float *b, float *dst, size_t n, hipStream_t s) {
-    if (n == 0) return hipSuccess;
-    add_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(a, b, dst, n);
     return hipGetLastError();
 }
 
