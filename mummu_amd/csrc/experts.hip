@@ -709,9 +709,11 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
 constexpr int kCombineMaxK = 512;
 
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ ids,
-                                                      const float *__restrict__ weights, int k, int hidden,
+                                                      const float *__restrict__ weights,
+                                                      const int32_t *__restrict__ inv, int k, int hidden,
                                                       const float *__restrict__ residual, float *__restrict__ out) {
     __shared__ int s_order[kCombineMaxK];
+    __shared__ int s_row[kCombineMaxK];
     __shared__ float s_w[kCombineMaxK];
     const int t = blockIdx.x;
     for (int s = threadIdx.x; s < k; s += blockDim.x) {
@@ -724,26 +726,30 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         s_order[rank] = s;
     }
     __syncthreads();
-    for (int s = threadIdx.x; s < k; s += blockDim.x) s_w[s] = weights[(size_t)t * k + s_order[s]];
+    for (int s = threadIdx.x; s < k; s += blockDim.x) {
+        const int a = t * k + s_order[s];
+        s_w[s] = weights[a];
+        s_row[s] = inv ? inv[a] : a;
+    }
     __syncthreads();
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < hidden; c += gridDim.y * blockDim.x) {
         float sum = 0.0f;
         for (int r = 0; r < k; r++) {
-            const float v = y[((size_t)t * k + s_order[r]) * (size_t)hidden + c];
+            const float v = y[(size_t)s_row[r] * (size_t)hidden + c];
             sum = __fadd_rn(sum, __fmul_rn(s_w[r], v));
         }
         out[(size_t)t * hidden + c] = residual ? __fadd_rn(residual[(size_t)t * hidden + c], sum) : sum;
     }
 }
 
-hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, int n, int k, int hidden,
-                          const float *residual, float *out, hipStream_t s) {
+hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, const int32_t *inv, int n, int k,
+                          int hidden, const float *residual, float *out, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     if (k > kCombineMaxK) return hipErrorInvalidValue;
     int ysplit = (hidden + 255) / 256;
     if (n >= 64) ysplit = 1;  // plenty of workgroups already
     dim3 block(256), grid(n, ysplit);
-    combine_kernel<<<grid, block, 0, s>>>(y, ids, weights, k, hidden, residual, out);
+    combine_kernel<<<grid, block, 0, s>>>(y, ids, weights, inv, k, hidden, residual, out);
     return hipGetLastError();
 }
 

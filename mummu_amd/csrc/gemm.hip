@@ -1,0 +1,518 @@
+// SwiGLU expert products for batches (prefill): grouped GEMMs over the dispatch-sorted
+// assignments on the matrix cores, one launch per projection for every routed expert of the
+// layer.
+//
+// Reference semantics: per hit expert, y = down(silu(gate.x_e) * (up.x_e)) over the rows routed
+// to it (nn/moe.rs:312-316, models/qwen4exp/experts.rs:1126-1135).
+//
+// Work list: (expert, first sorted position, rows <= 32*MT) tiles from the dispatch kernel;
+// blockIdx.x walks that list (ragged and skewed expert loads just make it longer or shorter),
+// blockIdx.y the output rows in slabs of 128.  A workgroup of 4 waves keeps a [32*MT x 64]
+// activation tile and a [128 x 64] weight tile (two for gate+up) in LDS per K step; wave w owns
+// output columns 32w..32w+31.  Weights are read from HBM once per tile in their GGUF bytes; the
+// next K step's global loads are in flight while the current one is multiplied.
+//
+// Two arithmetic families:
+//   F16 banks        v_mfma_f32_32x32x16_f16 on the stored halfs; activations rounded to f16.
+//   Q8_0/Q4_K banks  v_mfma_i32_32x32x32_i8 on the stored integers (Q4_K nibbles widened to
+//                    bytes) against activations quantized to 16 bits in two byte planes
+//                    (x ~ s*(256*hi + lo), one scale per 64 elements): per 32-element block the
+//                    integer sums are exact, C = 256*C_hi + C_lo, and the f32 accumulator takes
+//                    s * sum_blocks(d_block * C).  Q4_K's offset term -dmin*m*sum(x) is one
+//                    v_mfma_f32_32x32x2_f32 per K step over the per-block activation sums.
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace mummu {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int16v __attribute__((ext_vector_type(16)));
+
+constexpr int kBN = 128;            // output rows per workgroup
+constexpr int kBK = 64;             // K step
+constexpr int kLds = kBK + 8;       // f16 LDS row (halfs): 144 B keeps 16-byte reads conflict-free
+constexpr int kLdsQ = kBK + 16;     // int8 LDS row (bytes): 80 B, likewise
+constexpr int kLdsC = kBN + 4;      // f32 staging row of the gate/up epilogue
+
+__device__ inline uint32_t pack_half2(float a, float b) {
+    _Float16 h[2] = {(_Float16)a, (_Float16)b};
+    uint32_t u;
+    __builtin_memcpy(&u, h, 4);
+    return u;
+}
+
+__host__ __device__ inline size_t gemm_row_bytes(int type, int in_dim) {
+    return (size_t)(in_dim / block_elems(type)) * (size_t)block_bytes(type);
+}
+
+// Epilogue shared by both families: acc register r of lane l is element
+// (row 8*(r/4) + 4*(l/32) + r%4, column l%32) of the wave's 32x32 tile.
+__device__ inline int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// ---------------------------------------------------------------------------------------
+// F16 banks
+// ---------------------------------------------------------------------------------------
+
+// GATE_UP: A = x (f32, gathered by token through `sorted`), two weight matrices, epilogue
+//          act16[pos, n] = f16(silu(g) * u).
+// else   : A = act16 (f16, rows already in sorted order), one matrix, y[pos, n] = f32 sum.
+template <bool GATE_UP, int MT>
+__global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
+    const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const float *__restrict__ x,
+    const _Float16 *__restrict__ act_in, const int32_t *__restrict__ sorted, int k_slots,
+    const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim,
+    _Float16 *__restrict__ act_out, float *__restrict__ y_out) {
+    constexpr int NB = GATE_UP ? 2 : 1;
+    constexpr int BM = 32 * MT;
+    __shared__ __attribute__((aligned(16))) _Float16 s_a[BM][kLds];
+    __shared__ __attribute__((aligned(16))) _Float16 s_b[NB][kBN][kLds];
+
+    const int tile = blockIdx.x;
+    if (tile >= *n_tiles) return;
+    const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int n0 = blockIdx.y * kBN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t row_bytes = (size_t)in_dim * 2;
+
+    // weight tile: thread -> (row, half of the K step)
+    const int b_row = tid >> 1, b_half = tid & 1;
+    const int b_out = n0 + b_row < out_dim ? n0 + b_row : out_dim - 1;  // clamped; never stored
+    const uint8_t *b_ptr[NB];
+    b_ptr[0] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_half * 64;
+    if (GATE_UP) b_ptr[NB - 1] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_half * 64;
+
+    // activation tile: f32 source -> 16 threads per row, 4 elements each (2*MT passes of 16 rows);
+    // f16 source -> 8 threads per row, 8 elements each (MT passes of 32 rows)
+    constexpr int A_PASSES = GATE_UP ? 2 * MT : MT;
+    const int a_col = GATE_UP ? (tid & 15) * 4 : (tid & 7) * 8;
+    const float *a_src32[A_PASSES];
+    const _Float16 *a_src16[A_PASSES];
+    int a_row[A_PASSES];
+#pragma unroll
+    for (int p = 0; p < A_PASSES; p++) {
+        a_row[p] = GATE_UP ? p * 16 + (tid >> 4) : p * 32 + (tid >> 3);
+        const bool ok = a_row[p] < rows;
+        if (GATE_UP) {
+            const int a = ok ? sorted[p0 + a_row[p]] : 0;
+            a_src32[p] = ok ? x + (size_t)(a / k_slots) * (size_t)in_dim + a_col : nullptr;
+            a_src16[p] = nullptr;
+        } else {
+            a_src16[p] = ok ? act_in + (size_t)(p0 + a_row[p]) * (size_t)in_dim + a_col : nullptr;
+            a_src32[p] = nullptr;
+        }
+    }
+
+    float16v acc[NB][MT];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
+
+    uint4 rb[NB][4];
+    float4 ra32[A_PASSES];
+    uint4 ra16[A_PASSES];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint4 *p = (const uint4 *)(b_ptr[b] + (size_t)k0 * 2);
+#pragma unroll
+            for (int i = 0; i < 4; i++) rb[b][i] = p[i];
+        }
+#pragma unroll
+        for (int p = 0; p < A_PASSES; p++) {
+            if (GATE_UP) ra32[p] = a_src32[p] ? *(const float4 *)(a_src32[p] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            else ra16[p] = a_src16[p] ? *(const uint4 *)(a_src16[p] + k0) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    fetch(0);
+
+    for (int k0 = 0; k0 < in_dim; k0 += kBK) {
+        // registers -> LDS
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            uint4 *dst = (uint4 *)&s_b[b][b_row][b_half * 32];
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = rb[b][i];
+        }
+#pragma unroll
+        for (int p = 0; p < A_PASSES; p++) {
+            if (GATE_UP) {
+                uint2 v = make_uint2(pack_half2(ra32[p].x, ra32[p].y), pack_half2(ra32[p].z, ra32[p].w));
+                *(uint2 *)&s_a[a_row[p]][a_col] = v;
+            } else {
+                *(uint4 *)&s_a[a_row[p]][a_col] = ra16[p];
+            }
+        }
+        __syncthreads();
+        if (k0 + kBK < in_dim) fetch(k0 + kBK);
+        // multiply: wave owns columns 32*wave .. +31
+#pragma unroll
+        for (int kk = 0; kk < kBK / 16; kk++) {
+            half8 bfrag[NB];
+#pragma unroll
+            for (int b = 0; b < NB; b++) bfrag[b] = *(const half8 *)&s_b[b][32 * wave + (lane & 31)][kk * 16 + (lane >> 5) * 8];
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const half8 afrag = *(const half8 *)&s_a[32 * m + (lane & 31)][kk * 16 + (lane >> 5) * 8];
+#pragma unroll
+                for (int b = 0; b < NB; b++) acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[b], acc[b][m], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    const int n = n0 + 32 * wave + (lane & 31);
+    if (n < out_dim) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = 32 * m + acc_row(r, lane);
+                if (row < rows) {
+                    const size_t o = (size_t)(p0 + row) * (size_t)out_dim + (size_t)n;
+                    if (GATE_UP) act_out[o] = (_Float16)__fmul_rn(det_silu(acc[0][m][r]), acc[NB - 1][m][r]);
+                    else y_out[o] = acc[0][m][r];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Q8_0 / Q4_K banks
+// ---------------------------------------------------------------------------------------
+
+// Raw bytes of one thread's share of a weight tile: one 32-element block of one row.
+template <int WT>
+struct RawQ;
+template <>
+struct RawQ<T_Q8_0> {
+    uint32_t d;
+    uint32_t q[8];
+};
+template <>
+struct RawQ<T_Q4_K> {
+    uint4 hdr;
+    uint4 q[2];
+};
+
+// rowp: start of the weight row; k0: first element of the K step (multiple of 64); half: which
+// 32-element block of the step.
+template <int WT>
+__device__ inline void load_q(const uint8_t *__restrict__ rowp, int k0, int half, RawQ<WT> &r) {
+    if constexpr (WT == T_Q8_0) {
+        const uint8_t *blk = rowp + (size_t)(k0 / 32 + half) * 34;
+        uint16_t db;
+        __builtin_memcpy(&db, blk, 2);
+        r.d = db;
+#pragma unroll
+        for (int w = 0; w < 8; w++) __builtin_memcpy(&r.q[w], blk + 2 + 4 * w, 4);
+    } else {
+        const uint8_t *blk = rowp + (size_t)(k0 >> 8) * 144;
+        r.hdr = *(const uint4 *)blk;
+        const uint4 *q = (const uint4 *)(blk + 16 + ((k0 & 255) >> 6) * 32);
+        r.q[0] = q[0];
+        r.q[1] = q[1];
+    }
+}
+
+// The block's 32 integers as bytes in element order, its scale, and minus its offset.
+template <int WT>
+__device__ inline void expand_q(const RawQ<WT> &r, int k0, int half, uint32_t (&q)[8], float &scale, float &neg_min) {
+    if constexpr (WT == T_Q8_0) {
+#pragma unroll
+        for (int w = 0; w < 8; w++) q[w] = r.q[w];
+        scale = half_bits_to_float((uint16_t)r.d);
+        neg_min = 0.0f;
+    } else {
+        const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFFu));
+        const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
+        const int j = 2 * ((k0 & 255) >> 6) + half;  // sub-block: low nibbles first, then high
+        uint32_t sc, mn;
+        {
+            const uint32_t s0 = r.hdr.y, s1 = r.hdr.z, s2 = r.hdr.w;
+            auto byte_of = [&](int k) -> uint32_t {
+                const uint32_t w = k < 4 ? s0 : (k < 8 ? s1 : s2);
+                return (w >> (8 * (k & 3))) & 0xFFu;
+            };
+            if (j < 4) {
+                sc = byte_of(j) & 63u;
+                mn = byte_of(j + 4) & 63u;
+            } else {
+                const uint32_t hi = byte_of(j + 4);
+                sc = (hi & 0x0Fu) | ((byte_of(j - 4) >> 6) << 4);
+                mn = (hi >> 4) | ((byte_of(j) >> 6) << 4);
+            }
+        }
+        scale = __fmul_rn(d, (float)sc);
+        neg_min = -__fmul_rn(dmin, (float)mn);
+        const uint32_t qw[8] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w, r.q[1].x, r.q[1].y, r.q[1].z, r.q[1].w};
+#pragma unroll
+        for (int w = 0; w < 8; w++) q[w] = half ? (qw[w] >> 4) & 0x0F0F0F0Fu : qw[w] & 0x0F0F0F0Fu;
+    }
+}
+
+template <bool GATE_UP, int MT>
+struct QTileLds {
+    static constexpr int NB = GATE_UP ? 2 : 1;
+    static constexpr int BM = 32 * MT;
+    static constexpr int kA = 2 * BM * kLdsQ;                 // hi and lo planes
+    static constexpr int kB = NB * kBN * kLdsQ;
+    static constexpr int kC = GATE_UP ? BM * kLdsC * 4 : 0;   // f32 staging of the epilogue (aliases A and B)
+    static constexpr int kBytes = (kA + kB) > kC ? (kA + kB) : kC;
+};
+
+// GATE_UP: A = xq rows gathered by token through `sorted`; epilogue quantizes silu(g)*u into
+//          act_out rows in sorted order.
+// else   : A = act_in rows in sorted order; y[pos, n] = f32 sum.
+template <int WT, bool GATE_UP, int MT>
+__global__ __launch_bounds__(256) void grouped_gemm_q_kernel(
+    const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, QAct64 a_in, const int32_t *__restrict__ sorted,
+    int k_slots, const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim,
+    QAct64 act_out, float *__restrict__ y_out) {
+    using L = QTileLds<GATE_UP, MT>;
+    constexpr int NB = L::NB, BM = L::BM;
+    __shared__ __attribute__((aligned(16))) uint8_t s_raw[L::kBytes];
+    __shared__ __attribute__((aligned(16))) float s_as[BM];       // activation scale of this K step, per tile row
+    __shared__ float s_am[BM][2];                                 // activation ssum of its two blocks
+    __shared__ float s_bd[NB][kBN][2];                            // weight block scales
+    __shared__ float s_bm[NB][kBN][2];                            // minus the weight block offsets (Q4_K)
+    auto s_a = [&](int plane, int row) -> uint8_t * { return s_raw + ((size_t)plane * BM + row) * kLdsQ; };
+    auto s_b = [&](int b, int row) -> uint8_t * { return s_raw + L::kA + ((size_t)b * kBN + row) * kLdsQ; };
+
+    const int tile = blockIdx.x;
+    if (tile >= *n_tiles) return;
+    const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int n0 = blockIdx.y * kBN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t row_bytes = gemm_row_bytes(WT, in_dim);
+
+    // weight tile: thread -> (row, block of the K step)
+    const int b_row = tid >> 1, b_half = tid & 1;
+    const int b_out = n0 + b_row < out_dim ? n0 + b_row : out_dim - 1;  // clamped; never stored
+    const uint8_t *b_ptr[NB];
+    b_ptr[0] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes;
+    if (GATE_UP) b_ptr[NB - 1] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes;
+
+    // source row of tile row r (-1: past the tile's rows)
+    auto source_row = [&](int r) -> int {
+        if (r >= rows) return -1;
+        return GATE_UP ? sorted[p0 + r] / k_slots : p0 + r;
+    };
+    // activation tile: thread -> (plane, row, 16-byte chunk), MT passes of 32 rows
+    const int a_plane = tid >> 7, a_chunk = tid & 3;
+    const int8_t *a_src[MT];
+    int a_row[MT];
+#pragma unroll
+    for (int p = 0; p < MT; p++) {
+        a_row[p] = 32 * p + ((tid >> 2) & 31);
+        const int src = source_row(a_row[p]);
+        a_src[p] = src < 0 ? nullptr : (a_plane ? a_in.lo : a_in.hi) + (size_t)src * (size_t)in_dim + a_chunk * 16;
+    }
+    // its scales: thread t < BM -> scale of row t; thread t < 2*BM -> ssum of (row t/2, block t%2)
+    const int src_s = tid < BM ? source_row(tid) : -1;
+    const int src_m = tid < 2 * BM ? source_row(tid >> 1) : -1;
+    const float *as_ptr = src_s < 0 ? nullptr : a_in.scale + (size_t)src_s * (size_t)(in_dim / 64);
+    const float *am_ptr = src_m < 0 ? nullptr : a_in.ssum + (size_t)src_m * (size_t)(in_dim / 32) + (tid & 1);
+
+    float16v acc[NB][MT];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
+
+    RawQ<WT> rb[NB];
+    uint4 ra[MT];
+    float ras = 0.0f, ram = 0.0f;
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) load_q<WT>(b_ptr[b], k0, b_half, rb[b]);
+#pragma unroll
+        for (int p = 0; p < MT; p++) ra[p] = a_src[p] ? *(const uint4 *)(a_src[p] + k0) : make_uint4(0, 0, 0, 0);
+        ras = as_ptr ? as_ptr[k0 >> 6] : 0.0f;
+        if (WT == T_Q4_K) ram = am_ptr ? am_ptr[k0 >> 5] : 0.0f;
+    };
+    fetch(0);
+
+    const int col = 32 * wave + (lane & 31), g = lane >> 5;
+    for (int k0 = 0; k0 < in_dim; k0 += kBK) {
+        // registers -> LDS
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            uint32_t q[8];
+            float sc, nm;
+            expand_q<WT>(rb[b], k0, b_half, q, sc, nm);
+            uint4 *dst = (uint4 *)(s_b(b, b_row) + b_half * 32);
+            dst[0] = make_uint4(q[0], q[1], q[2], q[3]);
+            dst[1] = make_uint4(q[4], q[5], q[6], q[7]);
+            s_bd[b][b_row][b_half] = sc;
+            if (WT == T_Q4_K) s_bm[b][b_row][b_half] = nm;
+        }
+#pragma unroll
+        for (int p = 0; p < MT; p++) *(uint4 *)(s_a(a_plane, a_row[p]) + a_chunk * 16) = ra[p];
+        if (tid < BM) s_as[tid] = ras;
+        if (WT == T_Q4_K && tid < 2 * BM) s_am[tid >> 1][tid & 1] = ram;
+        __syncthreads();
+        if (k0 + kBK < in_dim) fetch(k0 + kBK);
+
+        // multiply: wave owns columns 32*wave .. +31
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const int4v bq0 = *(const int4v *)(s_b(b, col) + 16 * g);
+            const int4v bq1 = *(const int4v *)(s_b(b, col) + 32 + 16 * g);
+            const float d0 = s_bd[b][col][0], d1 = s_bd[b][col][1];
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const int arow = 32 * m + (lane & 31);
+                const int4v ah0 = *(const int4v *)(s_a(0, arow) + 16 * g), al0 = *(const int4v *)(s_a(1, arow) + 16 * g);
+                const int4v ah1 = *(const int4v *)(s_a(0, arow) + 32 + 16 * g), al1 = *(const int4v *)(s_a(1, arow) + 32 + 16 * g);
+                const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                const int16v ch0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah0, bq0, zero, 0, 0, 0);
+                const int16v cl0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al0, bq0, zero, 0, 0, 0);
+                const int16v ch1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah1, bq1, zero, 0, 0, 0);
+                const int16v cl1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al1, bq1, zero, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
+                    const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int r = 4 * j + i;
+                        const float f0 = (float)((ch0[r] << 8) + cl0[r]);
+                        const float f1 = (float)((ch1[r] << 8) + cl1[r]);
+                        const float t = fmaf(d1, f1, __fmul_rn(d0, f0));
+                        acc[b][m][r] = fmaf(t, sr[i], acc[b][m][r]);
+                    }
+                }
+                if (WT == T_Q4_K)
+                    acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][g], s_bm[b][col][g], acc[b][m], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    if (GATE_UP) {
+        // stage silu(g)*u of the whole tile as f32 (over the A and B tiles, no longer needed),
+        // then quantize it in 64-element blocks
+        float *s_c = (float *)s_raw;
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                s_c[(32 * m + acc_row(r, lane)) * kLdsC + col] = __fmul_rn(det_silu(acc[0][m][r]), acc[NB - 1][m][r]);
+        __syncthreads();
+        const int grp = tid >> 4, l16 = tid & 15;
+#pragma unroll
+        for (int pass = 0; pass < BM / 8; pass++) {
+            const int task = pass * 16 + grp, row = task >> 1, cb = task & 1;
+            const float4 v = *(const float4 *)&s_c[row * kLdsC + cb * 64 + 4 * l16];
+            const bool active = row < rows && n0 + cb * 64 < out_dim;
+            quantize_store64(active ? v : make_float4(0.f, 0.f, 0.f, 0.f), active, act_out, (size_t)(p0 + row), out_dim,
+                             n0 + cb * 64 + 4 * l16);
+        }
+    } else {
+        const int n = n0 + col;
+        if (n < out_dim) {
+#pragma unroll
+            for (int m = 0; m < MT; m++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = 32 * m + acc_row(r, lane);
+                    if (row < rows) y_out[(size_t)(p0 + row) * (size_t)out_dim + (size_t)n] = acc[0][m][r];
+                }
+        }
+    }
+}
+
+// x [n, d] f32 -> QAct64: one 16-lane row per 64-element block.
+__global__ __launch_bounds__(256) void quantize_rows64_kernel(const float *__restrict__ x, int d, QAct64 q) {
+    const int row = blockIdx.y;
+    const int elem0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    const bool active = elem0 < d;
+    const float4 v = active ? *(const float4 *)(x + (size_t)row * (size_t)d + elem0) : make_float4(0.f, 0.f, 0.f, 0.f);
+    quantize_store64(v, active, q, (size_t)row, d, elem0);
+}
+
+hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (d % 64 != 0) return hipErrorInvalidValue;
+    quantize_rows64_kernel<<<dim3((d + 1023) / 1024, n), dim3(256), 0, s>>>(x, d, q);
+    return hipGetLastError();
+}
+
+static bool gemm_q_type(int t) { return t == T_Q8_0 || t == T_Q4_K; }
+
+bool grouped_gemm_quantized(const ExpertBanks &b) {
+    return gemm_q_type(b.gate_type) && b.gate_type == b.up_type && gemm_q_type(b.down_type);
+}
+
+bool grouped_gemm_supported(const ExpertBanks &b) {
+    const bool f16 = b.gate_type == T_F16 && b.up_type == T_F16 && b.down_type == T_F16;
+    return (f16 || grouped_gemm_quantized(b)) && b.hidden % kBK == 0 && b.inter % kBK == 0;
+}
+
+int grouped_gemm_tile_rows(int n_assign, int n_experts) { return n_assign / n_experts > 32 ? 64 : 32; }
+
+template <int WT, bool GATE_UP>
+static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_in, const int32_t *sorted, int k_slots,
+                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
+                                int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
+    dim3 block(256), grid(max_tiles, (out_dim + kBN - 1) / kBN);
+    if (tile_rows == 64)
+        grouped_gemm_q_kernel<WT, GATE_UP, 2><<<grid, block, 0, s>>>(w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
+                                                                     out_dim, act_out, y_out);
+    else
+        grouped_gemm_q_kernel<WT, GATE_UP, 1><<<grid, block, 0, s>>>(w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
+                                                                     out_dim, act_out, y_out);
+    return hipGetLastError();
+}
+
+template <bool GATE_UP>
+static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const float *x, const _Float16 *act_in,
+                                  const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
+                                  int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
+                                  hipStream_t s) {
+    dim3 block(256), grid(max_tiles, (out_dim + kBN - 1) / kBN);
+    if (tile_rows == 64)
+        grouped_gemm_f16_kernel<GATE_UP, 2><<<grid, block, 0, s>>>(w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
+                                                                   out_dim, act_out, y_out);
+    else
+        grouped_gemm_f16_kernel<GATE_UP, 1><<<grid, block, 0, s>>>(w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
+                                                                   out_dim, act_out, y_out);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
+                               const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
+                               QAct64 actq, hipStream_t s) {
+    if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (b.gate_type == T_F16)
+        return launch_gemm_f16<true>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+                                     b.inter, (_Float16 *)act16, nullptr, s);
+    if (b.gate_type == T_Q8_0)
+        return launch_gemm_q<T_Q8_0, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+                                           b.inter, actq, nullptr, s);
+    return launch_gemm_q<T_Q4_K, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+                                       b.inter, actq, nullptr, s);
+}
+
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, const int32_t *tiles,
+                            const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s) {
+    if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (b.down_type == T_F16)
+        return launch_gemm_f16<false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+                                      tile_rows, b.inter, b.hidden, nullptr, y, s);
+    if (b.down_type == T_Q8_0)
+        return launch_gemm_q<T_Q8_0, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter,
+                                            b.hidden, QAct64(), y, s);
+    return launch_gemm_q<T_Q4_K, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter,
+                                        b.hidden, QAct64(), y, s);
+}
+
+}  // namespace mummu

@@ -56,11 +56,37 @@ hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const 
                        int fixed_expert, float *y, hipStream_t s);
 // out[t, c] = sum over the token's k slots in ASCENDING EXPERT ID of (w * y), two roundings.
 // residual (nullable): out = residual + that sum.
-hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, int n, int k, int hidden,
-                          const float *residual, float *out, hipStream_t s);
+// inv (nullable): y row of assignment a is inv[a] instead of a (dispatch-sorted layout).
+hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, const int32_t *inv, int n, int k,
+                          int hidden, const float *residual, float *out, hipStream_t s);
 // down + combine in one launch (no y round trip): quantized down bank and top_k <= 8.
 bool down_combine_supported(const ExpertBanks &b, int k);
 hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,
                                const float *residual, float *out, hipStream_t s);
+
+
+// dispatch.hip ------------------------------------------------------------------------
+// Stable counting sort of the assignments by expert (histogram, scan and cursors in LDS):
+// offsets[E+1], sorted[A] (position -> assignment), inv[A] (assignment -> position) and the
+// grouped GEMM's work list of (expert, first position, rows <= tile_rows) triples.
+hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int tile_rows, int32_t *offsets,
+                           int32_t *sorted, int32_t *inv, int32_t *tiles, int32_t *n_tiles, int32_t *flags,
+                           hipStream_t s);
+
+// gemm.hip ----------------------------------------------------------------------------
+// Grouped GEMMs over the dispatch-sorted assignments on the matrix cores (hidden and inter
+// multiples of 64): F16 banks on the f16 units (act16: f16 [A, inter] in sorted order), Q8_0 /
+// Q4_K banks on the int8 units against 16-bit activations (xq: tokens x hidden, actq: A x inter
+// in sorted order).
+bool grouped_gemm_supported(const ExpertBanks &b);
+bool grouped_gemm_quantized(const ExpertBanks &b);
+int grouped_gemm_tile_rows(int n_assign, int n_experts);
+// x [n, d] f32 -> QAct64 (d % 64 == 0).
+hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s);
+hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
+                               const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
+                               QAct64 actq, hipStream_t s);
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, const int32_t *tiles,
+                            const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s);
 
 }  // namespace mummu

@@ -21,9 +21,10 @@ namespace {
 
 thread_local std::string g_error;  // failures of calls that have no handle
 
-enum KernelSlot { K_ROUTER, K_ROUTER_LOGITS, K_ROUTE_TOPK, K_QUANTIZE, K_GATE_UP, K_DOWN_COMBINE, K_DOWN, K_COMBINE, K_RMSNORM, K_SLOTS };
+enum KernelSlot { K_ROUTER, K_ROUTER_LOGITS, K_ROUTE_TOPK, K_QUANTIZE, K_GATE_UP, K_DOWN_COMBINE, K_DOWN, K_COMBINE, K_RMSNORM,
+                  K_DISPATCH, K_GEMM_GATE_UP, K_GEMM_DOWN, K_SLOTS };
 const char *const kSlotNames[K_SLOTS] = {"router", "router_logits", "route_topk", "quantize", "gate_up", "down_combine",
-                                         "down", "combine", "rmsnorm"};
+                                         "down", "combine", "rmsnorm", "dispatch", "gemm_gate_up", "gemm_down"};
 
 struct Layer {
     void *router = nullptr;
@@ -57,6 +58,11 @@ struct mummu_moe {
     int32_t *ids = nullptr, *flags = nullptr;
     float *xin = nullptr, *xout = nullptr, *h2 = nullptr, *resid[2] = {nullptr, nullptr};
     QAct xq, actq;               // 16-bit activations: tokens x hidden, pairs x inter
+    // dispatch-sorted layout of the batched path
+    int32_t *offsets = nullptr, *sorted = nullptr, *inv = nullptr, *tiles = nullptr, *n_tiles = nullptr;
+    void *act16 = nullptr;       // f16 [pairs, inter]
+    int max_tiles = 0;
+    int gemm_min_tokens = 32;    // batches at least this large take the grouped GEMM
 
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing = false;
@@ -85,13 +91,16 @@ size_t row_bytes_of(int t, int in_dim) { return (size_t)(in_dim / block_elems(t)
 
 void free_ws(mummu_moe *h) {
     void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1],
-                    h->xq.hi, h->xq.lo, h->xq.scale, h->xq.sum, h->actq.hi, h->actq.lo, h->actq.scale, h->actq.sum};
+                    h->xq.hi, h->xq.lo, h->xq.scale, h->xq.sum, h->actq.hi, h->actq.lo, h->actq.scale, h->actq.sum,
+                    h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->act16};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     h->logits = h->weights = h->act = h->y = h->xin = h->xout = h->h2 = h->resid[0] = h->resid[1] = nullptr;
     h->ids = nullptr;
     h->xq = QAct();
     h->actq = QAct();
+    h->offsets = h->sorted = h->inv = h->tiles = h->n_tiles = nullptr;
+    h->act16 = nullptr;
     h->ws_tokens = h->ws_assign = 0;
     h->ws_experts = 0;
 }
@@ -128,6 +137,13 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     HIPCHK(h, hipMalloc(&h->actq.lo, ae));
     HIPCHK(h, hipMalloc(&h->actq.scale, sizeof(float) * (ae / 16)));
     HIPCHK(h, hipMalloc(&h->actq.sum, sizeof(int32_t) * (ae / 16)));
+    h->max_tiles = n_experts + (int)((na + 31) / 32) + 1;
+    HIPCHK(h, hipMalloc(&h->offsets, sizeof(int32_t) * (size_t)(n_experts + 1)));
+    HIPCHK(h, hipMalloc(&h->sorted, sizeof(int32_t) * (size_t)na));
+    HIPCHK(h, hipMalloc(&h->inv, sizeof(int32_t) * (size_t)na));
+    HIPCHK(h, hipMalloc(&h->tiles, sizeof(int32_t) * 3 * (size_t)h->max_tiles));
+    HIPCHK(h, hipMalloc(&h->n_tiles, sizeof(int32_t)));
+    HIPCHK(h, hipMalloc(&h->act16, 2 * (size_t)na * I));
     h->ws_tokens = nt;
     h->ws_assign = na;
     h->ws_experts = n_experts;
@@ -227,6 +243,22 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
                 float *out, hipStream_t s) {
     ExpertBanks b = banks_of(h, L);
     const int na = (int)(n * k);
+    if (n >= h->gemm_min_tokens && grouped_gemm_supported(b)) {
+        // batched: sort the assignments by expert, then one grouped GEMM per projection
+        const int tile_rows = grouped_gemm_tile_rows(na, b.n_experts);
+        // the 16-bit activation buffers, viewed in the batched path's 64-element-block layout
+        const QAct64 xq64{h->xq.hi, h->xq.lo, h->xq.scale, (float *)h->xq.sum};
+        const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
+        if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
+        LAUNCH(h, K_DISPATCH, s,
+               launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->flags, s));
+        LAUNCH(h, K_GEMM_GATE_UP, s,
+               launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, actq64, s));
+        LAUNCH(h, K_GEMM_DOWN, s,
+               launch_gemm_down(b, h->act16, actq64, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
+        LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, h->inv, (int)n, k, b.hidden, residual, out, s));
+        return MUMMU_OK;
+    }
     if (is_quant_type(b.gate_type) && !x_quantized)
         LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x, (int)n, b.hidden, h->xq, s));
     LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x, h->xq, h->ids, na, k, -1, h->act, h->actq, h->flags, s));
@@ -234,7 +266,7 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, k, residual, out, s));
     } else {
         LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->actq, h->ids, na, k, -1, h->y, s));
-        LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, (int)n, k, b.hidden, residual, out, s));
+        LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, nullptr, (int)n, k, b.hidden, residual, out, s));
     }
     return MUMMU_OK;
 }
@@ -244,7 +276,8 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
-    const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0;
+    const bool batched = n >= h->gemm_min_tokens && grouped_gemm_supported(banks_of(h, L));
+    const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0 && !batched;
     const QAct xq = want_xq ? h->xq : QAct();
     if (n > 8 && router_fused_supported(E)) {
         // many tokens: one workgroup per token tile does logits, routing and quantization

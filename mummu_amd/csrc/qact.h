@@ -47,4 +47,50 @@ __device__ inline void quantize_store16(float v, bool active, const QAct &q, siz
     }
 }
 
+// Activations quantized for the batched integer products: the same 16-bit hi/lo planes, with one
+// f32 scale per 64 elements and, per 32 elements, ssum = scale * (sum of the 16-bit values).
+//   hi, lo : int8 [rows][D]       scale : f32 [rows][D/64]       ssum : f32 [rows][D/32]
+struct QAct64 {
+    int8_t *hi = nullptr;
+    int8_t *lo = nullptr;
+    float *scale = nullptr;
+    float *ssum = nullptr;
+};
+
+// Quantize 64 consecutive activations held four per lane in an aligned 16-lane row (lane i holds
+// elements 4i..4i+3; an inactive row holds zeros) and store them.  elem0 is the index of this
+// lane's first element within the matrix row.
+__device__ inline void quantize_store64(float4 v, bool active, const QAct64 &q, size_t row, int d, int elem0) {
+    float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    m = fmaxf(m, dpp_move<0xB1>(m));
+    m = fmaxf(m, dpp_move<0x4E>(m));
+    m = fmaxf(m, dpp_move<0x141>(m));
+    m = fmaxf(m, dpp_move<0x140>(m));
+    const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
+    const float scale = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    uint32_t hi_w = 0, lo_w = 0;
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int xq = (int)__builtin_rintf(__fmul_rn(f[i], inv));
+        xq = xq > 32512 ? 32512 : (xq < -32512 ? -32512 : xq);
+        const int lo = ((xq + 128) & 255) - 128;
+        const int hi = (xq - lo) >> 8;
+        hi_w |= (uint32_t)(hi & 255) << (8 * i);
+        lo_w |= (uint32_t)(lo & 255) << (8 * i);
+        sum += xq;
+    }
+    // 32 elements = 8 lanes
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, false);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, false);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xF, 0xF, false);
+    if (active) {
+        *(uint32_t *)(q.hi + row * (size_t)d + elem0) = hi_w;
+        *(uint32_t *)(q.lo + row * (size_t)d + elem0) = lo_w;
+        if ((elem0 & 31) == 0) q.ssum[row * (size_t)(d / 32) + (elem0 >> 5)] = __fmul_rn(scale, (float)sum);
+        if ((elem0 & 63) == 0) q.scale[row * (size_t)(d / 64) + (elem0 >> 6)] = scale;
+    }
+}
+
 }  // namespace mummu
