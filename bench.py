@@ -34,6 +34,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per gate_up launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
+# same command (profiles/olmoe_q4k_decode_hbm_traffic.txt), each scaled by what the counter
+# reads for the library's 256 MiB copy kernel.  Only for the workload/batch they were taken on.
+PROFILED_GATE_UP_TRAFFIC = {("olmoe_q4k_decode", 1): 19119082}
+
 WORKLOADS = {
     # name: (hidden, inter, experts, top_k, norm, bank type, router type)
     "olmoe_q4k_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q4_K", router="F16"),
@@ -144,6 +149,15 @@ def main() -> int:
             for s in range(nsteps):
                 step(s0 + s)
 
+    # one plain copy of known size on the same stream (untimed): under `rocprofv3 --pmc
+    # FETCH_SIZE` / `WRITE_SIZE` its dispatch calibrates the counters the roofline's `traffic`
+    # figure is scaled by
+    probe_bytes = 256 << 20
+    probe_src, probe_dst = M.DeviceBuffer(probe_bytes), M.DeviceBuffer(probe_bytes)
+    M.probe_copy(probe_dst, probe_src, probe_bytes, moe.stream)
+    M.synchronize()
+    del probe_src, probe_dst
+
     run(args.warmup)
     M.synchronize()
     moe.check()
@@ -199,7 +213,8 @@ def main() -> int:
         "kernel_us": {k_: (round(v, 3) if v is not None else None) for k_, v in per_kernel_us.items()},
         "roofline": {"bound": "hbm", "kernel": "gate_up", "achieved": round(achieved, 1) if achieved else None,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None, "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
+                     "traffic": PROFILED_GATE_UP_TRAFFIC.get((args.workload, n)),
                      "algorithmic_bytes_per_launch": int(gu_bytes), "avg_launch_us": round(gu_us, 3) if gu_us else None},
         "device": M.device_name(),
         "setup_s": round(setup_s, 1),

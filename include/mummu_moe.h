@@ -180,6 +180,11 @@ MUMMU_API void mummu_graph_destroy(void *graph_exec);
 MUMMU_API int mummu_timer_start(mummu_moe *h);
 MUMMU_API int mummu_timer_stop(mummu_moe *h, float *ms);
 
+/* A plain streaming copy kernel (16 bytes per lane, grid-stride) of `bytes` bytes (a multiple
+ * of 16) on the given stream: the known-size dispatch that hardware traffic counters are
+ * calibrated against.  No counterpart in the reference. */
+MUMMU_API int mummu_probe_copy(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
+
 /* Per-kernel timing: when enabled, every kernel launched by the *_device entry points on
  * the handle's stream is bracketed by HIP events.  mummu_moe_kernel_times() synchronises and
  * returns, per kernel slot, the summed milliseconds and the launch count since the last

@@ -66,6 +66,7 @@ SIGNATURES = {
     "mummu_graph_destroy": (None, [_P]),
     "mummu_timer_start": (_I, [_P]),
     "mummu_timer_stop": (_I, [_P, C.POINTER(C.c_float)]),
+    "mummu_probe_copy": (_I, [_P, _P, _SZ, _P]),
     "mummu_moe_kernel_timing": (_I, [_P, _I]),
     "mummu_moe_kernel_times": (_I, [_P, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(C.c_int64), _I]),
 }

@@ -65,11 +65,11 @@ hipError_t launch_dequantize(int type, const uint8_t *bytes, size_t nblocks, flo
     if (n == 0) return hipSuccess;
     dim3 block(256), grid((unsigned)((n + 255) / 256));
     switch (type) {
-    case T_F32: dequantize_kernel<T_F32><<<grid, block, 0, s>>>(bytes, n, out); break;
-    case T_F16: dequantize_kernel<T_F16><<<grid, block, 0, s>>>(bytes, n, out); break;
-    case T_BF16: dequantize_kernel<T_BF16><<<grid, block, 0, s>>>(bytes, n, out); break;
-    case T_Q8_0: dequantize_kernel<T_Q8_0><<<grid, block, 0, s>>>(bytes, n, out); break;
-    case T_Q4_K: dequantize_kernel<T_Q4_K><<<grid, block, 0, s>>>(bytes, n, out); break;
+    case T_F32: launch_kernel(dequantize_kernel<T_F32>, grid, block, 0, s, bytes, n, out); break;
+    case T_F16: launch_kernel(dequantize_kernel<T_F16>, grid, block, 0, s, bytes, n, out); break;
+    case T_BF16: launch_kernel(dequantize_kernel<T_BF16>, grid, block, 0, s, bytes, n, out); break;
+    case T_Q8_0: launch_kernel(dequantize_kernel<T_Q8_0>, grid, block, 0, s, bytes, n, out); break;
+    case T_Q4_K: launch_kernel(dequantize_kernel<T_Q4_K>, grid, block, 0, s, bytes, n, out); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

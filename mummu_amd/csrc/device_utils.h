@@ -5,11 +5,29 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <type_traits>
 
 namespace mummu {
+
+// Every kernel of the library is launched through launch_kernel().  When the calling thread has
+// set g_launch_timing (the per-kernel timing mode of the C ABI), the two events are bound to
+// the dispatch itself and take its start and end timestamps - the duration a kernel trace
+// reports - instead of bracketing it with marker packets; otherwise this is a plain launch.
+struct LaunchTiming {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+extern thread_local LaunchTiming g_launch_timing;
+
+template <typename... KArgs, typename... Args>
+inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                          Args &&...args) {
+    hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds_bytes, stream, g_launch_timing.start, g_launch_timing.stop, 0,
+                          static_cast<KArgs>(args)...);
+}
+
 
 constexpr int kWave = 64;
 

@@ -128,7 +128,7 @@ hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int 
                            hipStream_t s) {
     if (n_assign <= 0) return hipSuccess;
     if (n_experts > kDispatchMaxExperts || tile_rows < 1) return hipErrorInvalidValue;
-    dispatch_kernel<<<dim3(1), dim3(kDispatchThreads), 0, s>>>(ids, n_assign, n_experts, tile_rows, offsets, sorted, inv,
+    launch_kernel(dispatch_kernel, dim3(1), dim3(kDispatchThreads), 0, s, ids, n_assign, n_experts, tile_rows, offsets, sorted, inv,
                                                                tiles, n_tiles, flags);
     return hipGetLastError();
 }

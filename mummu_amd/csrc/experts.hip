@@ -374,7 +374,7 @@ hipError_t launch_quantize_rows(const float *x, int n, int d, QAct q, hipStream_
     if (n <= 0) return hipSuccess;
     if (d % 16) return hipErrorInvalidValue;
     const size_t total = (size_t)n * (size_t)d;
-    quantize_rows_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>(x, n, d, q);
+    launch_kernel(quantize_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, x, n, d, q);
     return hipGetLastError();
 }
 
@@ -574,10 +574,10 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         dim3 grid(slots, (b.inter + rpb - 1) / rpb, n_assign / slots), block(64 * waves);                                      \
         const size_t lds = sizeof(float) * (size_t)rpb;                                                         \
         if (actq_out)                                                                                           \
-            gate_up_q_kernel<WT, UPL, NIT, true><<<grid, block, lds, s>>>(                                      \
+            launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true>, grid, block, lds, s,                                       \
                 b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags);      \
         else                                                                                                    \
-            gate_up_q_kernel<WT, UPL, NIT, false><<<grid, block, lds, s>>>(                                     \
+            launch_kernel(gate_up_q_kernel<WT, UPL, NIT, false>, grid, block, lds, s,                                      \
                 b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags);      \
     } while (0)
         if (upl == 1) MUMMU_GUQ(1, 4);
@@ -590,10 +590,10 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         dim3 block(64 * kGemvWaves), grid(slots, (b.inter + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_assign / slots);
         const bool vec = b.hidden % 4 == 0 && (((uintptr_t)x & 15) == 0);
         if (vec)
-            gate_up_f_kernel<WT, 4><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
+            launch_kernel(gate_up_f_kernel<WT, 4>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
                                                            b.n_experts, rpw, act, flags);
         else
-            gate_up_f_kernel<WT, 1><<<grid, block, 0, s>>>(b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
+            launch_kernel(gate_up_f_kernel<WT, 1>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
                                                            b.n_experts, rpw, act, flags);
         if (actq_out) {  // float gate/up feeding a quantized down bank: quantize the f32 act rows
             hipError_t e = hipGetLastError();
@@ -632,7 +632,7 @@ static hipError_t launch_down_t(const ExpertBanks &b, const float *act, QAct act
     do {                                                                                                       \
         const int rpb = kGemvWaves * (NIT)*rs.rows_per_it;                                                     \
         dim3 grid(slots, (b.hidden + rpb - 1) / rpb, n_assign / slots);                                        \
-        down_q_kernel<WT, UPL, NIT><<<grid, block, 0, s>>>(b.down, actq, ids, fixed_expert, b.hidden, b.inter, \
+        launch_kernel(down_q_kernel<WT, UPL, NIT>, grid, block, 0, s, b.down, actq, ids, fixed_expert, b.hidden, b.inter, \
                                                            b.n_experts, y);                                    \
     } while (0)
         if (upl == 1) MUMMU_DNQ(1, 4);
@@ -644,9 +644,9 @@ static hipError_t launch_down_t(const ExpertBanks &b, const float *act, QAct act
         const int rpw = pick_rows_per_wave(b.hidden, n_assign);
         dim3 grid(slots, (b.hidden + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_assign / slots);
         if (b.inter % 4 == 0)
-            down_f_kernel<WT, 4><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
+            launch_kernel(down_f_kernel<WT, 4>, grid, block, 0, s, b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
         else
-            down_f_kernel<WT, 1><<<grid, block, 0, s>>>(b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
+            launch_kernel(down_f_kernel<WT, 1>, grid, block, 0, s, b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
     }
     return hipGetLastError();
 }
@@ -680,7 +680,7 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
         const int rpb = (NIT)*rs.rows_per_it;                                                                      \
         dim3 grid(n, (b.hidden + rpb - 1) / rpb);                                                                  \
         const size_t lds = sizeof(float) * (size_t)(kDcWaves * (KPW)) * (size_t)(rpb + 1);                         \
-        down_combine_q_kernel<WT, UPL, NIT, KPW><<<grid, block, lds, s>>>(b.down, actq, ids, weights, k, b.hidden, \
+        launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW>, grid, block, lds, s, b.down, actq, ids, weights, k, b.hidden, \
                                                                           b.inter, b.n_experts, residual, out);    \
     } while (0)
     if (upl == 1) {
@@ -749,7 +749,7 @@ hipError_t launch_combine(const float *y, const int32_t *ids, const float *weigh
     int ysplit = (hidden + 255) / 256;
     if (n >= 64) ysplit = 1;  // plenty of workgroups already
     dim3 block(256), grid(n, ysplit);
-    combine_kernel<<<grid, block, 0, s>>>(y, ids, weights, inv, k, hidden, residual, out);
+    launch_kernel(combine_kernel, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out);
     return hipGetLastError();
 }
 

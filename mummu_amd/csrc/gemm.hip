@@ -442,7 +442,7 @@ __global__ __launch_bounds__(256) void quantize_rows64_kernel(const float *__res
 hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     if (d % 64 != 0) return hipErrorInvalidValue;
-    quantize_rows64_kernel<<<dim3((d + 1023) / 1024, n), dim3(256), 0, s>>>(x, d, q);
+    launch_kernel(quantize_rows64_kernel, dim3((d + 1023) / 1024, n), dim3(256), 0, s, x, d, q);
     return hipGetLastError();
 }
 
@@ -465,10 +465,10 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
                                 int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
     dim3 block(256), grid(max_tiles, (out_dim + kBN - 1) / kBN);
     if (tile_rows == 64)
-        grouped_gemm_q_kernel<WT, GATE_UP, 2><<<grid, block, 0, s>>>(w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
+        launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, 2>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                      out_dim, act_out, y_out);
     else
-        grouped_gemm_q_kernel<WT, GATE_UP, 1><<<grid, block, 0, s>>>(w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
+        launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, 1>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                      out_dim, act_out, y_out);
     return hipGetLastError();
 }
@@ -480,10 +480,10 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const fl
                                   hipStream_t s) {
     dim3 block(256), grid(max_tiles, (out_dim + kBN - 1) / kBN);
     if (tile_rows == 64)
-        grouped_gemm_f16_kernel<GATE_UP, 2><<<grid, block, 0, s>>>(w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
+        launch_kernel(grouped_gemm_f16_kernel<GATE_UP, 2>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                    out_dim, act_out, y_out);
     else
-        grouped_gemm_f16_kernel<GATE_UP, 1><<<grid, block, 0, s>>>(w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
+        launch_kernel(grouped_gemm_f16_kernel<GATE_UP, 1>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                    out_dim, act_out, y_out);
     return hipGetLastError();
 }

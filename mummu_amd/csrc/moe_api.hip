@@ -44,6 +44,10 @@ struct TimedLaunch {
 
 }  // namespace
 
+namespace mummu {
+thread_local LaunchTiming g_launch_timing;
+}
+
 struct mummu_moe {
     mummu_moe_config cfg{};
     std::vector<Layer> layers;
@@ -174,11 +178,11 @@ int check_flags(mummu_moe *h, hipStream_t s) {
     return fail(h, MUMMU_ERR_RANGE, "a routed expert id is out of range");
 }
 
+// Per-kernel timing: binds a pair of pooled events to the one kernel the enclosed launcher
+// dispatches (see launch_kernel).
 struct ScopedTimer {
-    mummu_moe *h;
-    hipStream_t s;
-    hipEvent_t stop = nullptr;
-    ScopedTimer(mummu_moe *h_, hipStream_t s_, int slot) : h(h_), s(s_) {
+    bool armed = false;
+    ScopedTimer(mummu_moe *h, hipStream_t, int slot) {
         if (!h->timing) return;
         hipEvent_t ev[2];
         for (auto &e : ev) {
@@ -189,12 +193,13 @@ struct ScopedTimer {
                 return;
             }
         }
-        (void)hipEventRecord(ev[0], s);
-        stop = ev[1];
+        g_launch_timing.start = ev[0];
+        g_launch_timing.stop = ev[1];
+        armed = true;
         h->timed.push_back({ev[0], ev[1], slot});
     }
     ~ScopedTimer() {
-        if (stop) (void)hipEventRecord(stop, s);
+        if (armed) g_launch_timing = LaunchTiming();
     }
 };
 
@@ -803,6 +808,26 @@ int mummu_timer_stop(mummu_moe *h, float *ms) {
     HIPCHK(h, hipEventRecord(h->t1, h->stream));
     HIPCHK(h, hipEventSynchronize(h->t1));
     HIPCHK(h, hipEventElapsedTime(ms, h->t0, h->t1));
+    return MUMMU_OK;
+}
+
+namespace {
+__global__ __launch_bounds__(256) void probe_copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+}  // namespace
+
+int mummu_probe_copy(void *dst_dev, const void *src_dev, size_t bytes, void *stream) {
+    if (!dst_dev || !src_dev || (bytes & 15) || ((uintptr_t)dst_dev & 15) || ((uintptr_t)src_dev & 15))
+        return fail(nullptr, MUMMU_ERR_ARG, "probe_copy: null, unaligned or ragged buffers");
+    if (bytes == 0) return MUMMU_OK;
+    const size_t n16 = bytes / 16;
+    const size_t want = (n16 + 255) / 256;
+    const unsigned grid = (unsigned)(want < 8192 ? want : 8192);
+    launch_kernel(probe_copy_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (uint4 *)dst_dev, (const uint4 *)src_dev, n16);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(nullptr, MUMMU_ERR_DEVICE, std::string("probe_copy: ") + hipGetErrorString(e));
     return MUMMU_OK;
 }
 

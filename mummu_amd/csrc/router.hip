@@ -131,8 +131,8 @@ hipError_t launch_router_logits(const float *x, const void *w, int wtype, float 
     dim3 grid((n + kRouterTokensPerBlock - 1) / kRouterTokensPerBlock, (n_experts + waves - 1) / waves);
 #define MUMMU_LAUNCH_ROUTER(WT)                                                                          \
     do {                                                                                                 \
-        if (vec) router_logits_kernel<WT, true><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts, xq);  \
-        else router_logits_kernel<WT, false><<<grid, block, 0, s>>>(x, w, logits, n, hidden, n_experts, xq);     \
+        if (vec) launch_kernel(router_logits_kernel<WT, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq);  \
+        else launch_kernel(router_logits_kernel<WT, false>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq);     \
     } while (0)
     switch (wtype) {
     case T_F32: MUMMU_LAUNCH_ROUTER(T_F32); break;
@@ -346,7 +346,7 @@ hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, i
     if (n_experts > kMaxExperts || k > n_experts || k < 1) return hipErrorInvalidValue;
     dim3 block(64 * kTopkWavesPerBlock), grid((n + kTopkWavesPerBlock - 1) / kTopkWavesPerBlock);
 #define MUMMU_TOPK(JN) \
-    route_topk_kernel<JN><<<grid, block, 0, s>>>(logits, n, n_experts, k, flavour, norm, ids, weights, hits, flags)
+    launch_kernel(route_topk_kernel<JN>, grid, block, 0, s, logits, n, n_experts, k, flavour, norm, ids, weights, hits, flags)
     if (n_experts <= 64) MUMMU_TOPK(1);
     else if (n_experts <= 128) MUMMU_TOPK(2);
     else if (n_experts <= 256) MUMMU_TOPK(4);
@@ -461,7 +461,7 @@ static hipError_t launch_router_block_t(const float *x, const void *w, int n, in
                                         unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s) {
     dim3 block(64 * kRouterWaves), grid((n + TT - 1) / TT);
 #define MUMMU_RB(JN, EPW)                                                                                            \
-    router_block_kernel<WT, VEC, TT, JN, EPW><<<grid, block, 0, s>>>(x, w, n, hidden, n_experts, k, flavour, norm,   \
+    launch_kernel(router_block_kernel<WT, VEC, TT, JN, EPW>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm,   \
                                                                      logits, ids, weights, hits, flags, xq)
     if (n_experts <= 64) MUMMU_RB(1, 4);
     else if (n_experts <= 128) MUMMU_RB(2, 8);
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ 
 hipError_t launch_rmsnorm(const float *x, const float *gamma, float eps, int n, int hidden, float *out, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     dim3 block(256), grid((n + 3) / 4);
-    rmsnorm_kernel<<<grid, block, 0, s>>>(x, gamma, eps, n, hidden, out);
+    launch_kernel(rmsnorm_kernel, grid, block, 0, s, x, gamma, eps, n, hidden, out);
     return hipGetLastError();
 }
 

@@ -310,6 +310,15 @@ class Graph:
             pass
 
 
+def probe_copy(dst: "DeviceBuffer", src: "DeviceBuffer", nbytes: int, stream=None):
+    """Launch the library's plain copy kernel over nbytes (the known-size dispatch that HBM
+    traffic counters are calibrated against)."""
+    lib = _lib.load()
+    rc = lib.mummu_probe_copy(dst.ptr, src.ptr, nbytes, stream)
+    if rc:
+        raise MoeError(rc, lib.mummu_moe_last_error(None).decode())
+
+
 class DeviceBuffer:
     """A plain HIP allocation (hipMalloc) addressed through the library."""
 
