@@ -1,0 +1,275 @@
+// mummu_moe.hpp - C++ host side above the C ABI of mummu_moe.h.
+//
+// Mirrors the reference's module interface for the sparse MoE block (physics515/Mummu, paths
+// under crates/mummu/src/): the same type and method names, argument meaning and error
+// behaviour, so that a caller written against the Rust API reads the same here.
+//
+//   reference                                         here
+//   SparseMoeConfig            nn/moe.rs:42-50        mummu::SparseMoeConfig
+//   SparseMoe::forward         nn/moe.rs:116          mummu::SparseMoe::forward
+//   SparseMoePerExpert::route  nn/moe.rs:247-290      mummu::SparseMoe::route -> mummu::Routing
+//   SparseMoePerExpert::run_local nn/moe.rs:296-328   mummu::SparseMoe::run_local
+//   Routing                    nn/moe.rs:333-337      mummu::Routing (per_expert rows + weights)
+//   ExpertExec                 nn/moe.rs:348-419      mummu::ExpertExec, mummu::HipExpert
+//   RoutedExperts::routed_moe / apply_routing / expert_ffn
+//                              models/qwen4exp/experts.rs:1015-1150
+//                                                      mummu::RoutedExperts
+//   route                      experts.rs:541-582     mummu::route
+//   gguf::dequantize           gguf.rs:1403-1463      mummu::dequantize
+//
+// Error behaviour: the reference panics on contract violations of SparseMoe (assert!) and
+// returns Err(String) from the qwen4exp functions.  Both surface here as mummu::MoeError (a
+// std::runtime_error carrying the status code and the library's message); nothing is swallowed.
+// Header-only; link with -lmummu_moe.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "mummu_moe.h"
+
+namespace mummu {
+
+class MoeError : public std::runtime_error {
+  public:
+    MoeError(int status, const std::string &msg) : std::runtime_error(msg), status_(status) {}
+    int status() const { return status_; }
+
+  private:
+    int status_;
+};
+
+// SparseMoeConfig (nn/moe.rs:42-50) plus the OlmoeConfig fields the block reads
+// (models/olmoe.rs:52-66).
+struct SparseMoeConfig {
+    int hidden_size = 0;
+    int expert_intermediate_size = 0;
+    int num_experts = 0;
+    int num_experts_per_tok = 0;
+    bool norm_topk_prob = false;
+    int router_flavour = MUMMU_ROUTER_SPARSE_MOE;
+    int num_layers = 1;
+    int max_tokens = 512;
+    float rms_norm_eps = 1e-5f;
+};
+
+// One GGUF tensor payload: host bytes in GGUF order plus its ggml type id.
+struct TensorBytes {
+    const void *data = nullptr;
+    int ggml_type = MUMMU_F32;
+};
+
+// Routing (nn/moe.rs:333-337): per expert, the token rows it serves (ascending, token-major
+// slot-minor fill) and the matching combine weights; plus the slot-ordered form.
+struct Routing {
+    int64_t tokens = 0;
+    int top_k = 0;
+    std::vector<int32_t> ids;      // [tokens, top_k], descending probability
+    std::vector<float> weights;    // [tokens, top_k]
+    std::vector<std::pair<std::vector<int32_t>, std::vector<float>>> per_expert;
+
+    static Routing from_slots(std::vector<int32_t> ids, std::vector<float> weights, int64_t tokens, int top_k,
+                              int num_experts) {
+        Routing r;
+        r.tokens = tokens;
+        r.top_k = top_k;
+        r.per_expert.resize((size_t)num_experts);
+        for (int64_t t = 0; t < tokens; t++)
+            for (int s = 0; s < top_k; s++) {
+                const int32_t e = ids[(size_t)(t * top_k + s)];
+                if (e < 0 || e >= num_experts) throw MoeError(MUMMU_ERR_RANGE, "routing names expert " + std::to_string(e));
+                r.per_expert[(size_t)e].first.push_back((int32_t)t);
+                r.per_expert[(size_t)e].second.push_back(weights[(size_t)(t * top_k + s)]);
+            }
+        r.ids = std::move(ids);
+        r.weights = std::move(weights);
+        return r;
+    }
+};
+
+// The block, resident on the MI355X.  One object holds every MoE layer of a model.
+class SparseMoe {
+  public:
+    explicit SparseMoe(const SparseMoeConfig &c) : cfg_(c) {
+        mummu_moe_config k{};
+        k.hidden_size = c.hidden_size;
+        k.expert_intermediate_size = c.expert_intermediate_size;
+        k.num_experts = c.num_experts;
+        k.num_experts_per_tok = c.num_experts_per_tok;
+        k.norm_topk_prob = c.norm_topk_prob ? 1 : 0;
+        k.router_flavour = c.router_flavour;
+        k.num_layers = c.num_layers;
+        k.max_tokens = c.max_tokens;
+        k.rms_norm_eps = c.rms_norm_eps;
+        mummu_moe *h = nullptr;
+        const int rc = mummu_moe_create(&k, &h);
+        if (rc != MUMMU_OK) throw MoeError(rc, mummu_moe_last_error(nullptr));
+        h_.reset(h, mummu_moe_destroy);
+    }
+
+    const SparseMoeConfig &config() const { return cfg_; }
+    mummu_moe *handle() const { return h_.get(); }
+
+    // The checked load of one block (models/olmoe.rs:338-345).
+    void load_layer(int layer, TensorBytes router, TensorBytes gate, TensorBytes up, TensorBytes down,
+                    const float *rms_gamma = nullptr) {
+        check(mummu_moe_load_layer(h_.get(), layer, router.data, router.ggml_type, gate.data, gate.ggml_type, up.data,
+                                   up.ggml_type, down.data, down.ggml_type, rms_gamma));
+    }
+
+    uint64_t resident_bytes() const { return mummu_moe_resident_bytes(h_.get()); }
+
+    // SparseMoe::forward (nn/moe.rs:116): x [tokens, hidden] -> [tokens, hidden].
+    std::vector<float> forward(const std::vector<float> &x, int top_k, bool norm_topk_prob, int layer = 0) {
+        const int64_t n = rows_of(x);
+        std::vector<float> out(x.size());
+        check(mummu_moe_forward(h_.get(), layer, x.data(), n, top_k, norm_topk_prob ? 1 : 0, out.data()));
+        return out;
+    }
+
+    // SparseMoePerExpert::route (nn/moe.rs:247-290).
+    Routing route(const std::vector<float> &x, int top_k, bool norm_topk_prob, int layer = 0) {
+        const int64_t n = rows_of(x);
+        std::vector<int32_t> ids((size_t)(n * top_k));
+        std::vector<float> w((size_t)(n * top_k));
+        check(mummu_moe_route(h_.get(), layer, x.data(), n, top_k, norm_topk_prob ? 1 : 0, ids.data(), w.data(), nullptr));
+        return Routing::from_slots(std::move(ids), std::move(w), n, top_k, cfg_.num_experts);
+    }
+
+    // SparseMoePerExpert::run_local (nn/moe.rs:296-328) / ExpertPool::run_layer (:1545-1607).
+    std::vector<float> run_local(const std::vector<float> &x, const Routing &routing, int layer = 0) {
+        const int64_t n = rows_of(x);
+        if (n != routing.tokens) throw MoeError(MUMMU_ERR_SHAPE, "routing was made for a different token count");
+        std::vector<float> out(x.size());
+        check(mummu_moe_apply_routing(h_.get(), layer, routing.ids.data(), routing.weights.data(), x.data(), n, routing.top_k,
+                                      out.data()));
+        return out;
+    }
+
+    // ExpertPool::take_hits (nn/moe.rs:857-874).
+    std::vector<uint64_t> take_hits(int layer = 0) {
+        std::vector<uint64_t> hits((size_t)cfg_.num_experts);
+        check(mummu_moe_take_hits(h_.get(), layer, hits.data()));
+        return hits;
+    }
+
+    // x <- x + MoE_l(RmsNorm_l(x)) over every layer (models/olmoe.rs:566-572).
+    std::vector<float> stack_forward(const std::vector<float> &x, int top_k, bool norm_topk_prob) {
+        const int64_t n = rows_of(x);
+        std::vector<float> out(x.size());
+        check(mummu_moe_stack_forward(h_.get(), x.data(), n, top_k, norm_topk_prob ? 1 : 0, out.data(), nullptr));
+        return out;
+    }
+
+    // gguf::dequantize of one resident expert matrix (which: 0 gate, 1 up, 2 down).
+    std::vector<float> dequantize_expert(int layer, int which, int expert) {
+        const size_t n = (size_t)cfg_.hidden_size * (size_t)cfg_.expert_intermediate_size;
+        std::vector<float> out(n);
+        check(mummu_moe_dequantize_expert(h_.get(), layer, which, expert, out.data()));
+        return out;
+    }
+
+    void check(int rc) const {
+        if (rc != MUMMU_OK) throw MoeError(rc, mummu_moe_last_error(h_.get()));
+    }
+
+  private:
+    int64_t rows_of(const std::vector<float> &x) const {
+        if (cfg_.hidden_size <= 0 || x.size() % (size_t)cfg_.hidden_size != 0)
+            throw MoeError(MUMMU_ERR_SHAPE, "input length is not a whole number of hidden-size rows");
+        return (int64_t)(x.size() / (size_t)cfg_.hidden_size);
+    }
+
+    SparseMoeConfig cfg_;
+    std::shared_ptr<mummu_moe> h_;
+};
+
+// SparseMoePerExpert (nn/moe.rs:202-329) has the same forward / route / run_local surface; on
+// this device both are the routed kernels.
+using SparseMoePerExpert = SparseMoe;
+
+// ExpertExec (nn/moe.rs:348-419), the host-slice seam: SwiGLU of one expert on rows x hidden f32.
+class ExpertExec {
+  public:
+    virtual ~ExpertExec() = default;
+    virtual std::vector<float> run(const float *x, size_t rows, size_t hidden) const = 0;
+    virtual uint64_t resident_bytes() const = 0;
+    virtual bool is_staged() const { return true; }  // pinned executors are always resident
+};
+
+// One expert of one layer of a SparseMoe, as an ExpertExec.
+class HipExpert final : public ExpertExec {
+  public:
+    HipExpert(SparseMoe moe, int layer, int expert) : moe_(std::move(moe)), layer_(layer), expert_(expert) {}
+    std::vector<float> run(const float *x, size_t rows, size_t hidden) const override {
+        std::vector<float> out(rows * hidden);
+        moe_.check(mummu_expert_run(moe_.handle(), layer_, expert_, x, (int64_t)rows, (int)hidden, out.data()));
+        return out;
+    }
+    uint64_t resident_bytes() const override {
+        const int e = moe_.config().num_experts * moe_.config().num_layers;
+        return e > 0 ? moe_.resident_bytes() / (uint64_t)e : 0;
+    }
+
+  private:
+    SparseMoe moe_;
+    int layer_, expert_;
+};
+
+// RoutedExperts (models/qwen4exp/experts.rs:1066-1150): caller-supplied router logits, qwen4exp
+// routing rules (f64 normaliser, 2^-14 floor, non-finite logits refused).
+class RoutedExperts {
+  public:
+    explicit RoutedExperts(SparseMoe moe) : moe_(std::move(moe)) {}
+
+    std::vector<float> routed_moe(int layer, const std::vector<float> &router_logits, const std::vector<float> &xs, size_t n,
+                                  int top_k) {
+        std::vector<float> out(xs.size());
+        moe_.check(mummu_moe_routed(moe_.handle(), layer, router_logits.data(), xs.data(), (int64_t)n, top_k, out.data()));
+        return out;
+    }
+
+    std::vector<float> apply_routing(int layer, const std::vector<int32_t> &ids, const std::vector<float> &weights,
+                                     const std::vector<float> &xs, size_t n, int top_k) {
+        std::vector<float> out(xs.size());
+        moe_.check(mummu_moe_apply_routing(moe_.handle(), layer, ids.data(), weights.data(), xs.data(), (int64_t)n, top_k,
+                                           out.data()));
+        return out;
+    }
+
+    std::vector<float> expert_ffn(int layer, int expert, const std::vector<float> &xs, size_t n) {
+        std::vector<float> out(xs.size());
+        moe_.check(mummu_expert_run(moe_.handle(), layer, expert, xs.data(), (int64_t)n, moe_.config().hidden_size, out.data()));
+        return out;
+    }
+
+  private:
+    SparseMoe moe_;
+};
+
+// `route` (experts.rs:541-582) on caller-supplied logits: (ids, weights), each [n, top_k].  The
+// SparseMoe only lends its device workspace; no weights are involved and n_experts is free.
+inline std::pair<std::vector<int32_t>, std::vector<float>> route(const SparseMoe &moe, const std::vector<float> &logits,
+                                                                  size_t n, int n_experts, int top_k,
+                                                                  int flavour = MUMMU_ROUTER_QWEN4EXP,
+                                                                  bool norm_topk_prob = true) {
+    std::vector<int32_t> ids(n * (size_t)top_k);
+    std::vector<float> w(n * (size_t)top_k);
+    moe.check(mummu_route_logits(moe.handle(), logits.data(), (int64_t)n, n_experts, top_k, flavour, norm_topk_prob ? 1 : 0,
+                                 ids.data(), w.data()));
+    return {std::move(ids), std::move(w)};
+}
+
+// gguf::dequantize (gguf.rs:1403-1463): payload bytes -> f32, bit-exact.
+inline std::vector<float> dequantize(int ggml_type, const void *bytes, size_t nbytes, size_t n_elements) {
+    std::vector<float> out(n_elements);
+    const int rc = mummu_dequantize(ggml_type, bytes, nbytes, out.data());
+    if (rc != MUMMU_OK) throw MoeError(rc, mummu_moe_last_error(nullptr));
+    return out;
+}
+
+}  // namespace mummu

@@ -48,7 +48,25 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
+    build_host_mirror_test(verbose)
     return LIB
+
+
+ROOT = os.path.dirname(HERE)
+HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "host_mirror_test.cpp")
+HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "host_mirror_test")
+
+
+def build_host_mirror_test(verbose: bool = False) -> str:
+    """The C++ host mirror (include/mummu_moe.hpp) and its test program: plain g++ over the C ABI."""
+    cmd = [os.environ.get("CXX", "g++"), "-O1", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "include"), HOST_TEST_SRC,
+           "-o", HOST_TEST_BIN, "-L", os.path.dirname(LIB), "-lmummu_moe", "-Wl,-rpath,$ORIGIN/../../mummu_amd/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"g++ failed on the host mirror test:\n{r.stderr}")
+    if verbose:
+        print(f"built {HOST_TEST_BIN}")
+    return HOST_TEST_BIN
 
 
 if __name__ == "__main__":

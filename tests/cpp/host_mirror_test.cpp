@@ -1,0 +1,215 @@
+// Exercises the C++ host mirror (include/mummu_moe.hpp) the way the reference's own unit tests
+// exercise the Rust API, on the reference's closed-form toy block (nn/moe.rs:1617-1651):
+//   forward_matches_the_hand_rolled_sparse_reference   nn/moe.rs:2177-2202
+//   routed == fused forward, hits == tokens * top_k    nn/moe.rs:1655-1700, 1976-1979
+//   zero input -> zero output                          nn/moe.rs:2340-2352
+//   contract violations are loud                       nn/moe.rs:119-130
+//   route known answers                                models/qwen4exp/experts.rs:1365-1388
+// `--no-gpu` runs only the checks that need no device (config validation).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "mummu_moe.hpp"
+
+static int failures = 0;
+#define EXPECT(cond, what)                                         \
+    do {                                                           \
+        if (!(cond)) {                                             \
+            std::printf("FAIL %s:%d %s\n", __FILE__, __LINE__, what); \
+            failures++;                                            \
+        }                                                          \
+    } while (0)
+
+static const int H = 4, I = 3, E = 4, K = 2;
+
+// f32_from_usize(i).mul_add(0.37, seed).sin() * 0.5  (nn/moe.rs:1627-1629)
+static std::vector<float> sin_fill(float seed, int n) {
+    std::vector<float> v((size_t)n);
+    for (int i = 0; i < n; i++) {
+        const float arg = (float)((double)i * (double)0.37f + (double)seed);
+        v[(size_t)i] = (float)std::sin((double)arg) * 0.5f;
+    }
+    return v;
+}
+
+// router stored [H,E] in the reference (nn/moe.rs:1642-1645); the ABI takes row-major [E,H].
+static std::vector<float> router_eh() {
+    std::vector<float> he((size_t)(H * E)), eh((size_t)(E * H));
+    for (int i = 0; i < H * E; i++) he[(size_t)i] = (float)std::cos((double)(float)((double)i * (double)0.61f + 1.0)) * 0.5f;
+    for (int h = 0; h < H; h++)
+        for (int e = 0; e < E; e++) eh[(size_t)(e * H + h)] = he[(size_t)(h * E + e)];
+    return eh;
+}
+
+// ((i + seed) * 0.9).sin()  (nn/moe.rs:2088-2093)
+static std::vector<float> input(int t, float seed) {
+    std::vector<float> x((size_t)(t * H));
+    for (int i = 0; i < t * H; i++) x[(size_t)i] = (float)std::sin((double)(((float)i + seed) * 0.9f));
+    return x;
+}
+
+// The hand-rolled scalar block of nn/moe.rs:2101-2175.
+static std::vector<float> reference(const std::vector<float> &r, const std::vector<float> &g, const std::vector<float> &u,
+                                    const std::vector<float> &d, const std::vector<float> &xs, int t, int top_k, bool norm) {
+    std::vector<float> out((size_t)(t * H), 0.0f);
+    for (int tok = 0; tok < t; tok++) {
+        const float *x = &xs[(size_t)(tok * H)];
+        float logits[E], probs[E];
+        for (int e = 0; e < E; e++) {
+            float s = 0.0f;
+            for (int i = 0; i < H; i++) s += x[i] * r[(size_t)(e * H + i)];
+            logits[e] = s;
+        }
+        float mx = logits[0];
+        for (int e = 1; e < E; e++) mx = logits[e] > mx ? logits[e] : mx;
+        float total = 0.0f;
+        for (int e = 0; e < E; e++) {
+            probs[e] = std::exp(logits[e] - mx);
+            total += probs[e];
+        }
+        for (int e = 0; e < E; e++) probs[e] /= total;
+        int order[E];
+        for (int e = 0; e < E; e++) order[e] = e;
+        for (int a = 1; a < E; a++)  // stable insertion sort, descending
+            for (int b = a; b > 0 && probs[order[b]] > probs[order[b - 1]]; b--) std::swap(order[b], order[b - 1]);
+        float denom = 1.0f;
+        if (norm) {
+            denom = 0.0f;
+            for (int s = 0; s < top_k; s++) denom += probs[order[s]];
+        }
+        for (int s = 0; s < top_k; s++) {
+            const int e = order[s];
+            const float weight = probs[e] / denom;
+            float act[I];
+            for (int j = 0; j < I; j++) {
+                float gg = 0.0f, uu = 0.0f;
+                for (int i = 0; i < H; i++) {
+                    gg += x[i] * g[(size_t)((e * I + j) * H + i)];
+                    uu += x[i] * u[(size_t)((e * I + j) * H + i)];
+                }
+                act[j] = gg / (1.0f + std::exp(-gg)) * uu;
+            }
+            for (int i = 0; i < H; i++) {
+                float dd = 0.0f;
+                for (int j = 0; j < I; j++) dd += act[j] * d[(size_t)((e * H + i) * I + j)];
+                out[(size_t)(tok * H + i)] += weight * dd;
+            }
+        }
+    }
+    return out;
+}
+
+template <typename F>
+static bool throws(F &&f, int status, const char *needle) {
+    try {
+        f();
+    } catch (const mummu::MoeError &e) {
+        return e.status() == status && std::strstr(e.what(), needle) != nullptr;
+    }
+    return false;
+}
+
+int main(int argc, char **argv) {
+    const bool no_gpu = argc > 1 && std::string(argv[1]) == "--no-gpu";
+    mummu::SparseMoeConfig cfg;
+    cfg.hidden_size = H;
+    cfg.expert_intermediate_size = I;
+    cfg.num_experts = E;
+    cfg.num_experts_per_tok = K;
+    cfg.max_tokens = 8;
+
+    // SparseMoeConfig::init refuses a block that is not a mixture (nn/moe.rs:62-76)
+    {
+        mummu::SparseMoeConfig bad = cfg;
+        bad.num_experts = 1;
+        EXPECT(throws([&] { mummu::SparseMoe m(bad); }, MUMMU_ERR_CONFIG, "experts"), "num_experts = 1 must be refused");
+        bad = cfg;
+        bad.num_experts_per_tok = E + 1;
+        EXPECT(throws([&] { mummu::SparseMoe m(bad); }, MUMMU_ERR_CONFIG, "num_experts_per_tok"), "top_k > E must be refused");
+        bad = cfg;
+        bad.hidden_size = 0;
+        EXPECT(throws([&] { mummu::SparseMoe m(bad); }, MUMMU_ERR_CONFIG, "hidden"), "zero hidden size must be refused");
+    }
+    if (no_gpu) {
+        std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror (no gpu): ok\n", failures);
+        return failures ? 1 : 0;
+    }
+
+    const std::vector<float> r = router_eh(), g = sin_fill(0.1f, E * I * H), u = sin_fill(1.7f, E * I * H),
+                             d = sin_fill(3.3f, E * H * I);
+    mummu::SparseMoe moe(cfg);
+    moe.load_layer(0, {r.data(), MUMMU_F32}, {g.data(), MUMMU_F32}, {u.data(), MUMMU_F32}, {d.data(), MUMMU_F32});
+    EXPECT(moe.resident_bytes() == (uint64_t)4 * (E * H + 3 * E * I * H), "resident bytes");
+
+    for (int t : {5, 1})
+        for (bool norm : {false, true})
+            for (int k : {K, E}) {
+                const std::vector<float> x = input(t, 0.0f);
+                const std::vector<float> got = moe.forward(x, k, norm), want = reference(r, g, u, d, x, t, k, norm);
+                float worst = 0.0f;
+                for (size_t i = 0; i < got.size(); i++) worst = std::fmax(worst, std::fabs(got[i] - want[i]));
+                EXPECT(worst <= 1e-5f, "forward vs hand-rolled reference (1e-5 absolute, nn/moe.rs:2197)");
+                // routed == fused, bit for bit; every token spends top_k hits
+                (void)moe.take_hits();
+                const mummu::Routing routing = moe.route(x, k, norm);
+                const std::vector<float> routed = moe.run_local(x, routing);
+                EXPECT(std::memcmp(routed.data(), got.data(), got.size() * 4) == 0, "run_local(route(x)) == forward(x)");
+                size_t served = 0;
+                for (const auto &pe : routing.per_expert) {
+                    served += pe.first.size();
+                    for (size_t i = 1; i < pe.first.size(); i++) EXPECT(pe.first[i - 1] < pe.first[i], "rows ascend per expert");
+                }
+                EXPECT(served == (size_t)(t * k), "every token is served top_k times");
+                uint64_t hits = 0;
+                for (uint64_t hh : moe.take_hits()) hits += hh;
+                EXPECT(hits == (uint64_t)(t * k), "hit counters count the rows run_local served (route alone serves none)");
+            }
+
+    // zero in, zero out (nn/moe.rs:2340-2352)
+    {
+        const std::vector<float> z((size_t)(3 * H), 0.0f);
+        for (float v : moe.forward(z, K, false)) EXPECT(v == 0.0f, "zero input gives zero output");
+    }
+    // contract violations are loud (nn/moe.rs:119-130)
+    {
+        const std::vector<float> x = input(2, 0.0f);
+        EXPECT(throws([&] { moe.forward(x, 0, false); }, MUMMU_ERR_TOPK, "top_k"), "top_k = 0");
+        EXPECT(throws([&] { moe.forward(x, E + 1, false); }, MUMMU_ERR_TOPK, "top_k"), "top_k > E");
+        EXPECT(throws([&] { moe.forward(std::vector<float>(7), K, false); }, MUMMU_ERR_SHAPE, "hidden"), "ragged input");
+        EXPECT(throws([&] { moe.forward(x, K, false, 1); }, MUMMU_ERR_RANGE, "layer"), "layer out of range");
+    }
+    // ExpertExec seam: one expert alone equals a top-1 routing to it with weight 1
+    {
+        mummu::HipExpert ex(moe, 0, 2);
+        const std::vector<float> x = input(3, 1.0f);
+        const std::vector<float> y = ex.run(x.data(), 3, H);
+        mummu::RoutedExperts re(moe);
+        const std::vector<float> y2 = re.apply_routing(0, {2, 2, 2}, {1.0f, 1.0f, 1.0f}, x, 3, 1);
+        EXPECT(std::memcmp(y.data(), y2.data(), y.size() * 4) == 0, "ExpertExec::run == apply_routing(top-1, weight 1)");
+        EXPECT(throws([&] { re.apply_routing(0, {2, 9, 2}, {1.0f, 1.0f, 1.0f}, x, 3, 1); }, MUMMU_ERR_RANGE, "expert"), "bad expert id");
+    }
+    // route known answers (experts.rs:1365-1388)
+    {
+        const std::vector<float> logits = {0.0f, 3.0f, 1.0f, 2.5f, -2.0f, 2.0f, 0.5f, 2.9f};
+        auto rw = mummu::route(moe, logits, 1, 8, 3);
+        EXPECT(rw.first == (std::vector<int32_t>{1, 7, 3}), "route ids [1,7,3]");
+        double sum = 0.0, den = std::exp(3.0) + std::exp(2.9) + std::exp(2.5);
+        for (int s = 0; s < 3; s++) {
+            sum += rw.second[(size_t)s];
+            EXPECT(std::fabs(rw.second[(size_t)s] - std::exp((double)logits[(size_t)rw.first[(size_t)s]]) / den) < 1e-6, "route weights");
+        }
+        EXPECT(std::fabs(sum - 1.0) < 1e-6, "weights sum to 1");
+        auto tie = mummu::route(moe, {1.0f, 1.0f, 1.0f, 1.0f}, 1, 4, 3);
+        EXPECT(tie.first == (std::vector<int32_t>{0, 1, 2}), "ties keep the lower id");
+        auto tie2 = mummu::route(moe, {1.0f, 0.0f, 2.0f, 1.0f}, 1, 4, 2);
+        EXPECT(tie2.first == (std::vector<int32_t>{2, 0}), "[1,0,2,1] k=2 -> [2,0]");
+        const float nan = std::nanf("");
+        EXPECT(throws([&] { mummu::route(moe, {0.0f, nan, 1.0f}, 1, 3, 1); }, MUMMU_ERR_NONFINITE, "finite"), "NaN logit refused");
+        EXPECT(throws([&] { mummu::route(moe, {0.0f, 1.0f}, 1, 2, 3); }, MUMMU_ERR_TOPK, "top-3"), "k > E refused");
+    }
+    std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror: ok\n", failures);
+    return failures ? 1 : 0;
+}
