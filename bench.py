@@ -13,7 +13,7 @@ The whole rotation is captured once in a HIP graph and replayed (the serving-loo
 --no-graph times eager launches instead.
 
 Prints ONE JSON line (the contract the round driver reads), including
-  roofline      the dominant kernel (gate_up) against the 8 TB/s HBM peak, its duration
+  roofline      the dominant kernel against the 8 TB/s HBM peak, its duration
                 measured live with HIP events on the library's stream,
   cpu_baseline  the CPU oracle (a C restatement of the reference's routed CPU path) timed on
                 this host on a bounded sample of the same workload.
@@ -34,10 +34,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per gate_up launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
+# HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
 # same command (profiles/olmoe_q4k_decode_hbm_traffic.txt), each scaled by what the counter
 # reads for the library's 256 MiB copy kernel.  Only for the workload/batch they were taken on.
-PROFILED_GATE_UP_TRAFFIC = {("olmoe_q4k_decode", 1): 19119082}
+PROFILED_TRAFFIC = {}
 
 WORKLOADS = {
     # name: (hidden, inter, experts, top_k, norm, bank type, router type)
@@ -180,11 +180,17 @@ def main() -> int:
     kt = moe.kernel_times()
     moe.kernel_timing(False)
     per_kernel_us = {name: (tot / cnt * 1e3 if cnt else None) for name, (tot, cnt) in kt.items()}
-    gu_us = per_kernel_us.get("gate_up")
-    gu_bytes = mean_distinct * gate_up_expert_bytes
+    layer_bytes = mean_distinct * expert_bytes + router_bytes + n * H * 8
+    # the dominant kernel and the bytes one launch of it has to move
+    kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes,
+                    "down_combine": mean_distinct * (expert_bytes - gate_up_expert_bytes),
+                    "gemm_gate_up": mean_distinct * gate_up_expert_bytes}
+    timed = {name: us for name, us in per_kernel_us.items() if us is not None and name in kernel_bytes}
+    dom = max(timed, key=lambda name: timed[name] * kt[name][1]) if timed else None
+    gu_us = timed.get(dom) if dom else None
+    gu_bytes = kernel_bytes[dom] if dom else 0.0
     achieved = gu_bytes / (gu_us * 1e-6) / 1e9 if gu_us else None
 
-    layer_bytes = mean_distinct * expert_bytes + router_bytes + n * H * 8
     layer_gbs = layer_bytes / (ms_per_step * 1e-3) / 1e9
 
     out = {
@@ -211,10 +217,10 @@ def main() -> int:
         "layer_hbm_gbs": round(layer_gbs, 1),
         "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4),
         "kernel_us": {k_: (round(v, 3) if v is not None else None) for k_, v in per_kernel_us.items()},
-        "roofline": {"bound": "hbm", "kernel": "gate_up", "achieved": round(achieved, 1) if achieved else None,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1) if achieved else None,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
-                     "traffic": PROFILED_GATE_UP_TRAFFIC.get((args.workload, n)),
+                     "traffic": PROFILED_TRAFFIC.get((args.workload, n, dom)),
                      "algorithmic_bytes_per_launch": int(gu_bytes), "avg_launch_us": round(gu_us, 3) if gu_us else None},
         "device": M.device_name(),
         "setup_s": round(setup_s, 1),

@@ -32,7 +32,7 @@ inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_
 constexpr int kWave = 64;
 
 // Phase marks for kernel timing studies.  A normal build compiles them away; with
-// -DMUMMU_TRACE every wave stores the shader clock at each mark into a caller-provided buffer
+// -DMUMMU_TRACE every wave stores the constant 100 MHz wall clock at each mark into a caller-provided buffer
 // (8 slots per wave), set per translation unit through mummu_trace_set_<unit>().
 #ifdef MUMMU_TRACE
 static __device__ long long *g_trace_buf = nullptr;
@@ -40,7 +40,7 @@ static __device__ long long *g_trace_buf = nullptr;
     do {                                                                                                          \
         if (g_trace_buf && (threadIdx.x & 63) == 0)                                                               \
             g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + \
-                        (ph)] = clock64();                                                                        \
+                        (ph)] = wall_clock64();                                                                       \
     } while (0)
 #define MUMMU_TRACE_UNIT(name)                                                                      \
     extern "C" __attribute__((visibility("default"))) int mummu_trace_set_##name(void *p) {         \

@@ -26,228 +26,13 @@
 // each weight and the f32 activation.
 #include "device_utils.h"
 #include "kernels.h"
+#include "gemv_common.h"
 
 MUMMU_TRACE_UNIT(experts)
 
 namespace mummu {
 
 constexpr int kGemvWaves = 4;  // waves per workgroup of the float kernels
-
-// ------------------------------------------------------------------------------------------
-// Lane geometry of one quantized weight row split in 32-element "units".
-// ------------------------------------------------------------------------------------------
-struct RowSplit {
-    int units;        // units per row (in_dim / 32)
-    int group;        // lanes that share a row (power of two, <= 64)
-    int group_log2;
-    int rows_per_it;  // rows a wave handles per iteration = 64 / group
-};
-
-__host__ __device__ inline RowSplit row_split(int in_dim) {
-    RowSplit r;
-    r.units = in_dim / 32;
-    int lg = 0;
-    while ((1 << lg) < r.units && lg < 6) lg++;
-    r.group_log2 = lg;
-    r.group = 1 << lg;
-    r.rows_per_it = 64 >> lg;
-    return r;
-}
-
-// Start elements of the two 16-element halves unit u of a row covers.
-template <int WT>
-__device__ inline void unit_halves(int u, int &e0, int &e1) {
-    if constexpr (WT == T_Q4_K) {
-        int sb = u >> 3, up = u & 7;
-        e0 = sb * 256 + (up >> 1) * 64 + (up & 1) * 16;  // low nibbles: elements of sub-block 2c
-        e1 = e0 + 32;                                    // high nibbles: sub-block 2c+1
-    } else {
-        e0 = u * 32;
-        e1 = e0 + 16;
-    }
-}
-
-// The lane's share of a quantized activation row: 32 values (two 16-element blocks).
-template <int UPL>
-struct LaneAct {
-    int xh[UPL][8];   // hi bytes, 4 per word: words 0-3 first half, 4-7 second half
-    int xl[UPL][8];   // lo bytes
-    float s[UPL][2];  // scale of each half
-    int sx[UPL][2];   // sum(xq) of each half
-};
-
-template <int WT, int UPL>
-__device__ inline void load_lane_act(const QAct &q, size_t row, int d, int unit0, int units, LaneAct<UPL> &a) {
-    const int8_t *hi = q.hi + row * (size_t)d;
-    const int8_t *lo = q.lo + row * (size_t)d;
-    const float *sc = q.scale + row * (size_t)(d / 16);
-    const int32_t *sm = q.sum + row * (size_t)(d / 16);
-#pragma unroll
-    for (int i = 0; i < UPL; i++) {
-        const int u = unit0 + 64 * i;
-        const bool on = u < units;
-        int e0, e1;
-        unit_halves<WT>(on ? u : 0, e0, e1);
-        const int4 h0 = *(const int4 *)(hi + e0), h1 = *(const int4 *)(hi + e1);
-        const int4 l0 = *(const int4 *)(lo + e0), l1 = *(const int4 *)(lo + e1);
-        a.xh[i][0] = h0.x; a.xh[i][1] = h0.y; a.xh[i][2] = h0.z; a.xh[i][3] = h0.w;
-        a.xh[i][4] = h1.x; a.xh[i][5] = h1.y; a.xh[i][6] = h1.z; a.xh[i][7] = h1.w;
-        a.xl[i][0] = l0.x; a.xl[i][1] = l0.y; a.xl[i][2] = l0.z; a.xl[i][3] = l0.w;
-        a.xl[i][4] = l1.x; a.xl[i][5] = l1.y; a.xl[i][6] = l1.z; a.xl[i][7] = l1.w;
-        a.s[i][0] = on ? sc[e0 >> 4] : 0.0f;
-        a.s[i][1] = on ? sc[e1 >> 4] : 0.0f;
-        a.sx[i][0] = on ? sm[e0 >> 4] : 0;
-        a.sx[i][1] = on ? sm[e1 >> 4] : 0;
-    }
-}
-
-// The lane's raw share of one quantized weight row, as loaded (nothing decoded yet).
-template <int WT, int UPL>
-struct RawRow;
-template <int UPL>
-struct RawRow<T_Q4_K, UPL> {
-    uint4 hdr[UPL];  // f16 d, f16 dmin, 12 B of 6-bit scales/mins
-    uint4 q[UPL];    // the lane's 16 bytes of nibbles
-};
-template <int UPL>
-struct RawRow<T_Q8_0, UPL> {
-    uint32_t d[UPL];     // f16 scale bits
-    uint32_t q[UPL][8];  // 32 int8 codes
-};
-
-template <int WT, int UPL>
-__device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int units, bool ok, RawRow<WT, UPL> &r) {
-#pragma unroll
-    for (int i = 0; i < UPL; i++) {
-        const int u = unit0 + 64 * i;
-        const bool on = ok && u < units;
-        if constexpr (WT == T_Q4_K) {
-            r.hdr[i] = make_uint4(0, 0, 0, 0);
-            r.q[i] = make_uint4(0, 0, 0, 0);
-            if (on) {
-                const uint8_t *blk = rowp + (size_t)(u >> 3) * 144;
-                r.hdr[i] = *(const uint4 *)blk;
-                r.q[i] = *(const uint4 *)(blk + 16 + (u & 7) * 16);
-            }
-        } else {
-            r.d[i] = 0;
-#pragma unroll
-            for (int w = 0; w < 8; w++) r.q[i][w] = 0;
-            if (on) {
-                const uint8_t *blk = rowp + (size_t)u * 34;
-                uint16_t db;
-                __builtin_memcpy(&db, blk, 2);
-                r.d[i] = db;
-#pragma unroll
-                for (int w = 0; w < 8; w++) __builtin_memcpy(&r.q[i][w], blk + 2 + 4 * w, 4);  // 2-byte aligned
-            }
-        }
-    }
-}
-
-// The lane's partial of <row, activation> (formulas in the file comment).  A lane that loaded
-// nothing holds zero scales and contributes exactly 0.
-template <int WT, int UPL>
-__device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneAct<UPL> &a) {
-    float acc = 0.0f;
-#pragma unroll
-    for (int i = 0; i < UPL; i++) {
-        if constexpr (WT == T_Q4_K) {
-            const int u = unit0 + 64 * i;
-            const uint4 hdr = r.hdr[i];
-            const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFFu));
-            const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
-            // 6-bit (scale, min) of sub-blocks 2c, 2c+1 (ggml get_scale_min_k4), c fixed per lane
-            const int c = (u & 7) >> 1;
-            const int sh = 16 * (c & 1);
-            int sc0, sc1, mn0, mn1;
-            if (c < 2) {
-                sc0 = (int)((hdr.y >> sh) & 63u);
-                sc1 = (int)((hdr.y >> (sh + 8)) & 63u);
-                mn0 = (int)((hdr.z >> sh) & 63u);
-                mn1 = (int)((hdr.z >> (sh + 8)) & 63u);
-            } else {
-                const uint32_t lo = hdr.w >> sh;
-                sc0 = (int)((lo & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4));
-                mn0 = (int)(((lo >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4));
-                sc1 = (int)(((lo >> 8) & 0xFu) | (((hdr.y >> (sh + 14)) & 3u) << 4));
-                mn1 = (int)(((lo >> 12) & 0xFu) | (((hdr.z >> (sh + 14)) & 3u) << 4));
-            }
-            const uint32_t q[4] = {r.q[i].x, r.q[i].y, r.q[i].z, r.q[i].w};
-            int lh = 0, ll = 0, hh = 0, hl = 0;
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                int lo = (int)(q[w] & 0x0F0F0F0Fu);
-                int hi = (int)((q[w] >> 4) & 0x0F0F0F0Fu);
-                lh = __builtin_amdgcn_sdot4(lo, a.xh[i][w], lh, false);
-                ll = __builtin_amdgcn_sdot4(lo, a.xl[i][w], ll, false);
-                hh = __builtin_amdgcn_sdot4(hi, a.xh[i][4 + w], hh, false);
-                hl = __builtin_amdgcn_sdot4(hi, a.xl[i][4 + w], hl, false);
-            }
-            // |sum(q*xq)| <= 15*32512*16 < 2^23 and |sum(xq)| <= 16*32512: 24-bit multiplies are exact
-            const float p0 = (float)__mul24(sc0, lh * 256 + ll), p1 = (float)__mul24(sc1, hh * 256 + hl);
-            const float n0 = (float)__mul24(mn0, a.sx[i][0]), n1 = (float)__mul24(mn1, a.sx[i][1]);
-            const float pos = __builtin_fmaf(a.s[i][0], p0, __fmul_rn(a.s[i][1], p1));
-            const float neg = __builtin_fmaf(a.s[i][0], n0, __fmul_rn(a.s[i][1], n1));
-            acc = __fadd_rn(acc, __builtin_fmaf(-dmin, neg, __fmul_rn(d, pos)));
-        } else {  // Q8_0
-            const float d = half_bits_to_float((uint16_t)r.d[i]);
-            int h0 = 0, l0 = 0, h1 = 0, l1 = 0;
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                h0 = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xh[i][w], h0, false);
-                l0 = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xl[i][w], l0, false);
-                h1 = __builtin_amdgcn_sdot4((int)r.q[i][4 + w], a.xh[i][4 + w], h1, false);
-                l1 = __builtin_amdgcn_sdot4((int)r.q[i][4 + w], a.xl[i][4 + w], l1, false);
-            }
-            const float t = __builtin_fmaf(a.s[i][0], (float)(h0 * 256 + l0), __fmul_rn(a.s[i][1], (float)(h1 * 256 + l1)));
-            acc = __builtin_fmaf(d, t, acc);
-        }
-    }
-    return acc;
-}
-
-// The lane's partial of <row, activation> for a float row: elements lane*VEC + 64*VEC*j.
-template <int WT, int VEC>
-__device__ inline float row_partial_f(const uint8_t *__restrict__ rowp, const float *__restrict__ xrow, int in_dim,
-                                      int lane) {
-    float acc = 0.0f;
-    for (int i = lane * VEC; i < in_dim; i += 64 * VEC) {
-        float w[VEC];
-        if constexpr (WT == T_F32) {
-            if constexpr (VEC == 4) {
-                float4 v = *(const float4 *)(rowp + (size_t)i * 4);
-                w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
-            } else {
-                w[0] = *(const float *)(rowp + (size_t)i * 4);
-            }
-        } else {
-            if constexpr (VEC == 4) {
-                uint2 v = *(const uint2 *)(rowp + (size_t)i * 2);
-                uint16_t h[4] = {(uint16_t)(v.x & 0xFFFF), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xFFFF), (uint16_t)(v.y >> 16)};
-#pragma unroll
-                for (int j = 0; j < 4; j++) w[j] = WT == T_F16 ? half_bits_to_float(h[j]) : bf16_bits_to_float(h[j]);
-            } else {
-                uint16_t h = *(const uint16_t *)(rowp + (size_t)i * 2);
-                w[0] = WT == T_F16 ? half_bits_to_float(h) : bf16_bits_to_float(h);
-            }
-        }
-        if constexpr (VEC == 4) {
-            float4 xv = *(const float4 *)(xrow + i);
-            acc = __builtin_fmaf(w[0], xv.x, acc);
-            acc = __builtin_fmaf(w[1], xv.y, acc);
-            acc = __builtin_fmaf(w[2], xv.z, acc);
-            acc = __builtin_fmaf(w[3], xv.w, acc);
-        } else {
-            acc = __builtin_fmaf(w[0], xrow[i], acc);
-        }
-    }
-    return acc;
-}
-
-__host__ __device__ inline size_t type_row_bytes(int type, int in_dim) {
-    return (size_t)(in_dim / block_elems(type)) * (size_t)block_bytes(type);
-}
 
 // ------------------------------------------------------------------------------------------
 // gate/up, quantized banks: NIT iterations of rows_per_it rows per wave; the workgroup's
@@ -685,7 +470,7 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
     } while (0)
     if (upl == 1) {
         if (k <= 4) MUMMU_DC(1, 4, 1);
-        else MUMMU_DC(1, 4, 2);
+        else MUMMU_DC(1, 2, 2);
     } else {
         if (k <= 4) MUMMU_DC(2, 2, 1);
         else MUMMU_DC(2, 2, 2);

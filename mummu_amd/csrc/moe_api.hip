@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <climits>
+#include <cstdlib>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -154,8 +155,11 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     return MUMMU_OK;
 }
 
+// Device error flags back to idle.
+constexpr int kFlagWords = 4;
+
 int reset_flags(mummu_moe *h) {
-    const int32_t init[4] = {0, INT_MAX, 0, 0};
+    const int32_t init[kFlagWords] = {0, INT_MAX, 0, 0};
     HIPCHK(h, hipMemcpy(h->flags, init, sizeof(init), hipMemcpyHostToDevice));
     return MUMMU_OK;
 }
@@ -372,7 +376,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     if (hipStreamCreate(&h->stream) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipStreamCreate failed"));
     if (hipEventCreate(&h->t0) != hipSuccess || hipEventCreate(&h->t1) != hipSuccess)
         return bail(fail(h, MUMMU_ERR_DEVICE, "hipEventCreate failed"));
-    if (hipMalloc(&h->flags, sizeof(int32_t) * 4) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(flags) failed"));
+    if (hipMalloc(&h->flags, sizeof(int32_t) * kFlagWords) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(flags) failed"));
     int rc = reset_flags(h);
     if (rc) return bail(rc);
     rc = ensure_ws(h, cfg->max_tokens, (int64_t)cfg->max_tokens * cfg->num_experts_per_tok, cfg->num_experts);

@@ -19,9 +19,8 @@ struct QAct {
 };
 
 // Quantize 16 consecutive activations held one per lane in an aligned 16-lane row (an inactive
-// row holds zeros) and store them: the lanes write their hi/lo bytes, the lane of the block's
-// first element the block scale and sum.
-__device__ inline void quantize_store16(float v, bool active, const QAct &q, size_t row, int d, int elem) {
+// row holds zeros): every lane gets its hi/lo bytes and the block's scale and integer sum.
+__device__ inline void quantize16(float v, int &hi, int &lo, float &scale, int &sum) {
     float m = fabsf(v);
     m = fmaxf(m, dpp_move<0xB1>(m));
     m = fmaxf(m, dpp_move<0x4E>(m));
@@ -30,18 +29,27 @@ __device__ inline void quantize_store16(float v, bool active, const QAct &q, siz
     const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
     int xq = (int)__builtin_rintf(__fmul_rn(v, inv));
     xq = xq > 32512 ? 32512 : (xq < -32512 ? -32512 : xq);
-    const int lo = ((xq + 128) & 255) - 128;
-    const int hi = (xq - lo) >> 8;
-    int sum = xq;
+    lo = ((xq + 128) & 255) - 128;
+    hi = (xq - lo) >> 8;
+    sum = xq;
     sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, false);
     sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, false);
     sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xF, 0xF, false);
     sum += __builtin_amdgcn_update_dpp(0, sum, 0x140, 0xF, 0xF, false);
+    scale = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
+}
+
+// ... and store them: the lanes write their hi/lo bytes, the lane of the block's first element
+// the block scale and sum.
+__device__ inline void quantize_store16(float v, bool active, const QAct &q, size_t row, int d, int elem) {
+    int hi, lo, sum;
+    float scale;
+    quantize16(v, hi, lo, scale, sum);
     if (active) {
         q.hi[row * (size_t)d + elem] = (int8_t)hi;
         q.lo[row * (size_t)d + elem] = (int8_t)lo;
         if ((elem & 15) == 0) {
-            q.scale[row * (size_t)(d / 16) + (elem >> 4)] = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
+            q.scale[row * (size_t)(d / 16) + (elem >> 4)] = scale;
             q.sum[row * (size_t)(d / 16) + (elem >> 4)] = sum;
         }
     }

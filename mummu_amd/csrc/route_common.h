@@ -1,0 +1,221 @@
+// Device pieces shared by the router kernels: router weight loads and the one-wave softmax /
+// top-k / renormalise of one token.
+#pragma once
+
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace mummu {
+
+constexpr int kMaxExpertsPerLane = 8;  // num_experts <= 512
+
+template <int WT>
+__device__ inline float load_w(const void *w, size_t i) {
+    if constexpr (WT == T_F32) return ((const float *)w)[i];
+    else if constexpr (WT == T_F16) return half_bits_to_float(((const uint16_t *)w)[i]);
+    else return bf16_bits_to_float(((const uint16_t *)w)[i]);
+}
+
+// 8 consecutive weights starting at element i (i % 8 == 0, 16-byte aligned rows).
+template <int WT>
+__device__ inline void load_w8(const void *w, size_t i, float (&o)[8]) {
+    if constexpr (WT == T_F32) {
+        const float4 *p = (const float4 *)((const float *)w + i);
+        float4 a = p[0], b = p[1];
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    } else {
+        uint4 v = *(const uint4 *)((const uint16_t *)w + i);
+        uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint16_t lo = (uint16_t)(u[j] & 0xFFFFu), hi = (uint16_t)(u[j] >> 16);
+            if constexpr (WT == T_F16) {
+                o[2 * j] = half_bits_to_float(lo);
+                o[2 * j + 1] = half_bits_to_float(hi);
+            } else {
+                o[2 * j] = bf16_bits_to_float(lo);
+                o[2 * j + 1] = bf16_bits_to_float(hi);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// softmax -> top-k -> renormalise, one wave per token.  Lane l holds experts l, l+64, ...
+// Ties: strictly-greater wins, so the lower expert id keeps a tie and equal slots ascend
+// by id (experts.rs:557-573; the stable descending sort of nn/moe.rs:2143-2144).
+//
+// The sequential sums and the ranking read every expert's value; the wave parks them in LDS
+// and every lane streams them back with broadcast 16-byte reads, which keeps the serial
+// chains to one add (or one compare) per element instead of a cross-lane move per element.
+// ---------------------------------------------------------------------------------------
+__device__ inline void wave_lds_sync() {
+    // LDS traffic of one wave is issued in order; this only stops the compiler from moving
+    // the reads above the writes.
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// Per-wave LDS scratch of the router.
+template <int JN>
+struct RouteScratch {
+    float p[64 * JN];   // per-expert values, expert order
+    float w[64 * JN];   // selected probabilities, slot order
+    int id[64 * JN];    // selected expert ids, slot order
+};
+
+// One wave routes one token whose logits sit in l[j] (expert lane + 64*j).  JN = experts held
+// per lane (num_experts <= 64 * JN).
+template <int JN>
+__device__ inline void route_token(float (&l)[JN], int t, int n_experts, int k, int flavour, int norm,
+                                   int32_t *__restrict__ ids, float *__restrict__ weights,
+                                   unsigned long long *__restrict__ hits, int32_t *__restrict__ flags,
+                                   RouteScratch<JN> &sc) {
+    const int lane = threadIdx.x & 63;
+    float p[JN];
+    bool bad = false;
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        const int e = lane + 64 * j;
+        if (e < n_experts) {
+            if (!(fabsf(l[j]) <= 3.402823466e38f)) {  // inf or NaN
+                bad = true;
+                atomicMin(&flags[FLAG_NONFINITE_INDEX], t * n_experts + e);
+            }
+            mx = fmaxf(mx, l[j]);
+        }
+    }
+    if (__any(bad)) {
+        // Refused like experts.rs:546-553: flag it and emit a harmless, in-range routing so
+        // the kernels downstream stay inside their buffers; the host reports the error.
+        if (lane == 0) atomicAdd(&flags[FLAG_NONFINITE], 1);
+        for (int s = lane; s < k; s += 64) {
+            ids[(size_t)t * k + s] = s;
+            weights[(size_t)t * k + s] = 0.0f;
+        }
+        return;
+    }
+    mx = wave_max(mx);
+    // experts past n_experts hold +0: it leaves a running sum unchanged bit for bit and never
+    // outranks a real expert (not greater; on a tie at 0 its id is higher)
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(l[j], mx)) : 0.0f;
+        sc.p[lane + 64 * j] = p[j];
+    }
+    wave_lds_sync();
+
+    // normaliser: sequential over ascending expert id (every lane computes the same sum)
+    const float4 *bp = (const float4 *)sc.p;
+    if (flavour == 0) {
+        float total = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 16 * JN; c++) {
+            const float4 v = bp[c];
+            total = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(total, v.x), v.y), v.z), v.w);
+        }
+#pragma unroll
+        for (int j = 0; j < JN; j++) p[j] = __fdiv_rn(p[j], total);
+    } else {
+        double total = 0.0;
+#pragma unroll
+        for (int c = 0; c < 16 * JN; c++) {
+            const float4 v = bp[c];
+            total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
+        }
+        const float scale = (float)__ddiv_rn(1.0, total);
+#pragma unroll
+        for (int j = 0; j < JN; j++) p[j] = __fmul_rn(p[j], scale);
+    }
+
+    if (k <= 16) {
+        // k rounds of "largest remaining probability, lowest id on a tie": the wave maximum,
+        // then the first lane (and, within a lane, the first expert) that holds it
+        float cand[JN];
+#pragma unroll
+        for (int j = 0; j < JN; j++) cand[j] = (lane + 64 * j < n_experts) ? p[j] : -1.0f;
+        for (int s = 0; s < k; s++) {
+            float best = cand[0];
+#pragma unroll
+            for (int j = 1; j < JN; j++) best = fmaxf(best, cand[j]);
+            best = wave_max(best);
+            // lowest expert id holding `best` (id = lane + 64*j)
+            int my = 0x7FFFFFFF;
+#pragma unroll
+            for (int j = JN - 1; j >= 0; j--)
+                if (cand[j] == best) my = lane + 64 * j;
+            int win = my;
+            if (JN == 1) {
+                const unsigned long long m = __ballot(my != 0x7FFFFFFF);
+                win = (int)__builtin_ctzll(m);
+            } else {
+                // minimum id over the wave
+                float f = -(float)win;  // ids < 2^24: exact in f32, negated so that max finds the minimum
+                f = wave_max(f);
+                win = (int)(-f);
+            }
+#pragma unroll
+            for (int j = 0; j < JN; j++)
+                if (lane + 64 * j == win) cand[j] = -1.0f;
+            if (lane == 0) {
+                sc.w[s] = best;
+                sc.id[s] = win;
+            }
+        }
+    } else {
+        // rank of each expert under (probability descending, id ascending); rank < k is its slot
+        wave_lds_sync();
+#pragma unroll
+        for (int j = 0; j < JN; j++) sc.p[lane + 64 * j] = p[j];
+        wave_lds_sync();
+        int rank[JN];
+#pragma unroll
+        for (int j = 0; j < JN; j++) rank[j] = 0;
+#pragma unroll
+        for (int c = 0; c < 16 * JN; c++) {
+            const float4 v = bp[c];
+            const float q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int eq = 4 * c + i;
+#pragma unroll
+                for (int j = 0; j < JN; j++) rank[j] += (q[i] > p[j]) || (q[i] == p[j] && eq < lane + 64 * j);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < JN; j++) {
+            if (lane + 64 * j < n_experts && rank[j] < k) {
+                sc.w[rank[j]] = p[j];
+                sc.id[rank[j]] = lane + 64 * j;
+            }
+        }
+    }
+    wave_lds_sync();
+
+    float denom = 1.0f;
+    if (flavour == 0) {
+        if (norm) {
+            float d = 0.0f;
+            for (int s = 0; s < k; s++) d = __fadd_rn(d, sc.w[s]);
+            denom = d;
+        }
+    } else {
+        double d = 0.0;
+        for (int s = 0; s < k; s++) d = __dadd_rn(d, (double)sc.w[s]);
+        const float fs = (float)d;
+        const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
+        denom = fs > floor_v ? fs : floor_v;
+    }
+    const bool divide = flavour != 0 || norm;
+    for (int s = lane; s < k; s += 64) {
+        float wv = sc.w[s];
+        const int id = sc.id[s];
+        if (divide) wv = __fdiv_rn(wv, denom);
+        ids[(size_t)t * k + s] = id;
+        weights[(size_t)t * k + s] = wv;
+        if (hits) atomicAdd(&hits[id], 1ULL);
+    }
+}
+
+}  // namespace mummu
