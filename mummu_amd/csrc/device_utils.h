@@ -46,9 +46,28 @@ static __device__ long long *g_trace_buf = nullptr;
     extern "C" __attribute__((visibility("default"))) int mummu_trace_set_##name(void *p) {         \
         return (int)hipMemcpyToSymbol(HIP_SYMBOL(mummu::g_trace_buf), &p, sizeof(p));                \
     }
+// Loop timers: MARK(i) adds the time since the previous mark to slot i; STORE writes the slot sums
+// (slot 6 = first mark's clock, slot 7 = last) to the wave's 8 trace words.
+#define MUMMU_TIMER_DECL long long tm_acc_[8] = {0, 0, 0, 0, 0, 0, 0, 0}, tm_last_ = wall_clock64(); tm_acc_[6] = tm_last_
+#define MUMMU_TIMER_MARK(i)                      \
+    do {                                         \
+        const long long now_ = wall_clock64();   \
+        tm_acc_[i] += now_ - tm_last_;           \
+        tm_last_ = now_;                         \
+    } while (0)
+#define MUMMU_TIMER_STORE                                                                                         \
+    do {                                                                                                          \
+        tm_acc_[7] = tm_last_;                                                                                    \
+        if (g_trace_buf && (threadIdx.x & 63) == 0)                                                               \
+            for (int i_ = 0; i_ < 8; i_++)                                                                        \
+                g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + i_] = tm_acc_[i_]; \
+    } while (0)
 #else
 #define MUMMU_PHASE(ph) do { } while (0)
 #define MUMMU_TRACE_UNIT(name)
+#define MUMMU_TIMER_DECL do { } while (0)
+#define MUMMU_TIMER_MARK(i) do { } while (0)
+#define MUMMU_TIMER_STORE do { } while (0)
 #endif
 
 // ggml tensor type ids (the values stored in GGUF tensor tables).
@@ -123,15 +142,6 @@ __device__ inline float det_silu(float x) {
     return __fdiv_rn(x, den);
 }
 
-// Butterfly sum over the whole wave, offsets 32,16,...,1.  Lane l ends with the value a
-// halving tree (s[l] += s[l+off] for l < off) leaves in s[0]; addition commutes, so every
-// lane holds the same bits.
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = __fadd_rn(v, __shfl_xor(v, off, kWave));
-    return v;
-}
-
 // Butterfly sum over aligned groups of `width` lanes (width a power of two <= 64).
 __device__ inline float group_sum(float v, int width) {
     for (int off = width >> 1; off >= 1; off >>= 1) v = __fadd_rn(v, __shfl_xor(v, off, kWave));
@@ -167,6 +177,18 @@ __device__ inline float swap32_add(float a, float b) {
 __device__ inline float swap16_add(float a, float b) {
     auto r = __builtin_amdgcn_permlane16_swap(__float_as_int(a), __float_as_int(b), false, false);
     return __fadd_rn(__int_as_float(r[0]), __int_as_float(r[1]));
+}
+
+// Sum over the whole wave as the pairwise tree over adjacent lanes: butterfly offsets
+// 1,2,4,8,16,32 (s[l] += s[l+off] for l a multiple of 2*off leaves the same value in s[0]).
+// Addition commutes, so every lane ends with the same bits.  Offsets 1 and 2 are quad permutes,
+// 4 and 8 the half-row and row mirrors (the mirrored partner holds the same value as the xor
+// partner, because the smaller groups are already uniform), 16 and 32 the gfx950 lane swaps:
+// no LDS round trip anywhere.  The whole wave must be active.
+__device__ inline float wave_sum(float v) {
+    v = row_group_sum<16>(v);
+    v = swap16_add(v, v);
+    return swap32_add(v, v);
 }
 
 // Number of finished sums a lane holds after reduce_partials<NV, GROUP>.

@@ -23,6 +23,8 @@
 #include "device_utils.h"
 #include "kernels.h"
 
+MUMMU_TRACE_UNIT(gemm)
+
 namespace mummu {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -51,6 +53,19 @@ __host__ __device__ inline size_t gemm_row_bytes(int type, int in_dim) {
 // (row 8*(r/4) + 4*(l/32) + r%4, column l%32) of the wave's 32x32 tile.
 __device__ inline int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 
+// Work-list entry of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin by their
+// linear id, and the grid's x extent is a multiple of 8, so workgroup x lands on XCD x % 8 for
+// every y.  Giving XCD j the contiguous run of tiles [j*ceil(T/8), (j+1)*ceil(T/8)) puts the
+// tiles of one expert (neighbours in the list) on the same XCD at about the same time - they
+// share that expert's weight slab in one L2 instead of pulling it into all eight - and keeps a
+// token tile on one XCD across the output slabs y.
+__device__ inline int xcd_tile(const int32_t *__restrict__ n_tiles) {
+    const int total = *n_tiles;
+    const int per_xcd = (total + 7) >> 3;
+    const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    return ((int)(blockIdx.x >> 3) < per_xcd && tile < total) ? tile : -1;
+}
+
 // ---------------------------------------------------------------------------------------
 // F16 banks
 // ---------------------------------------------------------------------------------------
@@ -69,19 +84,24 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     __shared__ __attribute__((aligned(16))) _Float16 s_a[BM][kLds];
     __shared__ __attribute__((aligned(16))) _Float16 s_b[NB][kBN][kLds];
 
-    const int tile = blockIdx.x;
-    if (tile >= *n_tiles) return;
+    const int tile = xcd_tile(n_tiles);
+    if (tile < 0) return;
     const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
     const int n0 = blockIdx.y * kBN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t row_bytes = (size_t)in_dim * 2;
 
-    // weight tile: thread -> (row, half of the K step)
-    const int b_row = tid >> 1, b_half = tid & 1;
-    const int b_out = n0 + b_row < out_dim ? n0 + b_row : out_dim - 1;  // clamped; never stored
-    const uint8_t *b_ptr[NB];
-    b_ptr[0] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_half * 64;
-    if (GATE_UP) b_ptr[NB - 1] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_half * 64;
+    // weight tile: a K step of one row is 128 contiguous bytes = 8 lanes x 16 B, so one load
+    // instruction of a wave covers 8 whole rows; thread -> chunk tid%8 of rows tid/8 + 32*i
+    const int b_chunk = tid & 7;
+    const uint8_t *b_ptr[NB][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = (tid >> 3) + 32 * i;
+        const int b_out = n0 + r < out_dim ? n0 + r : out_dim - 1;  // clamped; never stored
+        b_ptr[0][i] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_chunk * 16;
+        if (GATE_UP) b_ptr[NB - 1][i] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_chunk * 16;
+    }
 
     // activation tile: f32 source -> 16 threads per row, 4 elements each (2*MT passes of 16 rows);
     // f16 source -> 8 threads per row, 8 elements each (MT passes of 32 rows)
@@ -117,11 +137,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     uint4 ra16[A_PASSES];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const uint4 *p = (const uint4 *)(b_ptr[b] + (size_t)k0 * 2);
+        for (int b = 0; b < NB; b++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) rb[b][i] = p[i];
-        }
+            for (int i = 0; i < 4; i++) rb[b][i] = *(const uint4 *)(b_ptr[b][i] + (size_t)k0 * 2);
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) {
             if (GATE_UP) ra32[p] = a_src32[p] ? *(const float4 *)(a_src32[p] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -130,14 +148,14 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     };
     fetch(0);
 
+    MUMMU_TIMER_DECL;
     for (int k0 = 0; k0 < in_dim; k0 += kBK) {
+        MUMMU_TIMER_MARK(0);
         // registers -> LDS
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            uint4 *dst = (uint4 *)&s_b[b][b_row][b_half * 32];
+        for (int b = 0; b < NB; b++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) dst[i] = rb[b][i];
-        }
+            for (int i = 0; i < 4; i++) *(uint4 *)&s_b[b][(tid >> 3) + 32 * i][b_chunk * 8] = rb[b][i];
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) {
             if (GATE_UP) {
@@ -147,8 +165,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
                 *(uint4 *)&s_a[a_row[p]][a_col] = ra16[p];
             }
         }
+        MUMMU_TIMER_MARK(1);
         __syncthreads();
+        MUMMU_TIMER_MARK(2);
         if (k0 + kBK < in_dim) fetch(k0 + kBK);
+        MUMMU_TIMER_MARK(3);
         // multiply: wave owns columns 32*wave .. +31
 #pragma unroll
         for (int kk = 0; kk < kBK / 16; kk++) {
@@ -162,8 +183,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
                 for (int b = 0; b < NB; b++) acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[b], acc[b][m], 0, 0, 0);
             }
         }
+        MUMMU_TIMER_MARK(4);
         __syncthreads();
+        MUMMU_TIMER_MARK(5);
     }
+    MUMMU_TIMER_STORE;
 
     const int n = n0 + 32 * wave + (lane & 31);
     if (n < out_dim) {
@@ -270,7 +294,7 @@ struct QTileLds {
 //          act_out rows in sorted order.
 // else   : A = act_in rows in sorted order; y[pos, n] = f32 sum.
 template <int WT, bool GATE_UP, int MT>
-__global__ __launch_bounds__(256) void grouped_gemm_q_kernel(
+__global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
     const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, QAct64 a_in, const int32_t *__restrict__ sorted,
     int k_slots, const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim,
     QAct64 act_out, float *__restrict__ y_out) {
@@ -284,8 +308,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_q_kernel(
     auto s_a = [&](int plane, int row) -> uint8_t * { return s_raw + ((size_t)plane * BM + row) * kLdsQ; };
     auto s_b = [&](int b, int row) -> uint8_t * { return s_raw + L::kA + ((size_t)b * kBN + row) * kLdsQ; };
 
-    const int tile = blockIdx.x;
-    if (tile >= *n_tiles) return;
+    const int tile = xcd_tile(n_tiles);
+    if (tile < 0) return;
     const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
     const int n0 = blockIdx.y * kBN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -341,7 +365,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_q_kernel(
     fetch(0);
 
     const int col = 32 * wave + (lane & 31), g = lane >> 5;
+    MUMMU_TIMER_DECL;
     for (int k0 = 0; k0 < in_dim; k0 += kBK) {
+        MUMMU_TIMER_MARK(0);
         // registers -> LDS
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -358,8 +384,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_q_kernel(
         for (int p = 0; p < MT; p++) *(uint4 *)(s_a(a_plane, a_row[p]) + a_chunk * 16) = ra[p];
         if (tid < BM) s_as[tid] = ras;
         if (WT == T_Q4_K && tid < 2 * BM) s_am[tid >> 1][tid & 1] = ram;
+        MUMMU_TIMER_MARK(1);
         __syncthreads();
+        MUMMU_TIMER_MARK(2);
         if (k0 + kBK < in_dim) fetch(k0 + kBK);
+        MUMMU_TIMER_MARK(3);
 
         // multiply: wave owns columns 32*wave .. +31
 #pragma unroll
@@ -394,8 +423,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_q_kernel(
                     acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][g], s_bm[b][col][g], acc[b][m], 0, 0, 0);
             }
         }
+        MUMMU_TIMER_MARK(4);
         __syncthreads();
+        MUMMU_TIMER_MARK(5);
     }
+    MUMMU_TIMER_STORE;
 
     if (GATE_UP) {
         // stage silu(g)*u of the whole tile as f32 (over the A and B tiles, no longer needed),
@@ -463,7 +495,7 @@ template <int WT, bool GATE_UP>
 static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_in, const int32_t *sorted, int k_slots,
                                 const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
                                 int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
-    dim3 block(256), grid(max_tiles, (out_dim + kBN - 1) / kBN);
+    dim3 block(256), grid((max_tiles + 7) / 8 * 8, (out_dim + kBN - 1) / kBN);
     if (tile_rows == 64)
         launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, 2>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                      out_dim, act_out, y_out);
@@ -478,7 +510,7 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const fl
                                   const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
                                   int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
                                   hipStream_t s) {
-    dim3 block(256), grid(max_tiles, (out_dim + kBN - 1) / kBN);
+    dim3 block(256), grid((max_tiles + 7) / 8 * 8, (out_dim + kBN - 1) / kBN);
     if (tile_rows == 64)
         launch_kernel(grouped_gemm_f16_kernel<GATE_UP, 2>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                    out_dim, act_out, y_out);

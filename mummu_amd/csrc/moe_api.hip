@@ -64,7 +64,7 @@ struct mummu_moe {
     float *xin = nullptr, *xout = nullptr, *h2 = nullptr, *resid[2] = {nullptr, nullptr};
     QAct xq, actq;               // 16-bit activations: tokens x hidden, pairs x inter
     // dispatch-sorted layout of the batched path
-    int32_t *offsets = nullptr, *sorted = nullptr, *inv = nullptr, *tiles = nullptr, *n_tiles = nullptr;
+    int32_t *offsets = nullptr, *sorted = nullptr, *inv = nullptr, *tiles = nullptr, *n_tiles = nullptr, *disp_scratch = nullptr;
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
     int gemm_min_tokens = 32;    // batches at least this large take the grouped GEMM
@@ -97,14 +97,14 @@ size_t row_bytes_of(int t, int in_dim) { return (size_t)(in_dim / block_elems(t)
 void free_ws(mummu_moe *h) {
     void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1],
                     h->xq.hi, h->xq.lo, h->xq.scale, h->xq.sum, h->actq.hi, h->actq.lo, h->actq.scale, h->actq.sum,
-                    h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->act16};
+                    h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->act16, h->disp_scratch};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     h->logits = h->weights = h->act = h->y = h->xin = h->xout = h->h2 = h->resid[0] = h->resid[1] = nullptr;
     h->ids = nullptr;
     h->xq = QAct();
     h->actq = QAct();
-    h->offsets = h->sorted = h->inv = h->tiles = h->n_tiles = nullptr;
+    h->offsets = h->sorted = h->inv = h->tiles = h->n_tiles = h->disp_scratch = nullptr;
     h->act16 = nullptr;
     h->ws_tokens = h->ws_assign = 0;
     h->ws_experts = 0;
@@ -148,6 +148,7 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     HIPCHK(h, hipMalloc(&h->inv, sizeof(int32_t) * (size_t)na));
     HIPCHK(h, hipMalloc(&h->tiles, sizeof(int32_t) * 3 * (size_t)h->max_tiles));
     HIPCHK(h, hipMalloc(&h->n_tiles, sizeof(int32_t)));
+    HIPCHK(h, hipMalloc(&h->disp_scratch, sizeof(int32_t) * dispatch_scratch_ints((int)na, n_experts)));
     HIPCHK(h, hipMalloc(&h->act16, 2 * (size_t)na * I));
     h->ws_tokens = nt;
     h->ws_assign = na;
@@ -260,7 +261,7 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
         if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
         LAUNCH(h, K_DISPATCH, s,
-               launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->flags, s));
+               launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch, h->flags, s));
         LAUNCH(h, K_GEMM_GATE_UP, s,
                launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, actq64, s));
         LAUNCH(h, K_GEMM_DOWN, s,

@@ -67,7 +67,7 @@ struct RouteScratch {
 // One wave routes one token whose logits sit in l[j] (expert lane + 64*j).  JN = experts held
 // per lane (num_experts <= 64 * JN).
 template <int JN>
-__device__ inline void route_token(float (&l)[JN], int t, int n_experts, int k, int flavour, int norm,
+__device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts, int k, int flavour, int norm,
                                    int32_t *__restrict__ ids, float *__restrict__ weights,
                                    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags,
                                    RouteScratch<JN> &sc) {

@@ -8,8 +8,8 @@
 // Summation orders are fixed so the routing indices are reproducible bit for bit:
 //   * a logit is 512 strided partial sums (element i -> partial i mod 512, one fma per
 //     element in ascending i).  Lane l of the wave owns partials 8l..8l+7, folds them as
-//     ((a0+a4)+(a1+a5))+((a2+a6)+(a3+a7)), and the 64 lane sums fold by the xor butterfly
-//     32,16,...,1.
+//     ((a0+a4)+(a1+a5))+((a2+a6)+(a3+a7)), and the 64 lane sums fold pairwise over adjacent
+//     lanes (butterfly offsets 1,2,...,32).
 //   * softmax normaliser and top-k renorm sums run sequentially in ascending expert /
 //     slot order (f32, or f64 for the qwen4exp flavour), as the reference spells them out.
 #include "device_utils.h"
@@ -246,6 +246,93 @@ __global__ __launch_bounds__(64 * kRouterWaves) void router_block_kernel(
     MUMMU_PHASE(3);
 }
 
+constexpr int kRouterMaxChunks = 4;  // 512-element chunks of a row held in registers: hidden <= 2048 on the tiled path
+
+// Tiled form (hidden <= 2048, a multiple of 8): the tile's activation rows are staged in LDS
+// once and every wave walks its experts with the lane's slice of the weight row in registers
+// (lane l owns elements 8l..8l+7 of each 512-chunk, i.e. partials 8l..8l+7), so a weight row is
+// read once per tile and an activation row once per workgroup.  Same summation order as
+// router_logits_kernel.
+template <int WT, int TT, int JN>
+__global__ __launch_bounds__(64 * kRouterWaves) void router_tile_kernel(
+    const float *__restrict__ x, const void *__restrict__ w, int n, int hidden, int n_experts, int k, int flavour,
+    int norm, float *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ weights,
+    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags, QAct xq) {
+    extern __shared__ __attribute__((aligned(16))) float s_x[];  // [TT][hidden]
+    __shared__ float s_logits[TT][64 * JN];
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[TT];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t0 = blockIdx.x * TT;
+    const int tile_tokens = (n - t0) < TT ? (n - t0) : TT;
+    const int chunks = (hidden + 511) / 512;
+
+    // stage the tile (rows past the batch are zero) and quantize it where the expert kernels want that
+    for (int i = threadIdx.x * 4; i < TT * hidden; i += 64 * kRouterWaves * 4) {
+        const int t = i / hidden;
+        const float4 v = t < tile_tokens ? *(const float4 *)(x + (size_t)t0 * (size_t)hidden + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        *(float4 *)(s_x + i) = v;
+    }
+    if (xq.hi != nullptr) {
+        const int slices_per_row = hidden / 64;
+        for (int sl = wave; sl < tile_tokens * slices_per_row; sl += kRouterWaves) {
+            const int t = t0 + sl / slices_per_row;
+            const int elem = (sl % slices_per_row) * 64 + lane;
+            quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
+        }
+    }
+    __syncthreads();
+
+    for (int e = wave; e < n_experts; e += kRouterWaves) {
+        float wv[kRouterMaxChunks][8];
+#pragma unroll
+        for (int c = 0; c < kRouterMaxChunks; c++) {
+            const int base = c * 512 + lane * 8;
+            if (c < chunks && base < hidden) {
+                load_w8<WT>(w, (size_t)e * (size_t)hidden + (size_t)base, wv[c]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) wv[c][j] = 0.0f;
+            }
+        }
+        float sum[TT];
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[j] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < kRouterMaxChunks; c++) {
+                const int base = c * 512 + lane * 8;
+                if (c < chunks && base < hidden) {
+                    const float4 a = *(const float4 *)(s_x + t * hidden + base), b = *(const float4 *)(s_x + t * hidden + base + 4);
+                    const float xv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(xv[j], wv[c][j], acc[j]);
+                }
+            }
+            sum[t] = __fadd_rn(__fadd_rn(__fadd_rn(acc[0], acc[4]), __fadd_rn(acc[1], acc[5])),
+                               __fadd_rn(__fadd_rn(acc[2], acc[6]), __fadd_rn(acc[3], acc[7])));
+        }
+#pragma unroll
+        for (int t = 0; t < TT; t++) sum[t] = wave_sum(sum[t]);  // TT independent chains
+        if (lane < TT && lane < tile_tokens) {
+            float s = sum[0];
+#pragma unroll
+            for (int t = 1; t < TT; t++) s = lane == t ? sum[t] : s;
+            s_logits[lane][e] = s;
+            logits[(size_t)(t0 + lane) * (size_t)n_experts + (size_t)e] = s;
+        }
+    }
+    __syncthreads();
+    for (int t = wave; t < tile_tokens; t += kRouterWaves) {
+        float l[JN];
+#pragma unroll
+        for (int j = 0; j < JN; j++) l[j] = (lane + 64 * j < n_experts) ? s_logits[t][lane + 64 * j] : 0.0f;
+        route_token<JN>(l, t0 + t, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[t]);
+    }
+}
+
 template <int WT, bool VEC, int TT>
 static hipError_t launch_router_block_t(const float *x, const void *w, int n, int hidden, int n_experts, int k,
                                         int flavour, int norm, float *logits, int32_t *ids, float *weights,
@@ -270,6 +357,29 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
     if (n_experts > 128 || k > n_experts || k < 1) return hipErrorInvalidValue;
     if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
+    // enough tokens to fill the chip tile by tile: rows staged in LDS, weights in registers
+    if (n > 64 && vec && hidden <= 512 * kRouterMaxChunks) {
+        constexpr int TT = 4;
+        dim3 block(64 * kRouterWaves), grid((n + TT - 1) / TT);
+        const size_t lds = sizeof(float) * (size_t)TT * (size_t)hidden;
+#define MUMMU_RT(WT)                                                                                                     \
+    do {                                                                                                                 \
+        if (n_experts <= 64)                                                                                             \
+            launch_kernel(router_tile_kernel<WT, TT, 1>, grid, block, lds, s, x, w, n, hidden, n_experts, k, flavour, norm, logits, \
+                          ids, weights, hits, flags, xq);                                                                \
+        else                                                                                                             \
+            launch_kernel(router_tile_kernel<WT, TT, 2>, grid, block, lds, s, x, w, n, hidden, n_experts, k, flavour, norm, logits, \
+                          ids, weights, hits, flags, xq);                                                                \
+        return hipGetLastError();                                                                                        \
+    } while (0)
+        switch (wtype) {
+        case T_F32: MUMMU_RT(T_F32);
+        case T_F16: MUMMU_RT(T_F16);
+        case T_BF16: MUMMU_RT(T_BF16);
+        default: return hipErrorInvalidValue;
+        }
+#undef MUMMU_RT
+    }
     const bool few = n <= 64;  // few tokens: one token per workgroup
 #define MUMMU_RB2(WT)                                                                                                   \
     do {                                                                                                                \

@@ -516,8 +516,8 @@ ORC_API int orc_route_olmoe(const float *logits, size_t n, int n_experts, int k,
  *   512 partial sums; element i goes to partial (i mod 512), partials accumulate with one
  *   fma per element in ascending i.  View the partials as 64 groups of 8 consecutive
  *   ones: each group folds as ((a0+a4)+(a1+a5))+((a2+a6)+(a3+a7)) - the reference dot's
- *   own final fold, experts.rs:473 - and the 64 group sums fold by halving:
- *   s[l] += s[l+32], then +16, +8, +4, +2, +1.
+ *   own final fold, experts.rs:473 - and the 64 group sums fold pairwise over adjacent
+ *   groups: s[l] += s[l+1] for even l, then s[l] += s[l+2] for l % 4 == 0, ... up to +32.
  *
  * The weight is converted to f32 exactly (F32/F16/BF16) before the fma.
  * ---------------------------------------------------------------------------------- */
@@ -541,8 +541,8 @@ ORC_API float orc_router_dot(const float *x, const void *w, int wtype, size_t ro
         const float *a = acc + l * 8;
         s[l] = ((a[0] + a[4]) + (a[1] + a[5])) + ((a[2] + a[6]) + (a[3] + a[7]));
     }
-    for (int off = 32; off >= 1; off >>= 1)
-        for (int l = 0; l < off; l++) s[l] = s[l] + s[l + off];
+    for (int off = 1; off < 64; off <<= 1) /* pairwise tree over adjacent lane sums */
+        for (int l = 0; l < 64; l += 2 * off) s[l] = s[l] + s[l + off];
     return s[0];
 }
 

@@ -74,11 +74,11 @@ def py_router_dot(x, w):
     for l in range(64):
         a = [f(v) for v in acc[l * 8:l * 8 + 8]]
         s.append(f(f(f(a[0] + a[4]) + f(a[1] + a[5])) + f(f(a[2] + a[6]) + f(a[3] + a[7]))))
-    off = 32
-    while off >= 1:
-        for l in range(off):
+    off = 1
+    while off < 64:  # pairwise tree over adjacent group sums
+        for l in range(0, 64, 2 * off):
             s[l] = f(s[l] + s[l + off])
-        off //= 2
+        off *= 2
     return s[0]
 
 
