@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
 # same command (profiles/olmoe_q4k_decode_hbm_traffic.txt), each scaled by what the counter
 # reads for the library's 256 MiB copy kernel.  Only for the workload/batch they were taken on.
-PROFILED_TRAFFIC = {}
+PROFILED_TRAFFIC = {("olmoe_q4k_decode", 1, "gate_up"): 19173630}
 
 WORKLOADS = {
     # name: (hidden, inter, experts, top_k, norm, bank type, router type)
@@ -182,7 +182,7 @@ def main() -> int:
     per_kernel_us = {name: (tot / cnt * 1e3 if cnt else None) for name, (tot, cnt) in kt.items()}
     layer_bytes = mean_distinct * expert_bytes + router_bytes + n * H * 8
     # the dominant kernel and the bytes one launch of it has to move
-    kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes,
+    kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes + n * E * 4,
                     "down_combine": mean_distinct * (expert_bytes - gate_up_expert_bytes),
                     "gemm_gate_up": mean_distinct * gate_up_expert_bytes}
     timed = {name: us for name, us in per_kernel_us.items() if us is not None and name in kernel_bytes}

@@ -27,6 +27,7 @@
 #include "device_utils.h"
 #include "kernels.h"
 #include "gemv_common.h"
+#include "route_common.h"
 
 MUMMU_TRACE_UNIT(experts)
 
@@ -39,25 +40,45 @@ constexpr int kGemvWaves = 4;  // waves per workgroup of the float kernels
 // rows_per_block = waves*NIT*rows_per_it output rows are a whole number of 16-element
 // activation blocks, quantized for the down projection in the epilogue.
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int NIT, bool ACTQ>
+template <int WT, int UPL, int NIT, bool ACTQ, bool ROUTE = false>
 __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restrict__ gate,
                                                          const uint8_t *__restrict__ up, QAct xq,
                                                          const int32_t *__restrict__ ids, int k, int fixed_expert,
                                                          int hidden, int inter, int n_experts,
                                                          float *__restrict__ act, QAct actq,
-                                                         int32_t *__restrict__ flags) {
+                                                         int32_t *__restrict__ flags, RouteInline route) {
     extern __shared__ float s_act[];  // rows_per_block floats
+    __shared__ __attribute__((aligned(16))) RouteScratch<1> s_route;
+    __shared__ int s_ids[64];
+    __shared__ float s_w[64];
     MUMMU_PHASE(0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.z;  // grid = (slot, row tile, token)
     const int a = t * gridDim.x + blockIdx.x;
-    const int e = fixed_expert >= 0 ? fixed_expert : ids[a];
+    const RowSplit rs = row_split(hidden);
+    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
+    LaneAct<UPL> la;  // the token's activations do not depend on the routing: fetch them first
+    load_lane_act<WT, UPL>(xq, (size_t)t, hidden, unit0, rs.units, la);
+    if (ROUTE) {
+        // wave 0 routes token t from its logits; everybody else already has the activations coming
+        if (wave == 0) {
+            float l[1] = {lane < n_experts ? route.logits[(size_t)t * n_experts + lane] : 0.0f};
+            route_token<1>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
+            wave_lds_sync();
+            if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
+                const int id = s_ids[lane];
+                route.ids[(size_t)t * k + lane] = id;
+                route.weights[(size_t)t * k + lane] = s_w[lane];
+                if (route.hits) atomicAdd(&route.hits[id], 1ULL);
+            }
+        }
+        __syncthreads();
+    }
+    const int e = ROUTE ? s_ids[blockIdx.x] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
     if ((unsigned)e >= (unsigned)n_experts) {
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
     }
-    const RowSplit rs = row_split(hidden);
-    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
     const int rows_per_wave = NIT * rs.rows_per_it;
     const int rows_per_block = rows_per_wave * (blockDim.x >> 6);
     const int block_row0 = blockIdx.y * rows_per_block;
@@ -66,22 +87,30 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     const uint8_t *ge = gate + (size_t)e * (size_t)inter * row_bytes;
     const uint8_t *ue = up + (size_t)e * (size_t)inter * row_bytes;
 
-    LaneAct<UPL> la;
-    load_lane_act<WT, UPL>(xq, (size_t)t, hidden, unit0, rs.units, la);
+    // Software pipeline over the wave's NIT row iterations: the loads of iterations i+1 and i+2
+    // are in flight while iteration i is multiplied, so the integer dots run under the stream
+    // instead of after it (the scheduling barriers keep the compiler from hoisting every load
+    // to the top, where a wave would sit blocked on issue until most of its data had arrived).
     RawRow<WT, UPL> rg[NIT], ru[NIT];
-#pragma unroll
-    for (int i = 0; i < NIT; i++) {
+    auto fetch = [&](int i) {
         const int row = row0 + i * rs.rows_per_it + sub;
         const bool ok = row < inter;
         load_row<WT, UPL>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
         load_row<WT, UPL>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
-    }
+    };
+    constexpr int AHEAD = NIT < 2 ? NIT : 2;
+#pragma unroll
+    for (int i = 0; i < AHEAD; i++) fetch(i);
+    __builtin_amdgcn_sched_barrier(0);
     MUMMU_PHASE(1);
     float part[2 * NIT];
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
+        if (i + AHEAD < NIT) fetch(i + AHEAD);
+        __builtin_amdgcn_sched_barrier(0);
         part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
         part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
+        __builtin_amdgcn_sched_barrier(0);
     }
     MUMMU_PHASE(2);
     dispatch_group(rs.group, [&](auto group_tag) {
@@ -285,24 +314,31 @@ __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
     }
 
     MUMMU_PHASE(1);
+    // same software pipeline as gate/up, over the wave's KPW*NIT (expert, row iteration) steps
     RawRow<WT, UPL> rd[KPW][NIT];
     LaneAct<UPL> la[KPW];
-#pragma unroll
-    for (int i = 0; i < KPW; i++) {
+    auto fetch = [&](int step) {
+        const int i = step / NIT, it = step % NIT;
         const uint8_t *de = down + (size_t)(on_p[i] ? e_p[i] : 0) * (size_t)hidden * row_bytes;
+        const int row = row0 + it * rs.rows_per_it + sub;
+        const bool ok = on_p[i] && row < hidden;
+        load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i][it]);
+    };
+    constexpr int STEPS = KPW * NIT;
+    constexpr int AHEAD = STEPS < 2 ? STEPS : 2;
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            const int row = row0 + it * rs.rows_per_it + sub;
-            const bool ok = on_p[i] && row < hidden;
-            load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i][it]);
-        }
-        load_lane_act<WT, UPL>(actq, (size_t)(on_p[i] ? a_p[i] : 0), inter, unit0, rs.units, la[i]);
-    }
+    for (int i = 0; i < KPW; i++) load_lane_act<WT, UPL>(actq, (size_t)(on_p[i] ? a_p[i] : 0), inter, unit0, rs.units, la[i]);
+#pragma unroll
+    for (int st = 0; st < AHEAD; st++) fetch(st);
+    __builtin_amdgcn_sched_barrier(0);
     float part[KPW * NIT];
 #pragma unroll
-    for (int i = 0; i < KPW; i++)
-#pragma unroll
-        for (int it = 0; it < NIT; it++) part[i * NIT + it] = dot_row<WT, UPL>(rd[i][it], unit0, la[i]);
+    for (int st = 0; st < STEPS; st++) {
+        if (st + AHEAD < STEPS) fetch(st + AHEAD);
+        __builtin_amdgcn_sched_barrier(0);
+        part[st] = dot_row<WT, UPL>(rd[st / NIT][st % NIT], unit0, la[st / NIT]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     MUMMU_PHASE(2);
     dispatch_group(rs.group, [&](auto group_tag) {
         constexpr int GROUP = decltype(group_tag)::value;
@@ -360,10 +396,10 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         const size_t lds = sizeof(float) * (size_t)rpb;                                                         \
         if (actq_out)                                                                                           \
             launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true>, grid, block, lds, s,                                       \
-                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags);      \
+                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags, RouteInline());      \
         else                                                                                                    \
             launch_kernel(gate_up_q_kernel<WT, UPL, NIT, false>, grid, block, lds, s,                                      \
-                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags);      \
+                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags, RouteInline());      \
     } while (0)
         if (upl == 1) MUMMU_GUQ(1, 4);
         else if (upl == 2) MUMMU_GUQ(2, 2);
@@ -402,6 +438,32 @@ hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const i
     case T_Q4_K: return launch_gate_up_t<T_Q4_K>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
     default: return hipErrorInvalidValue;
     }
+}
+
+bool gate_up_routes_inline(const ExpertBanks &b, int k) {
+    const RowSplit rs = row_split(b.hidden);
+    return is_quant_type(b.gate_type) && b.gate_type == b.up_type && is_quant_type(b.down_type) && rs.units <= 64 &&
+           b.n_experts <= 64 && k >= 1 && k <= b.n_experts && k <= 64 && b.inter % 16 == 0;
+}
+
+hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInline &route, int n_tokens, int k, QAct actq,
+                                 int32_t *flags, hipStream_t s) {
+    if (n_tokens <= 0) return hipSuccess;
+    if (!gate_up_routes_inline(b, k) || n_tokens > 65535) return hipErrorInvalidValue;
+    const RowSplit rs = row_split(b.hidden);
+    constexpr int NIT = 4;
+    int waves = 4;
+    while (waves * NIT * rs.rows_per_it < 16) waves *= 2;
+    const int rpb = waves * NIT * rs.rows_per_it;
+    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(64 * waves);
+    const size_t lds = sizeof(float) * (size_t)rpb;
+    if (b.gate_type == T_Q4_K)
+        launch_kernel(gate_up_q_kernel<T_Q4_K, 1, NIT, true, true>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, k,
+                      -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route);
+    else
+        launch_kernel(gate_up_q_kernel<T_Q8_0, 1, NIT, true, true>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, k,
+                      -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route);
+    return hipGetLastError();
 }
 
 template <int WT>

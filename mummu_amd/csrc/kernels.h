@@ -51,6 +51,21 @@ inline bool is_quant_type(int t) { return t == 8 || t == 12; }
 // is quantized, else act (f32).
 hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const int32_t *ids, int n_assign, int k,
                           int fixed_expert, float *act, QAct actq, int32_t *flags, hipStream_t s);
+// gate/up that routes by itself: every workgroup of token t turns the token's router logits into
+// the routing (same arithmetic as route_topk, so the same bits in every workgroup) instead of
+// waiting for a separate launch to publish it; the workgroup of (slot 0, row tile 0) writes
+// ids / weights / hit counters for the kernels that follow.  Quantized gate/up banks feeding a
+// quantized down bank, hidden <= 2048, at most 64 experts.
+struct RouteInline {
+    const float *logits = nullptr;  // [n, n_experts]
+    int flavour = 0, norm = 0;
+    int32_t *ids = nullptr;         // [n, k] out
+    float *weights = nullptr;       // [n, k] out
+    unsigned long long *hits = nullptr;
+};
+bool gate_up_routes_inline(const ExpertBanks &b, int k);
+hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInline &route, int n_tokens, int k, QAct actq,
+                                 int32_t *flags, hipStream_t s);
 // y[a, c] = <down_e[c,:], act[a,:]>   (actq for a quantized down bank, else act)
 hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign, int k,
                        int fixed_expert, float *y, hipStream_t s);

@@ -297,6 +297,20 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     } else {
         // few tokens: the router rows are spread over as many CUs as there are experts
         LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s));
+        const ExpertBanks b = banks_of(h, L);
+        if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
+            // ... and the gate/up kernel routes by itself: one launch less on the decode path
+            RouteInline route;
+            route.logits = h->logits;
+            route.flavour = h->cfg.router_flavour;
+            route.norm = norm;
+            route.ids = h->ids;
+            route.weights = h->weights;
+            route.hits = L.hits;
+            LAUNCH(h, K_GATE_UP, s, launch_gate_up_routed(b, h->xq, route, (int)n, k, h->actq, h->flags, s));
+            LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, k, residual, out, s));
+            return MUMMU_OK;
+        }
         LAUNCH(h, K_ROUTE_TOPK, s,
                launch_route_topk(h->logits, (int)n, E, k, h->cfg.router_flavour, norm, h->ids, h->weights, L.hits, h->flags, s));
     }

@@ -70,8 +70,9 @@ template <int JN>
 __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts, int k, int flavour, int norm,
                                    int32_t *__restrict__ ids, float *__restrict__ weights,
                                    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags,
-                                   RouteScratch<JN> &sc) {
+                                   RouteScratch<JN> &sc, int out_row = -1) {
     const int lane = threadIdx.x & 63;
+    const size_t orow = out_row < 0 ? (size_t)t : (size_t)out_row;  // row of ids / weights this token's routing goes to
     float p[JN];
     bool bad = false;
     float mx = -__builtin_inff();
@@ -91,8 +92,8 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         // the kernels downstream stay inside their buffers; the host reports the error.
         if (lane == 0) atomicAdd(&flags[FLAG_NONFINITE], 1);
         for (int s = lane; s < k; s += 64) {
-            ids[(size_t)t * k + s] = s;
-            weights[(size_t)t * k + s] = 0.0f;
+            ids[orow * k + s] = s;
+            weights[orow * k + s] = 0.0f;
         }
         return;
     }
@@ -212,8 +213,8 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         float wv = sc.w[s];
         const int id = sc.id[s];
         if (divide) wv = __fdiv_rn(wv, denom);
-        ids[(size_t)t * k + s] = id;
-        weights[(size_t)t * k + s] = wv;
+        ids[orow * k + s] = id;
+        weights[orow * k + s] = wv;
         if (hits) atomicAdd(&hits[id], 1ULL);
     }
 }
