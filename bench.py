@@ -192,6 +192,15 @@ def main() -> int:
     achieved = gu_bytes / (gu_us * 1e-6) / 1e9 if gu_us else None
 
     layer_gbs = layer_bytes / (ms_per_step * 1e-3) / 1e9
+    # batched calls: matrix-core rate of the two grouped GEMMs (2*H*I flops per assignment and projection)
+    mfma = None
+    if per_kernel_us.get("gemm_gate_up") and per_kernel_us.get("gemm_down"):
+        peak = 2500.0 if w["bank"] == "F16" else 5000.0  # dense f16 TFLOP/s, int8 TOP/s
+        gu_t = n * k * 2 * 2 * H * I / (per_kernel_us["gemm_gate_up"] * 1e-6) / 1e12
+        dn_t = n * k * 2 * H * I / (per_kernel_us["gemm_down"] * 1e-6) / 1e12
+        mfma = {"unit": "TFLOP/s" if w["bank"] == "F16" else "TOP/s", "peak": peak, "gemm_gate_up": round(gu_t, 1),
+                "gemm_down": round(dn_t, 1), "gemm_gate_up_frac": round(gu_t / peak, 4), "gemm_down_frac": round(dn_t / peak, 4),
+                "hbm_floor_us": round(layer_bytes / (HBM_PEAK_GBS * 1e3), 1)}
 
     out = {
         "metric": "MoE-layer tokens/s + achieved HBM GB/s (Q4_K, OLMoE shape, 1 GPU)",
@@ -222,6 +231,7 @@ def main() -> int:
                      "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
                      "traffic": PROFILED_TRAFFIC.get((args.workload, n, dom)),
                      "algorithmic_bytes_per_launch": int(gu_bytes), "avg_launch_us": round(gu_us, 3) if gu_us else None},
+        "mfma": mfma,
         "device": M.device_name(),
         "setup_s": round(setup_s, 1),
     }

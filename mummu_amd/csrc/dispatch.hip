@@ -12,7 +12,9 @@
 //   count   per chunk: every assignment's rank among the chunk's assignments to the same expert
 //           (wave ballots, then a prefix over the workgroup's 16 waves in LDS) and the chunk's
 //           per-expert counts
-//   scan    one workgroup: per expert the running count over chunks and the total, the exclusive
+//   scan    one workgroup: per expert the running count over chunks and the total (also added to
+//           the layer's hit counters when asked: 8 atomics per token from the router would all
+//           land on the same few cache lines), the exclusive
 //           scan over experts (offsets), and the grouped GEMM's work list of
 //           (expert, first sorted position, rows <= tile_rows) triples - every expert writes its
 //           own tiles at the position an exclusive scan of the tile counts gives it
@@ -79,7 +81,8 @@ __global__ __launch_bounds__(kDispatchMaxExperts) void dispatch_scan_kernel(int3
                                                                             int n_experts, int tile_rows,
                                                                             int32_t *__restrict__ offsets,
                                                                             int32_t *__restrict__ tiles,
-                                                                            int32_t *__restrict__ n_tiles) {
+                                                                            int32_t *__restrict__ n_tiles,
+                                                                            unsigned long long *__restrict__ hits) {
     __shared__ int s_carry[kDispatchMaxExperts / 64][2];
     const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
     int total = 0;
@@ -114,6 +117,7 @@ __global__ __launch_bounds__(kDispatchMaxExperts) void dispatch_scan_kernel(int3
     }
     const int begin = base + incl - total;
     if (e < n_experts) {
+        if (hits) hits[e] += (unsigned long long)total;  // rows served per expert (nn/moe.rs:1562-1564)
         offsets[e] = begin;
         if (e == n_experts - 1) offsets[n_experts] = begin + total;
         if (tiles != nullptr) {
@@ -151,7 +155,7 @@ size_t dispatch_scratch_ints(int n_assign, int n_experts) {
 
 hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int tile_rows, int32_t *offsets,
                            int32_t *sorted, int32_t *inv, int32_t *tiles, int32_t *n_tiles, int32_t *scratch,
-                           int32_t *flags, hipStream_t s) {
+                           unsigned long long *hits, int32_t *flags, hipStream_t s) {
     if (n_assign <= 0) return hipSuccess;
     if (n_experts > kDispatchMaxExperts || tile_rows < 1) return hipErrorInvalidValue;
     const int chunks = (n_assign + kDispatchThreads - 1) / kDispatchThreads;
@@ -163,7 +167,7 @@ hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int 
                   flags);
     g_launch_timing.start = nullptr;
     launch_kernel(dispatch_scan_kernel, dim3(1), dim3(kDispatchMaxExperts), 0, s, counts, chunks, n_experts, tile_rows,
-                  offsets, tiles, n_tiles);
+                  offsets, tiles, n_tiles, hits);
     g_launch_timing.stop = timing.stop;
     launch_kernel(dispatch_place_kernel, dim3(chunks), dim3(kDispatchThreads), 0, s, ids, n_assign, n_experts,
                   (const int32_t *)rank, (const int32_t *)counts, (const int32_t *)offsets, sorted, inv);

@@ -31,6 +31,8 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int16v __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // staging registers: first-class vectors stay in VGPRs
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBN = 128;            // output rows per workgroup
 constexpr int kBK = 64;             // K step
@@ -53,17 +55,21 @@ __host__ __device__ inline size_t gemm_row_bytes(int type, int in_dim) {
 // (row 8*(r/4) + 4*(l/32) + r%4, column l%32) of the wave's 32x32 tile.
 __device__ inline int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 
-// Work-list entry of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin by their
-// linear id, and the grid's x extent is a multiple of 8, so workgroup x lands on XCD x % 8 for
-// every y.  Giving XCD j the contiguous run of tiles [j*ceil(T/8), (j+1)*ceil(T/8)) puts the
-// tiles of one expert (neighbours in the list) on the same XCD at about the same time - they
-// share that expert's weight slab in one L2 instead of pulling it into all eight - and keeps a
-// token tile on one XCD across the output slabs y.
-__device__ inline int xcd_tile(const int32_t *__restrict__ n_tiles) {
+// Work-list entry (tile, output slab) of this workgroup of a 1-D grid.  Workgroups are dealt to
+// the 8 XCDs round-robin by their linear id, each XCD with its own L2.  XCD j gets the contiguous
+// run of tiles [j*ceil(T/8), (j+1)*ceil(T/8)) and walks it tile by tile with the slab index
+// running fastest, so the workgroups resident on an XCD at any time are a few neighbouring tiles
+// (the same expert, mostly) times all output slabs: the slabs of a tile share its activation rows
+// in that L2 and the tiles of an expert share its weight slabs, instead of every L2 streaming
+// everything.
+__device__ inline bool xcd_tile(const int32_t *__restrict__ n_tiles, int slabs, int &tile, int &slab) {
     const int total = *n_tiles;
     const int per_xcd = (total + 7) >> 3;
-    const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    return ((int)(blockIdx.x >> 3) < per_xcd && tile < total) ? tile : -1;
+    const int xcd = (int)(blockIdx.x & 7), i = (int)(blockIdx.x >> 3);
+    slab = i % slabs;
+    const int local = i / slabs;
+    tile = xcd * per_xcd + local;
+    return local < per_xcd && tile < total;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -84,10 +90,10 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     __shared__ __attribute__((aligned(16))) _Float16 s_a[BM][kLds];
     __shared__ __attribute__((aligned(16))) _Float16 s_b[NB][kBN][kLds];
 
-    const int tile = xcd_tile(n_tiles);
-    if (tile < 0) return;
+    int tile, slab;
+    if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
     const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
-    const int n0 = blockIdx.y * kBN;
+    const int n0 = slab * kBN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t row_bytes = (size_t)in_dim * 2;
 
@@ -107,19 +113,20 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     // f16 source -> 8 threads per row, 8 elements each (MT passes of 32 rows)
     constexpr int A_PASSES = GATE_UP ? 2 * MT : MT;
     const int a_col = GATE_UP ? (tid & 15) * 4 : (tid & 7) * 8;
+    // rows past the tile's end read the tile's last row: their products are never stored
     const float *a_src32[A_PASSES];
     const _Float16 *a_src16[A_PASSES];
     int a_row[A_PASSES];
 #pragma unroll
     for (int p = 0; p < A_PASSES; p++) {
         a_row[p] = GATE_UP ? p * 16 + (tid >> 4) : p * 32 + (tid >> 3);
-        const bool ok = a_row[p] < rows;
+        const int r = a_row[p] < rows ? a_row[p] : rows - 1;
         if (GATE_UP) {
-            const int a = ok ? sorted[p0 + a_row[p]] : 0;
-            a_src32[p] = ok ? x + (size_t)(a / k_slots) * (size_t)in_dim + a_col : nullptr;
+            const int a = sorted[p0 + r];
+            a_src32[p] = x + (size_t)(a / k_slots) * (size_t)in_dim + a_col;
             a_src16[p] = nullptr;
         } else {
-            a_src16[p] = ok ? act_in + (size_t)(p0 + a_row[p]) * (size_t)in_dim + a_col : nullptr;
+            a_src16[p] = act_in + (size_t)(p0 + r) * (size_t)in_dim + a_col;
             a_src32[p] = nullptr;
         }
     }
@@ -132,43 +139,53 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
 
-    uint4 rb[NB][4];
-    float4 ra32[A_PASSES];
-    uint4 ra16[A_PASSES];
+    u32x4 rb[NB][4];
+    f32x4 ra32[A_PASSES];
+    u32x4 ra16[A_PASSES];
     auto fetch = [&](int k0) {
 #pragma unroll
         for (int b = 0; b < NB; b++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) rb[b][i] = *(const uint4 *)(b_ptr[b][i] + (size_t)k0 * 2);
+            for (int i = 0; i < 4; i++) rb[b][i] = *(const u32x4 *)(b_ptr[b][i] + (size_t)k0 * 2);
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) {
-            if (GATE_UP) ra32[p] = a_src32[p] ? *(const float4 *)(a_src32[p] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
-            else ra16[p] = a_src16[p] ? *(const uint4 *)(a_src16[p] + k0) : make_uint4(0, 0, 0, 0);
+            if (GATE_UP) ra32[p] = *(const f32x4 *)(a_src32[p] + k0);
+            else ra16[p] = *(const u32x4 *)(a_src16[p] + k0);
         }
     };
-    fetch(0);
+    // The K loop starts at a slab-dependent step and wraps.  An f16 row of 2048 elements is 4096
+    // bytes - the period of the memory channel interleave - so one K step of ALL rows lives in one
+    // channel, and with every workgroup of the chip marching through K in lockstep the whole
+    // launch would queue on one or two channels at a time.  Rotating by slab spreads the slabs
+    // over the channels; a token's result still depends only on its output slab, never on which
+    // tile or batch it arrived in.
+    const int n_steps = in_dim / kBK;
+    const int n_slabs = (out_dim + kBN - 1) / kBN;
+    const int rot = (slab * (n_steps / n_slabs > 0 ? n_steps / n_slabs : 1)) % n_steps;
+    auto step_k0 = [&](int step) { return ((step + rot) % n_steps) * kBK; };
+    fetch(step_k0(0));
 
     MUMMU_TIMER_DECL;
-    for (int k0 = 0; k0 < in_dim; k0 += kBK) {
+    for (int step = 0; step < n_steps; step++) {
         MUMMU_TIMER_MARK(0);
         // registers -> LDS
 #pragma unroll
         for (int b = 0; b < NB; b++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) *(uint4 *)&s_b[b][(tid >> 3) + 32 * i][b_chunk * 8] = rb[b][i];
+            for (int i = 0; i < 4; i++) *(u32x4 *)&s_b[b][(tid >> 3) + 32 * i][b_chunk * 8] = rb[b][i];
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) {
             if (GATE_UP) {
                 uint2 v = make_uint2(pack_half2(ra32[p].x, ra32[p].y), pack_half2(ra32[p].z, ra32[p].w));
                 *(uint2 *)&s_a[a_row[p]][a_col] = v;
             } else {
-                *(uint4 *)&s_a[a_row[p]][a_col] = ra16[p];
+                *(u32x4 *)&s_a[a_row[p]][a_col] = ra16[p];
             }
         }
         MUMMU_TIMER_MARK(1);
         __syncthreads();
         MUMMU_TIMER_MARK(2);
-        if (k0 + kBK < in_dim) fetch(k0 + kBK);
+        if (step + 1 < n_steps) fetch(step_k0(step + 1));
         MUMMU_TIMER_MARK(3);
         // multiply: wave owns columns 32*wave .. +31
 #pragma unroll
@@ -308,10 +325,10 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
     auto s_a = [&](int plane, int row) -> uint8_t * { return s_raw + ((size_t)plane * BM + row) * kLdsQ; };
     auto s_b = [&](int b, int row) -> uint8_t * { return s_raw + L::kA + ((size_t)b * kBN + row) * kLdsQ; };
 
-    const int tile = xcd_tile(n_tiles);
-    if (tile < 0) return;
+    int tile, slab;
+    if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
     const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
-    const int n0 = blockIdx.y * kBN;
+    const int n0 = slab * kBN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t row_bytes = gemm_row_bytes(WT, in_dim);
 
@@ -495,7 +512,7 @@ template <int WT, bool GATE_UP>
 static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_in, const int32_t *sorted, int k_slots,
                                 const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
                                 int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
-    dim3 block(256), grid((max_tiles + 7) / 8 * 8, (out_dim + kBN - 1) / kBN);
+    dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
     if (tile_rows == 64)
         launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, 2>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                      out_dim, act_out, y_out);
@@ -510,7 +527,7 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const fl
                                   const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
                                   int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
                                   hipStream_t s) {
-    dim3 block(256), grid((max_tiles + 7) / 8 * 8, (out_dim + kBN - 1) / kBN);
+    dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
     if (tile_rows == 64)
         launch_kernel(grouped_gemm_f16_kernel<GATE_UP, 2>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
                                                                    out_dim, act_out, y_out);

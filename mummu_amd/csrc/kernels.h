@@ -84,11 +84,12 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
 // Stable counting sort of the assignments by expert (ranks, histograms and scans in LDS, three
 // small launches): offsets[E+1], sorted[A] (position -> assignment), inv[A] (assignment ->
 // position) and the grouped GEMM's work list of (expert, first position, rows <= tile_rows)
-// triples.  scratch: dispatch_scratch_ints(A, E) ints.
+// triples.  scratch: dispatch_scratch_ints(A, E) ints.  hits (optional): per-expert row counters to
+// add this batch to.
 size_t dispatch_scratch_ints(int n_assign, int n_experts);
 hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int tile_rows, int32_t *offsets,
                            int32_t *sorted, int32_t *inv, int32_t *tiles, int32_t *n_tiles, int32_t *scratch,
-                           int32_t *flags, hipStream_t s);
+                           unsigned long long *hits, int32_t *flags, hipStream_t s);
 
 // gemm.hip ----------------------------------------------------------------------------
 // Grouped GEMMs over the dispatch-sorted assignments on the matrix cores (hidden and inter

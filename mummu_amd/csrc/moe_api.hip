@@ -250,7 +250,7 @@ int check_topk(mummu_moe *h, int top_k, int n_experts) {
 // experts of an already-made routing: gate/up -> down -> combine.  x_quantized says h->xq
 // already holds the 16-bit form of x (the fused router produced it).
 int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, int64_t n, int k, const float *residual,
-                float *out, hipStream_t s) {
+                float *out, hipStream_t s, bool count_hits = false) {
     ExpertBanks b = banks_of(h, L);
     const int na = (int)(n * k);
     if (n >= h->gemm_min_tokens && grouped_gemm_supported(b)) {
@@ -261,7 +261,8 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
         if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
         LAUNCH(h, K_DISPATCH, s,
-               launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch, h->flags, s));
+               launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch,
+                               count_hits ? L.hits : nullptr, h->flags, s));
         LAUNCH(h, K_GEMM_GATE_UP, s,
                launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, actq64, s));
         LAUNCH(h, K_GEMM_DOWN, s,
@@ -291,9 +292,11 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     const QAct xq = want_xq ? h->xq : QAct();
     if (n > 8 && router_fused_supported(E)) {
         // many tokens: one workgroup per token tile does logits, routing and quantization
+        // on the batched path the dispatch adds the per-expert row counts to the hit counters
         LAUNCH(h, K_ROUTER, s,
                launch_router_fused(x, L.router, L.router_type, (int)n, H, E, k, h->cfg.router_flavour, norm, h->logits,
-                                   h->ids, h->weights, L.hits, h->flags, xq, s));
+                                   h->ids, h->weights, batched ? nullptr : L.hits, h->flags, xq, s));
+        return run_experts(h, L, x, want_xq, n, k, residual, out, s, batched);
     } else {
         // few tokens: the router rows are spread over as many CUs as there are experts
         LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s));

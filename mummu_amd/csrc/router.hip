@@ -246,53 +246,88 @@ __global__ __launch_bounds__(64 * kRouterWaves) void router_block_kernel(
     MUMMU_PHASE(3);
 }
 
-constexpr int kRouterMaxChunks = 4;  // 512-element chunks of a row held in registers: hidden <= 2048 on the tiled path
+constexpr int kRouterMaxChunks = 4;  // 512-element chunks of a row held in registers: hidden <= 2048 on the streaming path
 
-// Tiled form (hidden <= 2048, a multiple of 8): the tile's activation rows are staged in LDS
-// once and every wave walks its experts with the lane's slice of the weight row in registers
-// (lane l owns elements 8l..8l+7 of each 512-chunk, i.e. partials 8l..8l+7), so a weight row is
-// read once per tile and an activation row once per workgroup.  Same summation order as
-// router_logits_kernel.
-template <int WT, int TT, int JN>
-__global__ __launch_bounds__(64 * kRouterWaves) void router_tile_kernel(
+// Streaming form (hidden = CHUNKS*512 <= 2048) for large batches: one wave owns TT tokens, keeps
+// the lane's slices of their activation rows in registers (lane l owns elements 8l..8l+7 of each
+// 512-chunk, i.e. partials 8l..8l+7) and walks all experts, the next weight row already in
+// flight while the current one is multiplied.  The wave-wide sum leaves logit e in lane e%64, which
+// is the layout the routing step wants, so nothing goes through LDS but the routing scratch and
+// nothing waits on another wave.  Same summation order as router_logits_kernel.
+constexpr int kStreamWaves = 4;
+
+template <int WT, int TT, int JN, int CHUNKS>
+__global__ __launch_bounds__(64 * kStreamWaves) void router_stream_kernel(
     const float *__restrict__ x, const void *__restrict__ w, int n, int hidden, int n_experts, int k, int flavour,
     int norm, float *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ weights,
-    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags, QAct xq) {
-    extern __shared__ __attribute__((aligned(16))) float s_x[];  // [TT][hidden]
-    __shared__ float s_logits[TT][64 * JN];
-    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[TT];
+    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[kStreamWaves];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int t0 = blockIdx.x * TT;
-    const int tile_tokens = (n - t0) < TT ? (n - t0) : TT;
-    const int chunks = (hidden + 511) / 512;
+    const int t0 = (blockIdx.x * kStreamWaves + wave) * TT;
+    if (t0 >= n) return;
+    MUMMU_PHASE(0);
 
-    // stage the tile (rows past the batch are zero) and quantize it where the expert kernels want that
-    for (int i = threadIdx.x * 4; i < TT * hidden; i += 64 * kRouterWaves * 4) {
-        const int t = i / hidden;
-        const float4 v = t < tile_tokens ? *(const float4 *)(x + (size_t)t0 * (size_t)hidden + i) : make_float4(0.f, 0.f, 0.f, 0.f);
-        *(float4 *)(s_x + i) = v;
-    }
-    if (xq.hi != nullptr) {
-        const int slices_per_row = hidden / 64;
-        for (int sl = wave; sl < tile_tokens * slices_per_row; sl += kRouterWaves) {
-            const int t = t0 + sl / slices_per_row;
-            const int elem = (sl % slices_per_row) * 64 + lane;
-            quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
+    float xv[TT][CHUNKS][8];
+#pragma unroll
+    for (int t = 0; t < TT; t++) {
+        const int tok = t0 + t < n ? t0 + t : n - 1;  // a ragged last group repeats its last token
+#pragma unroll
+        for (int c = 0; c < CHUNKS; c++) {
+            const float4 *p = (const float4 *)(x + (size_t)tok * (size_t)hidden + c * 512 + lane * 8);
+            const float4 a = p[0], b = p[1];
+            xv[t][c][0] = a.x; xv[t][c][1] = a.y; xv[t][c][2] = a.z; xv[t][c][3] = a.w;
+            xv[t][c][4] = b.x; xv[t][c][5] = b.y; xv[t][c][6] = b.z; xv[t][c][7] = b.w;
         }
     }
-    __syncthreads();
-
-    for (int e = wave; e < n_experts; e += kRouterWaves) {
-        float wv[kRouterMaxChunks][8];
+    // the lane's slice of a weight row, as stored (f32: two 16-byte words per chunk, 16-bit types: one)
+    constexpr int WORDS = WT == T_F32 ? 2 : 1;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 raw[CHUNKS][WORDS], cur[CHUNKS][WORDS];
+    auto fetch_row = [&](int e) {
 #pragma unroll
-        for (int c = 0; c < kRouterMaxChunks; c++) {
-            const int base = c * 512 + lane * 8;
-            if (c < chunks && base < hidden) {
-                load_w8<WT>(w, (size_t)e * (size_t)hidden + (size_t)base, wv[c]);
+        for (int c = 0; c < CHUNKS; c++) {
+            // past the last expert the row of expert 0 is read and never used
+            const size_t at = (size_t)(e < n_experts ? e : 0) * (size_t)hidden + (size_t)(c * 512 + lane * 8);
+            const u32x4 *src = (const u32x4 *)((const uint8_t *)w + at * (WT == T_F32 ? 4 : 2));
+#pragma unroll
+            for (int i = 0; i < WORDS; i++) raw[c][i] = src[i];
+        }
+    };
+    float l[TT][JN];
+#pragma unroll
+    for (int t = 0; t < TT; t++)
+#pragma unroll
+        for (int j = 0; j < JN; j++) l[t][j] = 0.0f;
+
+    fetch_row(0);
+    MUMMU_PHASE(1);
+    for (int e = 0; e < n_experts; e++) {
+        // take over the row that was in flight, start the next one, and only then touch the data:
+        // the scheduling barriers keep the compiler from sinking the new loads' first use up here
+#pragma unroll
+        for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+            for (int i = 0; i < WORDS; i++) cur[c][i] = raw[c][i];
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_row(e + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        float wv[CHUNKS][8];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; c++) {
+            if constexpr (WT == T_F32) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    wv[c][q] = __uint_as_float(cur[c][0][q]);
+                    wv[c][4 + q] = __uint_as_float(cur[c][1][q]);
+                }
             } else {
 #pragma unroll
-                for (int j = 0; j < 8; j++) wv[c][j] = 0.0f;
+                for (int q = 0; q < 4; q++) {
+                    const uint16_t lo = (uint16_t)(cur[c][0][q] & 0xFFFFu), hi = (uint16_t)(cur[c][0][q] >> 16);
+                    wv[c][2 * q] = WT == T_F16 ? half_bits_to_float(lo) : bf16_bits_to_float(lo);
+                    wv[c][2 * q + 1] = WT == T_F16 ? half_bits_to_float(hi) : bf16_bits_to_float(hi);
+                }
             }
         }
         float sum[TT];
@@ -300,37 +335,33 @@ __global__ __launch_bounds__(64 * kRouterWaves) void router_tile_kernel(
         for (int t = 0; t < TT; t++) {
             float acc[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) acc[j] = 0.0f;
+            for (int q = 0; q < 8; q++) acc[q] = 0.0f;
 #pragma unroll
-            for (int c = 0; c < kRouterMaxChunks; c++) {
-                const int base = c * 512 + lane * 8;
-                if (c < chunks && base < hidden) {
-                    const float4 a = *(const float4 *)(s_x + t * hidden + base), b = *(const float4 *)(s_x + t * hidden + base + 4);
-                    const float xv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            for (int c = 0; c < CHUNKS; c++)
 #pragma unroll
-                    for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(xv[j], wv[c][j], acc[j]);
-                }
-            }
+                for (int q = 0; q < 8; q++) acc[q] = __builtin_fmaf(xv[t][c][q], wv[c][q], acc[q]);
             sum[t] = __fadd_rn(__fadd_rn(__fadd_rn(acc[0], acc[4]), __fadd_rn(acc[1], acc[5])),
                                __fadd_rn(__fadd_rn(acc[2], acc[6]), __fadd_rn(acc[3], acc[7])));
         }
 #pragma unroll
-        for (int t = 0; t < TT; t++) sum[t] = wave_sum(sum[t]);  // TT independent chains
-        if (lane < TT && lane < tile_tokens) {
-            float s = sum[0];
+        for (int t = 0; t < TT; t++) {
+            sum[t] = wave_sum(sum[t]);
 #pragma unroll
-            for (int t = 1; t < TT; t++) s = lane == t ? sum[t] : s;
-            s_logits[lane][e] = s;
-            logits[(size_t)(t0 + lane) * (size_t)n_experts + (size_t)e] = s;
+            for (int j = 0; j < JN; j++) l[t][j] = (e == lane + 64 * j) ? sum[t] : l[t][j];
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();
-    for (int t = wave; t < tile_tokens; t += kRouterWaves) {
-        float l[JN];
+    MUMMU_PHASE(2);
 #pragma unroll
-        for (int j = 0; j < JN; j++) l[j] = (lane + 64 * j < n_experts) ? s_logits[t][lane + 64 * j] : 0.0f;
-        route_token<JN>(l, t0 + t, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[t]);
+    for (int t = 0; t < TT; t++) {
+        if (t0 + t >= n) break;
+#pragma unroll
+        for (int j = 0; j < JN; j++)
+            if (lane + 64 * j < n_experts) logits[(size_t)(t0 + t) * (size_t)n_experts + lane + 64 * j] = l[t][j];
+        route_token<JN>(l[t], t0 + t, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[wave]);
+        wave_lds_sync();
     }
+    MUMMU_PHASE(3);
 }
 
 template <int WT, bool VEC, int TT>
@@ -357,19 +388,34 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
     if (n_experts > 128 || k > n_experts || k < 1) return hipErrorInvalidValue;
     if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
-    // enough tokens to fill the chip tile by tile: rows staged in LDS, weights in registers
-    if (n > 64 && vec && hidden <= 512 * kRouterMaxChunks) {
-        constexpr int TT = 4;
-        dim3 block(64 * kRouterWaves), grid((n + TT - 1) / TT);
-        const size_t lds = sizeof(float) * (size_t)TT * (size_t)hidden;
+    // enough tokens to fill the chip with independent waves: activations in registers, weight
+    // rows streamed (on this path the caller quantizes x separately)
+    if (n > 64 && vec && xq.hi == nullptr && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks) {
+        // two tokens per wave once there are enough waves to keep every SIMD busy, else one
+        const int tt = n > 2048 ? 2 : 1;
+        dim3 block(64 * kStreamWaves), grid((n + tt * kStreamWaves - 1) / (tt * kStreamWaves));
+#define MUMMU_RT3(WT, JN, CH)                                                                                            \
+    do {                                                                                                                 \
+        if (tt == 2)                                                                                                     \
+            launch_kernel(router_stream_kernel<WT, 2, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
+                          logits, ids, weights, hits, flags);                                                            \
+        else                                                                                                             \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
+                          logits, ids, weights, hits, flags);                                                            \
+    } while (0)
+#define MUMMU_RT2(WT, JN)                                                                                                \
+    do {                                                                                                                 \
+        switch (hidden / 512) {                                                                                          \
+        case 1: MUMMU_RT3(WT, JN, 1); break;                                                                             \
+        case 2: MUMMU_RT3(WT, JN, 2); break;                                                                             \
+        case 3: MUMMU_RT3(WT, JN, 3); break;                                                                             \
+        default: MUMMU_RT3(WT, JN, 4); break;                                                                            \
+        }                                                                                                                \
+    } while (0)
 #define MUMMU_RT(WT)                                                                                                     \
     do {                                                                                                                 \
-        if (n_experts <= 64)                                                                                             \
-            launch_kernel(router_tile_kernel<WT, TT, 1>, grid, block, lds, s, x, w, n, hidden, n_experts, k, flavour, norm, logits, \
-                          ids, weights, hits, flags, xq);                                                                \
-        else                                                                                                             \
-            launch_kernel(router_tile_kernel<WT, TT, 2>, grid, block, lds, s, x, w, n, hidden, n_experts, k, flavour, norm, logits, \
-                          ids, weights, hits, flags, xq);                                                                \
+        if (n_experts <= 64) MUMMU_RT2(WT, 1);                                                                           \
+        else MUMMU_RT2(WT, 2);                                                                                           \
         return hipGetLastError();                                                                                        \
     } while (0)
         switch (wtype) {
@@ -379,6 +425,8 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
         default: return hipErrorInvalidValue;
         }
 #undef MUMMU_RT
+#undef MUMMU_RT2
+#undef MUMMU_RT3
     }
     const bool few = n <= 64;  // few tokens: one token per workgroup
 #define MUMMU_RB2(WT)                                                                                                   \
