@@ -91,30 +91,27 @@ struct RawRow<T_Q8_0, UPL> {
 
 template <int WT, int UPL>
 __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int units, bool ok, RawRow<WT, UPL> &r) {
+    // Every lane loads unconditionally (a lane without a unit re-reads the row's last unit, a
+    // lane of a row past the matrix reads the valid row the caller passes instead): straight-line
+    // loads keep the wait counts exact, so rows still in flight are not waited for early.  What
+    // must not count gets a zero block scale, which makes its contribution exactly 0.
 #pragma unroll
     for (int i = 0; i < UPL; i++) {
         const int u = unit0 + 64 * i;
         const bool on = ok && u < units;
+        const int uc = u < units ? u : units - 1;
         if constexpr (WT == T_Q4_K) {
-            r.hdr[i] = make_uint4(0, 0, 0, 0);
-            r.q[i] = make_uint4(0, 0, 0, 0);
-            if (on) {
-                const uint8_t *blk = rowp + (size_t)(u >> 3) * 144;
-                r.hdr[i] = *(const uint4 *)blk;
-                r.q[i] = *(const uint4 *)(blk + 16 + (u & 7) * 16);
-            }
+            const uint8_t *blk = rowp + (size_t)(uc >> 3) * 144;
+            r.hdr[i] = *(const uint4 *)blk;
+            r.q[i] = *(const uint4 *)(blk + 16 + (uc & 7) * 16);
+            r.hdr[i].x = on ? r.hdr[i].x : 0u;  // d = dmin = 0
         } else {
-            r.d[i] = 0;
+            const uint8_t *blk = rowp + (size_t)uc * 34;
+            uint16_t db;
+            __builtin_memcpy(&db, blk, 2);
+            r.d[i] = on ? (uint32_t)db : 0u;
 #pragma unroll
-            for (int w = 0; w < 8; w++) r.q[i][w] = 0;
-            if (on) {
-                const uint8_t *blk = rowp + (size_t)u * 34;
-                uint16_t db;
-                __builtin_memcpy(&db, blk, 2);
-                r.d[i] = db;
-#pragma unroll
-                for (int w = 0; w < 8; w++) __builtin_memcpy(&r.q[i][w], blk + 2 + 4 * w, 4);  // 2-byte aligned
-            }
+            for (int w = 0; w < 8; w++) __builtin_memcpy(&r.q[i][w], blk + 2 + 4 * w, 4);  // 2-byte aligned
         }
     }
 }
