@@ -506,7 +506,19 @@ bool grouped_gemm_supported(const ExpertBanks &b) {
     return (f16 || grouped_gemm_quantized(b)) && b.hidden % kBK == 0 && b.inter % kBK == 0;
 }
 
-int grouped_gemm_tile_rows(int n_assign, int n_experts) { return n_assign / n_experts > 32 ? 64 : 32; }
+// Rows per tile.  An expert with one row more than a tile holds runs a second, almost empty tile
+// that streams its whole weight slab again, so the tile is sized to hold the average expert load
+// plus its spread (binomial: about +-sqrt(avg) per expert, 3.5 sigma here) when that fits; the f16
+// kernel goes up to 128 rows, the int8 kernel (more registers per row) to 64.
+int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts) {
+    const int max_rows = grouped_gemm_quantized(b) ? 64 : 128;
+    const double avg = (double)n_assign / (double)n_experts;
+    const int want = (int)(avg + 3.5 * __builtin_sqrt(avg) + 1.0);
+    if (want > max_rows) return 64;  // several full tiles per expert whatever the size: 64 rows measured best
+    int rows = 32;
+    while (rows < want) rows += 32;
+    return rows;
+}
 
 template <int WT, bool GATE_UP>
 static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_in, const int32_t *sorted, int k_slots,
@@ -528,12 +540,17 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const fl
                                   int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
                                   hipStream_t s) {
     dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
-    if (tile_rows == 64)
-        launch_kernel(grouped_gemm_f16_kernel<GATE_UP, 2>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
-                                                                   out_dim, act_out, y_out);
-    else
-        launch_kernel(grouped_gemm_f16_kernel<GATE_UP, 1>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, in_dim,
-                                                                   out_dim, act_out, y_out);
+#define MUMMU_F16(MT)                                                                                                    \
+    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, \
+                  in_dim, out_dim, act_out, y_out)
+    switch (tile_rows) {
+    case 32: MUMMU_F16(1); break;
+    case 64: MUMMU_F16(2); break;
+    case 96: MUMMU_F16(3); break;
+    case 128: MUMMU_F16(4); break;
+    default: return hipErrorInvalidValue;
+    }
+#undef MUMMU_F16
     return hipGetLastError();
 }
 

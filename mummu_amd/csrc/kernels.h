@@ -98,7 +98,7 @@ hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int 
 // in sorted order).
 bool grouped_gemm_supported(const ExpertBanks &b);
 bool grouped_gemm_quantized(const ExpertBanks &b);
-int grouped_gemm_tile_rows(int n_assign, int n_experts);
+int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts);
 // x [n, d] f32 -> QAct64 (d % 64 == 0).
 hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s);
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,

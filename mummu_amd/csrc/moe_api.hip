@@ -255,7 +255,7 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
     const int na = (int)(n * k);
     if (n >= h->gemm_min_tokens && grouped_gemm_supported(b)) {
         // batched: sort the assignments by expert, then one grouped GEMM per projection
-        const int tile_rows = grouped_gemm_tile_rows(na, b.n_experts);
+        const int tile_rows = grouped_gemm_tile_rows(b, na, b.n_experts);
         // the 16-bit activation buffers, viewed in the batched path's 64-element-block layout
         const QAct64 xq64{h->xq.hi, h->xq.lo, h->xq.scale, (float *)h->xq.sum};
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
