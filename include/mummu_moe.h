@@ -49,7 +49,9 @@ enum mummu_status {
     MUMMU_ERR_NOT_LOADED = 8, /* the layer has no weights yet */
     MUMMU_ERR_TOKENS = 9,     /* more tokens than the workspace was sized for */
     MUMMU_ERR_DEVICE = 10,    /* no HIP device / a HIP call failed */
-    MUMMU_ERR_ARG = 11        /* null pointer or otherwise unusable argument */
+    MUMMU_ERR_ARG = 11,       /* null pointer or otherwise unusable argument */
+    MUMMU_ERR_IO = 12,        /* a file cannot be opened, read or mapped, or ends inside its header */
+    MUMMU_ERR_GGUF = 13       /* the GGUF container breaks one of the reader's rules (gguf.rs:1226-1376) */
 };
 
 /* Router arithmetic.  0: SparseMoe / SparseMoePerExpert (nn/moe.rs:144-150: f32 softmax,
@@ -159,6 +161,69 @@ MUMMU_API int mummu_moe_stack_forward_device(mummu_moe *h, const float *x_dev, i
 MUMMU_API int mummu_moe_check(mummu_moe *h, void *stream);
 /* Device copies of the last call's routing: ids int32 [n, k], weights f32 [n, k]. */
 MUMMU_API int mummu_moe_last_routing(mummu_moe *h, int64_t n_tokens, int top_k, int32_t *ids, float *weights);
+
+/* ---- GGUF container reader and expert-bank locator (host side, no device work) ----------
+ * GgufFile::open / open_sharded (gguf.rs:577-714): magic, version 2 or 3, bounded counts
+ * (65,536 tensors, 4,096 metadata pairs, 1 MiB strings, 2^22 array items, 4 dims, 64 shards),
+ * typed metadata, `general.alignment` (a power of two, default 32), tensor table with known
+ * type ids, aligned offsets, whole blocks, no duplicate names and no overlapping payloads;
+ * a split set (`split.count` > 1, names `<base>-NNNNN-of-NNNNN.gguf`) is opened as one. */
+typedef struct mummu_gguf mummu_gguf;
+
+/* GgufTensorInfo (gguf.rs:403-430) plus GgufFile::payload_location (gguf.rs:1096).  Strings live as long as the
+ * mummu_gguf does.  dims are in GGUF order (fastest first), padded with 1. */
+typedef struct mummu_gguf_tensor {
+    const char *name;
+    int32_t n_dims;
+    int64_t dims[4];
+    int32_t ggml_type;
+    int32_t shard;        /* index of the file of the split set that holds the payload */
+    uint64_t file_offset; /* absolute offset in that file: its payload base + the table's offset */
+    uint64_t nbytes;
+    const char *path;     /* that file */
+} mummu_gguf_tensor;
+
+/* Message of the last failed mummu_gguf_* / mummu_moe_load_gguf call on this thread. */
+MUMMU_API const char *mummu_gguf_last_error(void);
+MUMMU_API int mummu_gguf_open(const char *path, mummu_gguf **out);
+MUMMU_API void mummu_gguf_close(mummu_gguf *g);
+MUMMU_API int mummu_gguf_version(const mummu_gguf *g);
+MUMMU_API int64_t mummu_gguf_alignment(const mummu_gguf *g);
+MUMMU_API int mummu_gguf_shard_count(const mummu_gguf *g);
+MUMMU_API int mummu_gguf_tensor_count(const mummu_gguf *g);
+MUMMU_API int mummu_gguf_kv_count(const mummu_gguf *g);
+/* GgufFile::tensor_index (gguf.rs:1082): index of the named tensor or -1. */
+MUMMU_API int mummu_gguf_find_tensor(const mummu_gguf *g, const char *name);
+MUMMU_API int mummu_gguf_tensor_info(const mummu_gguf *g, int index, mummu_gguf_tensor *out);
+/* The payload bytes (what GgufFile::read_tensor_f32, gguf.rs:733, reads before dequantizing),
+ * mapped read-only from the owning shard; valid until close. */
+MUMMU_API int mummu_gguf_tensor_data(mummu_gguf *g, int index, const void **data, uint64_t *nbytes);
+/* GgufFile::get with GgufValue::as_u64 / as_f32 / as_bool / as_str (gguf.rs:140-188, 1062): typed metadata reads.
+ * get_u64 takes any unsigned integer type and bool (0/1); get_f64 takes f32 and f64; get_str
+ * returns NULL when the key is absent or not a string. */
+MUMMU_API int mummu_gguf_get_u64(const mummu_gguf *g, const char *key, uint64_t *out);
+MUMMU_API int mummu_gguf_get_f64(const mummu_gguf *g, const char *key, double *out);
+MUMMU_API const char *mummu_gguf_get_str(const mummu_gguf *g, const char *key);
+/* OlmoeConfig::from_gguf (models/olmoe.rs:116-179), the fields the MoE block reads, from
+ * `<general.architecture>.*`: embedding_length, expert_feed_forward_length (else
+ * feed_forward_length), expert_count, expert_used_count, block_count, expert_weights_norm
+ * (bool, default false), attention.layer_norm_rms_epsilon (f32, required).  router_flavour is set
+ * to MUMMU_ROUTER_SPARSE_MOE and max_tokens to 512; the caller may change both. */
+MUMMU_API int mummu_gguf_moe_config(const mummu_gguf *g, mummu_moe_config *cfg);
+/* The expert-bank locator for one layer (models/olmoe.rs:325-347, qwen4exp/experts.rs:869-911):
+ * tensor indices of `blk.L.ffn_gate_inp.weight` [H,E], `blk.L.ffn_{gate,up}_exps.weight` [H,I,E],
+ * `blk.L.ffn_down_exps.weight` [I,H,E] and `blk.L.ffn_norm.weight` [H] (-1 when absent), with
+ * dims checked against the header's configuration, rows checked to be whole blocks and the bank
+ * geometry checked against the table's byte length.  Host only. */
+typedef struct mummu_gguf_moe_layer {
+    int32_t router, gate, up, down, norm;
+} mummu_gguf_moe_layer;
+MUMMU_API int mummu_gguf_locate_moe_layer(const mummu_gguf *g, int layer, mummu_gguf_moe_layer *out);
+/* RoutedExperts::open (experts.rs:869-911) + Olmoe's MoE-block load (models/olmoe.rs:338-345):
+ * locates layers [first_layer, first_layer + n_layers) as above and loads them into the
+ * handle's layers 0..n_layers through mummu_moe_load_layer, payload bytes unchanged (mapped
+ * read-only from their shard, offsets relative to that shard's own payload base). */
+MUMMU_API int mummu_moe_load_gguf(mummu_moe *h, mummu_gguf *g, int first_layer, int n_layers);
 
 /* ---- plumbing for harnesses that do not link HIP themselves -----------------------------*/
 MUMMU_API void *mummu_device_alloc(size_t bytes);

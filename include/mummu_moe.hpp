@@ -16,6 +16,12 @@
 //                                                      mummu::RoutedExperts
 //   route                      experts.rs:541-582     mummu::route
 //   gguf::dequantize           gguf.rs:1403-1463      mummu::dequantize
+//   GgufFile::open_sharded, tensor, get, payload_location
+//                              gguf.rs:577-714, 1062-1122
+//                                                      mummu::GgufFile
+//   OlmoeConfig::from_gguf (MoE fields) models/olmoe.rs:116-179   mummu::GgufFile::moe_config
+//   RoutedExperts::open (bank locator) experts.rs:869-911         mummu::GgufFile::locate_moe_layer,
+//                                                                  mummu::SparseMoe::from_gguf
 //
 // Error behaviour: the reference panics on contract violations of SparseMoe (assert!) and
 // returns Err(String) from the qwen4exp functions.  Both surface here as mummu::MoeError (a
@@ -25,6 +31,7 @@
 
 #include <cstdint>
 #include <memory>
+#include <optional>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -91,6 +98,120 @@ struct Routing {
     }
 };
 
+// GgufError (gguf.rs:65-118): every refusal of the container reader.
+class GgufError : public MoeError {
+  public:
+    using MoeError::MoeError;
+};
+
+// GgufTensorInfo (gguf.rs:403-430) with its payload location (gguf.rs:1096).
+struct GgufTensorInfo {
+    std::string name;
+    std::vector<uint64_t> dims;  // GGUF order, fastest-varying first
+    int ggml_type = 0;
+    int shard = 0;
+    std::string path;
+    uint64_t file_offset = 0;
+    uint64_t byte_len = 0;
+};
+
+// A parsed and validated GGUF file or split set (gguf.rs:538-714).
+class GgufFile {
+  public:
+    // GgufFile::open_sharded (gguf.rs:628): a single file, or any member of a split set.
+    static GgufFile open(const std::string &path) {
+        mummu_gguf *g = nullptr;
+        const int rc = mummu_gguf_open(path.c_str(), &g);
+        if (rc != MUMMU_OK) throw GgufError(rc, mummu_gguf_last_error());
+        return GgufFile(g);
+    }
+    mummu_gguf *handle() const { return g_.get(); }
+    int version() const { return mummu_gguf_version(g_.get()); }
+    uint64_t alignment() const { return (uint64_t)mummu_gguf_alignment(g_.get()); }
+    size_t shard_count() const { return (size_t)mummu_gguf_shard_count(g_.get()); }
+    size_t tensor_count() const { return (size_t)mummu_gguf_tensor_count(g_.get()); }
+    std::optional<std::string> architecture() const { return get_str("general.architecture"); }
+
+    std::optional<uint64_t> get_u64(const std::string &key) const {
+        uint64_t v = 0;
+        if (mummu_gguf_get_u64(g_.get(), key.c_str(), &v) != MUMMU_OK) return std::nullopt;
+        return v;
+    }
+    std::optional<double> get_f64(const std::string &key) const {
+        double v = 0;
+        if (mummu_gguf_get_f64(g_.get(), key.c_str(), &v) != MUMMU_OK) return std::nullopt;
+        return v;
+    }
+    std::optional<std::string> get_str(const std::string &key) const {
+        const char *s = mummu_gguf_get_str(g_.get(), key.c_str());
+        if (!s) return std::nullopt;
+        return std::string(s);
+    }
+
+    std::optional<size_t> tensor_index(const std::string &name) const {
+        const int i = mummu_gguf_find_tensor(g_.get(), name.c_str());
+        if (i < 0) return std::nullopt;
+        return (size_t)i;
+    }
+    GgufTensorInfo tensor_at(size_t index) const {
+        mummu_gguf_tensor t{};
+        check(mummu_gguf_tensor_info(g_.get(), (int)index, &t));
+        GgufTensorInfo out;
+        out.name = t.name;
+        out.dims.assign(t.dims, t.dims + t.n_dims);
+        out.ggml_type = t.ggml_type;
+        out.shard = t.shard;
+        out.path = t.path;
+        out.file_offset = t.file_offset;
+        out.byte_len = t.nbytes;
+        return out;
+    }
+    std::optional<GgufTensorInfo> tensor(const std::string &name) const {
+        const auto i = tensor_index(name);
+        if (!i) return std::nullopt;
+        return tensor_at(*i);
+    }
+    // The payload bytes, mapped read-only; valid while this object lives.
+    std::pair<const uint8_t *, uint64_t> tensor_bytes(const std::string &name) const {
+        const auto i = tensor_index(name);
+        if (!i) throw GgufError(MUMMU_ERR_GGUF, "GGUF has no " + name);
+        const void *p = nullptr;
+        uint64_t n = 0;
+        check(mummu_gguf_tensor_data(g_.get(), (int)*i, &p, &n));
+        return {(const uint8_t *)p, n};
+    }
+
+    // The MoE fields of OlmoeConfig::from_gguf (models/olmoe.rs:116-179).
+    SparseMoeConfig moe_config() const {
+        mummu_moe_config k{};
+        check(mummu_gguf_moe_config(g_.get(), &k));
+        SparseMoeConfig c;
+        c.hidden_size = k.hidden_size;
+        c.expert_intermediate_size = k.expert_intermediate_size;
+        c.num_experts = k.num_experts;
+        c.num_experts_per_tok = k.num_experts_per_tok;
+        c.norm_topk_prob = k.norm_topk_prob != 0;
+        c.router_flavour = k.router_flavour;
+        c.num_layers = k.num_layers;
+        c.max_tokens = k.max_tokens;
+        c.rms_norm_eps = k.rms_norm_eps;
+        return c;
+    }
+    // The bank locator for one layer (experts.rs:869-911): tensor indices, norm -1 when absent.
+    mummu_gguf_moe_layer locate_moe_layer(int layer) const {
+        mummu_gguf_moe_layer at{};
+        check(mummu_gguf_locate_moe_layer(g_.get(), layer, &at));
+        return at;
+    }
+
+  private:
+    explicit GgufFile(mummu_gguf *g) : g_(g, mummu_gguf_close) {}
+    static void check(int rc) {
+        if (rc != MUMMU_OK) throw GgufError(rc, mummu_gguf_last_error());
+    }
+    std::shared_ptr<mummu_gguf> g_;
+};
+
 // The block, resident on the MI355X.  One object holds every MoE layer of a model.
 class SparseMoe {
   public:
@@ -119,6 +240,22 @@ class SparseMoe {
                     const float *rms_gamma = nullptr) {
         check(mummu_moe_load_layer(h_.get(), layer, router.data, router.ggml_type, gate.data, gate.ggml_type, up.data,
                                    up.ggml_type, down.data, down.ggml_type, rms_gamma));
+    }
+
+    // The MoE blocks of file layers [first_layer, first_layer + n_layers) as layers 0.. of a new
+    // object, payload bytes unchanged (RoutedExperts::open, experts.rs:869-911).  n_layers < 0
+    // takes every layer from first_layer on.
+    static SparseMoe from_gguf(const GgufFile &f, int first_layer = 0, int n_layers = -1, int max_tokens = 512,
+                               int router_flavour = MUMMU_ROUTER_SPARSE_MOE) {
+        SparseMoeConfig c = f.moe_config();
+        if (n_layers < 0) n_layers = c.num_layers - first_layer;
+        c.num_layers = n_layers > 0 ? n_layers : 1;
+        c.max_tokens = max_tokens;
+        c.router_flavour = router_flavour;
+        SparseMoe m(c);
+        const int rc = mummu_moe_load_gguf(m.handle(), f.handle(), first_layer, n_layers);
+        if (rc != MUMMU_OK) throw GgufError(rc, mummu_gguf_last_error());
+        return m;
     }
 
     uint64_t resident_bytes() const { return mummu_moe_resident_bytes(h_.get()); }

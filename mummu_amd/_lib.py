@@ -15,10 +15,10 @@ F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
 ROUTER_SPARSE_MOE, ROUTER_QWEN4EXP = 0, 1
 
 (OK, ERR_CONFIG, ERR_TYPE, ERR_BLOCKS, ERR_TOPK, ERR_SHAPE, ERR_NONFINITE, ERR_RANGE, ERR_NOT_LOADED, ERR_TOKENS,
- ERR_DEVICE, ERR_ARG) = range(12)
+ ERR_DEVICE, ERR_ARG, ERR_IO, ERR_GGUF) = range(14)
 
 STATUS_NAMES = ["ok", "config", "type", "blocks", "topk", "shape", "nonfinite", "range", "not_loaded", "tokens",
-                "device", "arg"]
+                "device", "arg", "io", "gguf"]
 
 
 class Config(C.Structure):
@@ -28,6 +28,19 @@ class Config(C.Structure):
         ("num_experts_per_tok", C.c_int32), ("norm_topk_prob", C.c_int32), ("router_flavour", C.c_int32),
         ("num_layers", C.c_int32), ("max_tokens", C.c_int32), ("rms_norm_eps", C.c_float),
     ]
+
+
+class GgufTensor(C.Structure):
+    """mummu_gguf_tensor."""
+    _fields_ = [
+        ("name", C.c_char_p), ("n_dims", C.c_int32), ("dims", C.c_int64 * 4), ("ggml_type", C.c_int32),
+        ("shard", C.c_int32), ("file_offset", C.c_uint64), ("nbytes", C.c_uint64), ("path", C.c_char_p),
+    ]
+
+
+class GgufMoeLayer(C.Structure):
+    """mummu_gguf_moe_layer."""
+    _fields_ = [("router", C.c_int32), ("gate", C.c_int32), ("up", C.c_int32), ("down", C.c_int32), ("norm", C.c_int32)]
 
 
 # name -> (restype, argtypes); the list the header declares, checked against the .so by the tests
@@ -67,6 +80,23 @@ SIGNATURES = {
     "mummu_timer_start": (_I, [_P]),
     "mummu_timer_stop": (_I, [_P, C.POINTER(C.c_float)]),
     "mummu_probe_copy": (_I, [_P, _P, _SZ, _P]),
+    "mummu_gguf_last_error": (C.c_char_p, []),
+    "mummu_gguf_open": (_I, [C.c_char_p, C.POINTER(_P)]),
+    "mummu_gguf_close": (None, [_P]),
+    "mummu_gguf_version": (_I, [_P]),
+    "mummu_gguf_alignment": (_I64, [_P]),
+    "mummu_gguf_shard_count": (_I, [_P]),
+    "mummu_gguf_tensor_count": (_I, [_P]),
+    "mummu_gguf_kv_count": (_I, [_P]),
+    "mummu_gguf_find_tensor": (_I, [_P, C.c_char_p]),
+    "mummu_gguf_tensor_info": (_I, [_P, _I, C.POINTER(GgufTensor)]),
+    "mummu_gguf_tensor_data": (_I, [_P, _I, C.POINTER(_P), C.POINTER(C.c_uint64)]),
+    "mummu_gguf_get_u64": (_I, [_P, C.c_char_p, C.POINTER(C.c_uint64)]),
+    "mummu_gguf_get_f64": (_I, [_P, C.c_char_p, C.POINTER(C.c_double)]),
+    "mummu_gguf_get_str": (C.c_char_p, [_P, C.c_char_p]),
+    "mummu_gguf_moe_config": (_I, [_P, C.POINTER(Config)]),
+    "mummu_gguf_locate_moe_layer": (_I, [_P, _I, C.POINTER(GgufMoeLayer)]),
+    "mummu_moe_load_gguf": (_I, [_P, _P, _I, _I]),
     "mummu_moe_kernel_timing": (_I, [_P, _I]),
     "mummu_moe_kernel_times": (_I, [_P, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(C.c_int64), _I]),
 }

@@ -5,7 +5,10 @@
 //   zero input -> zero output                          nn/moe.rs:2340-2352
 //   contract violations are loud                       nn/moe.rs:119-130
 //   route known answers                                models/qwen4exp/experts.rs:1365-1388
-// `--no-gpu` runs only the checks that need no device (config validation).
+//   GGUF reader: round trip, refusals, bank locator    gguf.rs:2280-2378, experts.rs:869-911
+// `--no-gpu` runs only the checks that need no device (config validation, GGUF parsing).
+#include <unistd.h>
+
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -112,6 +115,133 @@ static bool throws(F &&f, int status, const char *needle) {
     return false;
 }
 
+
+// ---- a minimal GGUF v3 writer for the toy block (little-endian host) ---------------------------
+struct GgufBytes {
+    std::string head, payload;
+    uint64_t n_kv = 0, n_tensors = 0;
+    template <typename T>
+    static void put(std::string &s, T v) {
+        s.append((const char *)&v, sizeof(T));
+    }
+    static void put_str(std::string &s, const std::string &v) {
+        put<uint64_t>(s, v.size());
+        s += v;
+    }
+    std::string kvs, table;
+    void kv_str(const std::string &k, const std::string &v) {
+        put_str(kvs, k);
+        put<uint32_t>(kvs, 8);
+        put_str(kvs, v);
+        n_kv++;
+    }
+    void kv_u32(const std::string &k, uint32_t v) {
+        put_str(kvs, k);
+        put<uint32_t>(kvs, 4);
+        put<uint32_t>(kvs, v);
+        n_kv++;
+    }
+    void kv_f32(const std::string &k, float v) {
+        put_str(kvs, k);
+        put<uint32_t>(kvs, 6);
+        put<float>(kvs, v);
+        n_kv++;
+    }
+    void tensor(const std::string &name, std::vector<uint64_t> dims, uint32_t type, const void *data, size_t nbytes) {
+        payload.append((32 - payload.size() % 32) % 32, '\0');
+        put_str(table, name);
+        put<uint32_t>(table, (uint32_t)dims.size());
+        for (uint64_t d : dims) put<uint64_t>(table, d);
+        put<uint32_t>(table, type);
+        put<uint64_t>(table, payload.size());
+        payload.append((const char *)data, nbytes);
+        n_tensors++;
+    }
+    std::string write(const std::string &name) const {
+        std::string out = "GGUF";
+        put<uint32_t>(out, 3);
+        put<uint64_t>(out, n_tensors);
+        put<uint64_t>(out, n_kv);
+        out += kvs + table;
+        out.append((32 - out.size() % 32) % 32, '\0');
+        out += payload;
+        const std::string path = "/tmp/mummu-host-mirror-" + std::to_string((long)getpid()) + "-" + name;
+        FILE *f = std::fopen(path.c_str(), "wb");
+        if (!f || std::fwrite(out.data(), 1, out.size(), f) != out.size()) {
+            std::printf("FAIL cannot write %s\n", path.c_str());
+            failures++;
+        }
+        if (f) std::fclose(f);
+        return path;
+    }
+};
+
+// The toy block as an OLMoE-named model file: router [H,E] in GGUF dims = row-major [E,H] bytes.
+static GgufBytes toy_gguf(const std::vector<float> &r, const std::vector<float> &g, const std::vector<float> &u,
+                          const std::vector<float> &d) {
+    GgufBytes w;
+    w.kv_str("general.architecture", "olmoe");
+    w.kv_u32("olmoe.block_count", 1);
+    w.kv_u32("olmoe.embedding_length", H);
+    w.kv_u32("olmoe.feed_forward_length", I);
+    w.kv_u32("olmoe.expert_count", E);
+    w.kv_u32("olmoe.expert_used_count", K);
+    w.kv_f32("olmoe.attention.layer_norm_rms_epsilon", 1e-5f);
+    w.tensor("blk.0.ffn_gate_inp.weight", {H, E}, 0, r.data(), r.size() * 4);
+    w.tensor("blk.0.ffn_gate_exps.weight", {H, I, E}, 0, g.data(), g.size() * 4);
+    w.tensor("blk.0.ffn_up_exps.weight", {H, I, E}, 0, u.data(), u.size() * 4);
+    w.tensor("blk.0.ffn_down_exps.weight", {I, H, E}, 0, d.data(), d.size() * 4);
+    return w;
+}
+
+static void gguf_host_checks(const std::vector<float> &r, const std::vector<float> &g, const std::vector<float> &u,
+                             const std::vector<float> &d) {
+    const std::string path = toy_gguf(r, g, u, d).write("toy.gguf");
+    {
+        mummu::GgufFile f = mummu::GgufFile::open(path);
+        EXPECT(f.version() == 3 && f.alignment() == 32 && f.shard_count() == 1 && f.tensor_count() == 4, "header fields");
+        EXPECT(f.architecture() == std::optional<std::string>("olmoe"), "architecture");
+        EXPECT(f.get_u64("olmoe.expert_count") == std::optional<uint64_t>(E), "typed metadata read");
+        EXPECT(!f.get_u64("general.architecture") && !f.get_str("olmoe.expert_count") && !f.tensor("absent"), "absent or wrongly typed reads give nothing");
+        const mummu::SparseMoeConfig c = f.moe_config();
+        EXPECT(c.hidden_size == H && c.expert_intermediate_size == I && c.num_experts == E && c.num_experts_per_tok == K &&
+                   c.num_layers == 1 && !c.norm_topk_prob,
+               "MoE configuration from the header");
+        const auto gate = f.tensor("blk.0.ffn_gate_exps.weight");
+        EXPECT(gate && gate->dims == (std::vector<uint64_t>{H, I, E}) && gate->byte_len == (uint64_t)E * I * H * 4 && gate->file_offset % 32 == 0, "tensor info");
+        const auto bytes = f.tensor_bytes("blk.0.ffn_down_exps.weight");
+        EXPECT(bytes.second == d.size() * 4 && std::memcmp(bytes.first, d.data(), d.size() * 4) == 0, "payload bytes unchanged");
+        const mummu_gguf_moe_layer at = f.locate_moe_layer(0);
+        EXPECT(at.router >= 0 && at.gate >= 0 && at.up >= 0 && at.down >= 0 && at.norm == -1, "locator finds the four tensors, no norm");
+        EXPECT(throws([&] { f.locate_moe_layer(1); }, MUMMU_ERR_RANGE, "layer 1"), "layer outside the file");
+    }
+    ::unlink(path.c_str());
+    // refusals: magic, truncation, a bank with swapped dims
+    {
+        GgufBytes w = toy_gguf(r, g, u, d);
+        std::string p2 = w.write("bad.gguf");
+        FILE *fp = std::fopen(p2.c_str(), "r+b");
+        if (fp) {
+            std::fwrite("FUGG", 1, 4, fp);
+            std::fclose(fp);
+        }
+        EXPECT(throws([&] { mummu::GgufFile::open(p2); }, MUMMU_ERR_GGUF, "not a GGUF file"), "bad magic");
+        ::unlink(p2.c_str());
+        EXPECT(throws([&] { mummu::GgufFile::open(p2); }, MUMMU_ERR_IO, "cannot open"), "missing file");
+        GgufBytes sw;
+        sw.kvs = w.kvs;
+        sw.n_kv = w.n_kv;
+        sw.tensor("blk.0.ffn_gate_inp.weight", {H, E}, 0, r.data(), r.size() * 4);
+        sw.tensor("blk.0.ffn_gate_exps.weight", {I, H, E}, 0, g.data(), g.size() * 4);
+        sw.tensor("blk.0.ffn_up_exps.weight", {H, I, E}, 0, u.data(), u.size() * 4);
+        sw.tensor("blk.0.ffn_down_exps.weight", {I, H, E}, 0, d.data(), d.size() * 4);
+        const std::string p3 = sw.write("swapped.gguf");
+        mummu::GgufFile f = mummu::GgufFile::open(p3);
+        EXPECT(throws([&] { f.locate_moe_layer(0); }, MUMMU_ERR_SHAPE, "ffn_gate_exps.weight: dim 0"), "swapped bank dims");
+        ::unlink(p3.c_str());
+    }
+}
+
 int main(int argc, char **argv) {
     const bool no_gpu = argc > 1 && std::string(argv[1]) == "--no-gpu";
     mummu::SparseMoeConfig cfg;
@@ -132,6 +262,11 @@ int main(int argc, char **argv) {
         bad = cfg;
         bad.hidden_size = 0;
         EXPECT(throws([&] { mummu::SparseMoe m(bad); }, MUMMU_ERR_CONFIG, "hidden"), "zero hidden size must be refused");
+    }
+    {
+        const std::vector<float> r = router_eh(), g = sin_fill(0.1f, E * I * H), u = sin_fill(1.7f, E * I * H),
+                                 d = sin_fill(3.3f, E * H * I);
+        gguf_host_checks(r, g, u, d);
     }
     if (no_gpu) {
         std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror (no gpu): ok\n", failures);
@@ -167,6 +302,20 @@ int main(int argc, char **argv) {
                 for (uint64_t hh : moe.take_hits()) hits += hh;
                 EXPECT(hits == (uint64_t)(t * k), "hit counters count the rows run_local served (route alone serves none)");
             }
+
+    // the same block read back from a model file gives the same bits
+    {
+        const std::string path = toy_gguf(r, g, u, d).write("load.gguf");
+        {
+            mummu::GgufFile f = mummu::GgufFile::open(path);
+            mummu::SparseMoe from_file = mummu::SparseMoe::from_gguf(f, 0, -1, 8);
+            EXPECT(from_file.resident_bytes() == moe.resident_bytes(), "resident bytes after load_gguf");
+            const std::vector<float> x = input(5, 2.0f);
+            const std::vector<float> a = from_file.forward(x, K, true), b = moe.forward(x, K, true);
+            EXPECT(std::memcmp(a.data(), b.data(), a.size() * 4) == 0, "from_gguf(file) == load_layer(bytes)");
+        }
+        ::unlink(path.c_str());
+    }
 
     // zero in, zero out (nn/moe.rs:2340-2352)
     {
