@@ -27,13 +27,19 @@ extern "C" {
 
 #define MUMMU_API __attribute__((visibility("default")))
 
-/* ggml tensor type ids (gguf.rs:298-324).  Expert banks: F32, F16, BF16, Q8_0, Q4_K.
- * Router: F32, F16, BF16. */
+/* ggml tensor type ids (gguf.rs:298-324).  Expert banks and mummu_dequantize: all of these
+ * (the block layouts of gguf.rs:1535-1797).  Router: F32, F16, BF16. */
 enum mummu_ggml_type {
     MUMMU_F32 = 0,
     MUMMU_F16 = 1,
+    MUMMU_Q4_0 = 2,
+    MUMMU_Q4_1 = 3,
+    MUMMU_Q5_0 = 6,
+    MUMMU_Q5_1 = 7,
     MUMMU_Q8_0 = 8,
     MUMMU_Q4_K = 12,
+    MUMMU_Q5_K = 13,
+    MUMMU_Q6_K = 14,
     MUMMU_BF16 = 30
 };
 

@@ -12,6 +12,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libmummu_moe.so")
 
 F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
+Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q6_K = 2, 3, 6, 7, 13, 14
+# ggml type id -> (elements per block, bytes per block)
+BLOCKS = {F32: (1, 4), F16: (1, 2), BF16: (1, 2), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24),
+          Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
 ROUTER_SPARSE_MOE, ROUTER_QWEN4EXP = 0, 1
 
 (OK, ERR_CONFIG, ERR_TYPE, ERR_BLOCKS, ERR_TOPK, ERR_SHAPE, ERR_NONFINITE, ERR_RANGE, ERR_NOT_LOADED, ERR_TOKENS,

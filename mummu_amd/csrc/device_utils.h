@@ -71,26 +71,38 @@ static __device__ long long *g_trace_buf = nullptr;
 #endif
 
 // ggml tensor type ids (the values stored in GGUF tensor tables).
-enum : int { T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_BF16 = 30 };
+enum : int {
+    T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8,
+    T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30
+};
 
-__host__ __device__ inline int block_elems(int t) {
+__host__ __device__ constexpr int block_elems(int t) {
     switch (t) {
     case T_F32: case T_F16: case T_BF16: return 1;
-    case T_Q8_0: return 32;
-    case T_Q4_K: return 256;
+    case T_Q4_0: case T_Q4_1: case T_Q5_0: case T_Q5_1: case T_Q8_0: return 32;
+    case T_Q4_K: case T_Q5_K: case T_Q6_K: return 256;
     default: return 0;
     }
 }
 
-__host__ __device__ inline int block_bytes(int t) {
+__host__ __device__ constexpr int block_bytes(int t) {
     switch (t) {
     case T_F32: return 4;
     case T_F16: case T_BF16: return 2;
+    case T_Q4_0: return 18;
+    case T_Q4_1: return 20;
+    case T_Q5_0: return 22;
+    case T_Q5_1: return 24;
     case T_Q8_0: return 34;
     case T_Q4_K: return 144;
+    case T_Q5_K: return 176;
+    case T_Q6_K: return 210;
     default: return 0;
     }
 }
+
+// The block-quantized types (everything but the plain float types).
+__host__ __device__ constexpr bool is_quant_type(int t) { return block_elems(t) > 1; }
 
 // IEEE half bits -> f32, exact (subnormals included: gfx9 keeps f16 denormals).
 __device__ inline float half_bits_to_float(uint16_t bits) {

@@ -29,11 +29,34 @@
 #include "gemv_common.h"
 #include "route_common.h"
 
+#include <type_traits>
+
 MUMMU_TRACE_UNIT(experts)
 
 namespace mummu {
 
 constexpr int kGemvWaves = 4;  // waves per workgroup of the float kernels
+
+// Calls f(std::integral_constant<int, TYPE>) for a bank type this file has kernels for.
+template <typename F>
+static hipError_t with_bank_type(int type, F &&f) {
+#define MUMMU_TYPE_CASE(T) case T: return f(std::integral_constant<int, T>())
+    switch (type) {
+        MUMMU_TYPE_CASE(T_F32);
+        MUMMU_TYPE_CASE(T_F16);
+        MUMMU_TYPE_CASE(T_BF16);
+        MUMMU_TYPE_CASE(T_Q8_0);
+        MUMMU_TYPE_CASE(T_Q4_K);
+        MUMMU_TYPE_CASE(T_Q4_0);
+        MUMMU_TYPE_CASE(T_Q4_1);
+        MUMMU_TYPE_CASE(T_Q5_0);
+        MUMMU_TYPE_CASE(T_Q5_1);
+        MUMMU_TYPE_CASE(T_Q5_K);
+        MUMMU_TYPE_CASE(T_Q6_K);
+    default: return hipErrorInvalidValue;
+    }
+#undef MUMMU_TYPE_CASE
+}
 
 // ------------------------------------------------------------------------------------------
 // gate/up, quantized banks: NIT iterations of rows_per_it rows per wave; the workgroup's
@@ -115,8 +138,23 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     MUMMU_PHASE(2);
     dispatch_group(rs.group, [&](auto group_tag) {
         constexpr int GROUP = decltype(group_tag)::value;
-        const int offset = reduce_partials<2 * NIT, GROUP>(part, lane);
         constexpr int count = reduced_count<2 * NIT, GROUP>();
+        if constexpr (count < 2) {
+            // whole-wave rows and fewer than four iterations: the shared reduction would leave a
+            // row's gate and up sums in different lanes, so reduce each over the wave instead
+#pragma unroll
+            for (int i = 0; i < NIT; i++) {
+                const float g = wave_sum(part[2 * i]), u = wave_sum(part[2 * i + 1]);
+                const int row = row0 + i * rs.rows_per_it + sub;
+                if (lane == 0 && row < inter) {
+                    const float v = __fmul_rn(det_silu(g), u);
+                    if (ACTQ) s_act[row - block_row0] = v;
+                    else act[(size_t)a * (size_t)inter + row] = v;
+                }
+            }
+            return;
+        }
+        const int offset = reduce_partials<2 * NIT, GROUP>(part, lane);
         constexpr int width = GROUP < 16 ? GROUP : 16;
         if ((lane & (width - 1)) == 0) {
 #pragma unroll
@@ -381,7 +419,7 @@ static int pick_rows_per_wave(int out_dim, int n_assign) {
 template <int WT>
 static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq, const int32_t *ids, int n_assign,
                                    int k, int fixed_expert, float *act, QAct actq, int32_t *flags, hipStream_t s) {
-    constexpr bool quant = WT == T_Q4_K || WT == T_Q8_0;
+    constexpr bool quant = is_quant_type(WT);
     const bool actq_out = is_quant_type(b.down_type);
     const int slots = fixed_expert >= 0 ? 1 : k;  // n_assign = tokens * slots
     if constexpr (quant) {
@@ -430,14 +468,9 @@ hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const i
     if (n_assign <= 0) return hipSuccess;
     if (b.gate_type != b.up_type) return hipErrorInvalidValue;
     if (n_assign / (fixed_expert >= 0 ? 1 : k) > 65535) return hipErrorInvalidValue;
-    switch (b.gate_type) {
-    case T_F32: return launch_gate_up_t<T_F32>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
-    case T_F16: return launch_gate_up_t<T_F16>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
-    case T_BF16: return launch_gate_up_t<T_BF16>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
-    case T_Q8_0: return launch_gate_up_t<T_Q8_0>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
-    case T_Q4_K: return launch_gate_up_t<T_Q4_K>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
-    default: return hipErrorInvalidValue;
-    }
+    return with_bank_type(b.gate_type, [&](auto tag) {
+        return launch_gate_up_t<decltype(tag)::value>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
+    });
 }
 
 bool gate_up_routes_inline(const ExpertBanks &b, int k) {
@@ -457,19 +490,22 @@ hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInlin
     const int rpb = waves * NIT * rs.rows_per_it;
     dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(64 * waves);
     const size_t lds = sizeof(float) * (size_t)rpb;
-    if (b.gate_type == T_Q4_K)
-        launch_kernel(gate_up_q_kernel<T_Q4_K, 1, NIT, true, true>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, k,
-                      -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route);
-    else
-        launch_kernel(gate_up_q_kernel<T_Q8_0, 1, NIT, true, true>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, k,
-                      -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route);
-    return hipGetLastError();
+    return with_bank_type(b.gate_type, [&](auto tag) {
+        constexpr int WT = decltype(tag)::value;
+        if constexpr (is_quant_type(WT)) {
+            launch_kernel(gate_up_q_kernel<WT, 1, NIT, true, true>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, k,
+                          -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route);
+            return hipGetLastError();
+        } else {
+            return hipErrorInvalidValue;
+        }
+    });
 }
 
 template <int WT>
 static hipError_t launch_down_t(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign,
                                 int k, int fixed_expert, float *y, hipStream_t s) {
-    constexpr bool quant = WT == T_Q4_K || WT == T_Q8_0;
+    constexpr bool quant = is_quant_type(WT);
     const int slots = fixed_expert >= 0 ? 1 : k;  // n_assign = tokens * slots
     dim3 block(64 * kGemvWaves);
     if constexpr (quant) {
@@ -502,14 +538,9 @@ hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const 
                        int fixed_expert, float *y, hipStream_t s) {
     if (n_assign <= 0) return hipSuccess;
     if (n_assign / (fixed_expert >= 0 ? 1 : k) > 65535) return hipErrorInvalidValue;
-    switch (b.down_type) {
-    case T_F32: return launch_down_t<T_F32>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
-    case T_F16: return launch_down_t<T_F16>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
-    case T_BF16: return launch_down_t<T_BF16>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
-    case T_Q8_0: return launch_down_t<T_Q8_0>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
-    case T_Q4_K: return launch_down_t<T_Q4_K>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
-    default: return hipErrorInvalidValue;
-    }
+    return with_bank_type(b.down_type, [&](auto tag) {
+        return launch_down_t<decltype(tag)::value>(b, act, actq, ids, n_assign, k, fixed_expert, y, s);
+    });
 }
 
 bool down_combine_supported(const ExpertBanks &b, int k) {
@@ -545,8 +576,11 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
                                const float *residual, float *out, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     if (!down_combine_supported(b, k)) return hipErrorInvalidValue;
-    return b.down_type == T_Q4_K ? launch_down_combine_t<T_Q4_K>(b, actq, ids, weights, n, k, residual, out, s)
-                                 : launch_down_combine_t<T_Q8_0>(b, actq, ids, weights, n, k, residual, out, s);
+    return with_bank_type(b.down_type, [&](auto tag) {
+        constexpr int WT = decltype(tag)::value;
+        if constexpr (is_quant_type(WT)) return launch_down_combine_t<WT>(b, actq, ids, weights, n, k, residual, out, s);
+        else return hipErrorInvalidValue;
+    });
 }
 
 // ------------------------------------------------------------------------------------------

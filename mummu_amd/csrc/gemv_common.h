@@ -31,10 +31,16 @@ __host__ __device__ inline RowSplit row_split(int in_dim) {
 // Start elements of the two 16-element halves unit u of a row covers.
 template <int WT>
 __device__ inline void unit_halves(int u, int &e0, int &e1) {
-    if constexpr (WT == T_Q4_K) {
+    if constexpr (WT == T_Q4_K || WT == T_Q5_K) {
         int sb = u >> 3, up = u & 7;
         e0 = sb * 256 + (up >> 1) * 64 + (up & 1) * 16;  // low nibbles: elements of sub-block 2c
         e1 = e0 + 32;                                    // high nibbles: sub-block 2c+1
+    } else if constexpr (WT == T_Q6_K) {
+        // unit = 16 bytes of ql: their low nibbles are 16 consecutive elements, their high
+        // nibbles the 16 elements 64 further on (ql byte offset inside the super-block = 16*up)
+        int sb = u >> 3, up = u & 7;
+        e0 = sb * 256 + (up >> 2) * 128 + (up & 3) * 16;
+        e1 = e0 + 64;
     } else {
         e0 = u * 32;
         e1 = e0 + 16;
@@ -89,6 +95,34 @@ struct RawRow<T_Q8_0, UPL> {
     uint32_t q[UPL][8];  // 32 int8 codes
 };
 
+// Legacy 32-element blocks (Q4_0 18 B, Q4_1 20 B, Q5_0 22 B, Q5_1 24 B): f16 d (, f16 m)
+// (, u32 fifth bits), 16 bytes of nibbles.
+template <int WT, int UPL>
+struct RawLegacy {
+    uint32_t dm[UPL];    // f16 d in the low half, f16 m in the high half (0 where the type has none)
+    uint32_t qh[UPL];    // fifth bits (Q5_0, Q5_1)
+    uint32_t q[UPL][4];  // nibbles
+};
+template <int UPL> struct RawRow<T_Q4_0, UPL> : RawLegacy<T_Q4_0, UPL> {};
+template <int UPL> struct RawRow<T_Q4_1, UPL> : RawLegacy<T_Q4_1, UPL> {};
+template <int UPL> struct RawRow<T_Q5_0, UPL> : RawLegacy<T_Q5_0, UPL> {};
+template <int UPL> struct RawRow<T_Q5_1, UPL> : RawLegacy<T_Q5_1, UPL> {};
+template <int UPL>
+struct RawRow<T_Q5_K, UPL> {
+    uint4 hdr[UPL];  // f16 d, f16 dmin, 12 B of 6-bit scales/mins
+    uint4 qh[UPL];   // fifth bits of the lane's 16 byte positions (all four chunks)
+    uint4 q[UPL];    // the lane's 16 bytes of nibbles
+};
+template <int UPL>
+struct RawRow<T_Q6_K, UPL> {
+    uint32_t ql[UPL][4];  // 16 bytes of low 4 bits
+    uint32_t qh[UPL][4];  // the 16 bytes of high 2 bits they share with the unit 32 elements on
+    uint32_t sc[UPL];     // int8 scale of the low-nibble elements | int8 scale of the high-nibble ones << 8
+    uint32_t d[UPL];      // f16 super-block scale bits
+};
+
+constexpr bool is_legacy32(int t) { return t == T_Q4_0 || t == T_Q4_1 || t == T_Q5_0 || t == T_Q5_1; }
+
 template <int WT, int UPL>
 __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int units, bool ok, RawRow<WT, UPL> &r) {
     // Every lane loads unconditionally (a lane without a unit re-reads the row's last unit, a
@@ -105,6 +139,41 @@ __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int
             r.hdr[i] = *(const uint4 *)blk;
             r.q[i] = *(const uint4 *)(blk + 16 + (uc & 7) * 16);
             r.hdr[i].x = on ? r.hdr[i].x : 0u;  // d = dmin = 0
+        } else if constexpr (WT == T_Q5_K) {
+            const uint8_t *blk = rowp + (size_t)(uc >> 3) * 176;  // 176 = 11 * 16: every piece is 16-byte aligned
+            r.hdr[i] = *(const uint4 *)blk;
+            r.qh[i] = *(const uint4 *)(blk + 16 + (uc & 1) * 16);
+            r.q[i] = *(const uint4 *)(blk + 48 + (uc & 7) * 16);
+            r.hdr[i].x = on ? r.hdr[i].x : 0u;
+        } else if constexpr (WT == T_Q6_K) {
+            const uint8_t *blk = rowp + (size_t)(uc >> 3) * 210;  // 2-byte aligned only
+            const int up = uc & 7;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                __builtin_memcpy(&r.ql[i][w], blk + 16 * up + 4 * w, 4);
+                __builtin_memcpy(&r.qh[i][w], blk + 128 + (up >> 2) * 32 + (up & 1) * 16 + 4 * w, 4);
+            }
+            const uint8_t *sc = blk + 192 + (up >> 2) * 8 + ((up >> 1) & 1) * 2 + (up & 1);
+            r.sc[i] = (uint32_t)sc[0] | ((uint32_t)sc[4] << 8);
+            uint16_t db;
+            __builtin_memcpy(&db, blk + 208, 2);
+            r.d[i] = on ? (uint32_t)db : 0u;
+        } else if constexpr (is_legacy32(WT)) {
+            constexpr bool has_m = WT == T_Q4_1 || WT == T_Q5_1;
+            constexpr bool has_h = WT == T_Q5_0 || WT == T_Q5_1;
+            const uint8_t *blk = rowp + (size_t)uc * block_bytes(WT);
+            uint16_t db, mb = 0;
+            __builtin_memcpy(&db, blk, 2);
+            if constexpr (has_m) __builtin_memcpy(&mb, blk + 2, 2);
+            r.dm[i] = on ? ((uint32_t)db | ((uint32_t)mb << 16)) : 0u;
+            const uint8_t *p = blk + (has_m ? 4 : 2);
+            r.qh[i] = 0u;
+            if constexpr (has_h) {
+                __builtin_memcpy(&r.qh[i], p, 4);
+                p += 4;
+            }
+#pragma unroll
+            for (int w = 0; w < 4; w++) __builtin_memcpy(&r.q[i][w], p + 4 * w, 4);
         } else {
             const uint8_t *blk = rowp + (size_t)uc * 34;
             uint16_t db;
@@ -161,6 +230,85 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
             const float pos = __builtin_fmaf(a.s[i][0], p0, __fmul_rn(a.s[i][1], p1));
             const float neg = __builtin_fmaf(a.s[i][0], n0, __fmul_rn(a.s[i][1], n1));
             acc = __fadd_rn(acc, __builtin_fmaf(-dmin, neg, __fmul_rn(d, pos)));
+        } else if constexpr (WT != T_Q8_0) {
+            // Every other type: the two 16-element halves as non-negative byte codes c0, c1 with
+            //     weight = A_h * code + B_h,
+            // so the half's share is s_h * (A_h * sum(code * xq) + B_h * sum(xq)).
+            uint32_t c0[4], c1[4];
+            float A0, A1, B0, B1;
+            if constexpr (is_legacy32(WT)) {
+                const float d = half_bits_to_float((uint16_t)(r.dm[i] & 0xFFFFu));
+                const float m = half_bits_to_float((uint16_t)(r.dm[i] >> 16));
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    c0[w] = r.q[i][w] & 0x0F0F0F0Fu;
+                    c1[w] = (r.q[i][w] >> 4) & 0x0F0F0F0Fu;
+                    if constexpr (WT == T_Q5_0 || WT == T_Q5_1) {
+                        // fifth bit of element j is bit j of qh: 4 bits -> bit 4 of 4 bytes
+                        c0[w] |= (((r.qh[i] >> (4 * w)) & 0xFu) * 0x02040810u) & 0x10101010u;
+                        c1[w] |= (((r.qh[i] >> (16 + 4 * w)) & 0xFu) * 0x02040810u) & 0x10101010u;
+                    }
+                }
+                A0 = A1 = d;
+                B0 = B1 = WT == T_Q4_0 ? __fmul_rn(-8.0f, d) : (WT == T_Q5_0 ? __fmul_rn(-16.0f, d) : m);
+            } else if constexpr (WT == T_Q5_K) {
+                const int u = unit0 + 64 * i;
+                const uint4 hdr = r.hdr[i];
+                const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFFu));
+                const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
+                const int c = (u & 7) >> 1;
+                const int sh = 16 * (c & 1);
+                int sc0, sc1, mn0, mn1;
+                if (c < 2) {
+                    sc0 = (int)((hdr.y >> sh) & 63u);
+                    sc1 = (int)((hdr.y >> (sh + 8)) & 63u);
+                    mn0 = (int)((hdr.z >> sh) & 63u);
+                    mn1 = (int)((hdr.z >> (sh + 8)) & 63u);
+                } else {
+                    const uint32_t lo = hdr.w >> sh;
+                    sc0 = (int)((lo & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4));
+                    mn0 = (int)(((lo >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4));
+                    sc1 = (int)(((lo >> 8) & 0xFu) | (((hdr.y >> (sh + 14)) & 3u) << 4));
+                    mn1 = (int)(((lo >> 12) & 0xFu) | (((hdr.z >> (sh + 14)) & 3u) << 4));
+                }
+                const uint32_t q[4] = {r.q[i].x, r.q[i].y, r.q[i].z, r.q[i].w};
+                const uint32_t h[4] = {r.qh[i].x, r.qh[i].y, r.qh[i].z, r.qh[i].w};
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    c0[w] = (q[w] & 0x0F0F0F0Fu) | (((h[w] >> (2 * c)) & 0x01010101u) << 4);
+                    c1[w] = ((q[w] >> 4) & 0x0F0F0F0Fu) | (((h[w] >> (2 * c + 1)) & 0x01010101u) << 4);
+                }
+                A0 = __fmul_rn(d, (float)sc0);
+                A1 = __fmul_rn(d, (float)sc1);
+                B0 = -__fmul_rn(dmin, (float)mn0);
+                B1 = -__fmul_rn(dmin, (float)mn1);
+            } else {  // Q6_K
+                const int u = unit0 + 64 * i;
+                const int jj = ((u & 7) >> 1) & 1;  // which pair of 2-bit fields of qh: (0, 4) or (2, 6)
+                const float d = half_bits_to_float((uint16_t)r.d[i]);
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    c0[w] = (r.ql[i][w] & 0x0F0F0F0Fu) | (((r.qh[i][w] >> (2 * jj)) & 0x03030303u) << 4);
+                    c1[w] = ((r.ql[i][w] >> 4) & 0x0F0F0F0Fu) | (((r.qh[i][w] >> (2 * jj + 4)) & 0x03030303u) << 4);
+                }
+                A0 = __fmul_rn(d, (float)(int)(int8_t)(r.sc[i] & 0xFFu));
+                A1 = __fmul_rn(d, (float)(int)(int8_t)((r.sc[i] >> 8) & 0xFFu));
+                B0 = __fmul_rn(-32.0f, A0);
+                B1 = __fmul_rn(-32.0f, A1);
+            }
+            int h0 = 0, l0 = 0, h1 = 0, l1 = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                h0 = __builtin_amdgcn_sdot4((int)c0[w], a.xh[i][w], h0, false);
+                l0 = __builtin_amdgcn_sdot4((int)c0[w], a.xl[i][w], l0, false);
+                h1 = __builtin_amdgcn_sdot4((int)c1[w], a.xh[i][4 + w], h1, false);
+                l1 = __builtin_amdgcn_sdot4((int)c1[w], a.xl[i][4 + w], l1, false);
+            }
+            // codes <= 63 and |xq| <= 32512: every integer sum fits 32 bits
+            const float t0 = __builtin_fmaf(A0, (float)(h0 * 256 + l0), __fmul_rn(B0, (float)a.sx[i][0]));
+            const float t1 = __builtin_fmaf(A1, (float)(h1 * 256 + l1), __fmul_rn(B1, (float)a.sx[i][1]));
+            acc = __builtin_fmaf(a.s[i][0], t0, acc);
+            acc = __builtin_fmaf(a.s[i][1], t1, acc);
         } else {  // Q8_0
             const float d = half_bits_to_float((uint16_t)r.d[i]);
             int h0 = 0, l0 = 0, h1 = 0, l1 = 0;

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "device_utils.h"
 #include "qact.h"
 
 namespace mummu {
@@ -43,7 +44,6 @@ struct ExpertBanks {
     int hidden, inter, n_experts;
 };
 
-inline bool is_quant_type(int t) { return t == 8 || t == 12; }
 
 // act[a, j] = silu(<gate_e[j,:], x_t>) * <up_e[j,:], x_t>  for assignment a = t*k + s,
 // e = ids[a] (or fixed_expert >= 0 with token = a: the single-expert entry point).

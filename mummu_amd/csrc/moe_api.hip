@@ -90,7 +90,7 @@ int fail(mummu_moe *h, int code, const std::string &msg) {
             return fail(h, MUMMU_ERR_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_));            \
     } while (0)
 
-bool bank_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16 || t == T_Q8_0 || t == T_Q4_K; }
+bool bank_type_ok(int t) { return block_elems(t) > 0; }  // F32, F16, BF16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K
 bool router_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16; }
 size_t row_bytes_of(int t, int in_dim) { return (size_t)(in_dim / block_elems(t)) * (size_t)block_bytes(t); }
 
@@ -441,9 +441,9 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
         return fail(h, MUMMU_ERR_BLOCKS, "row width " + std::to_string(H) + " is not whole blocks of " + std::to_string(block_elems(gate_type)));
     if (I % block_elems(down_type))
         return fail(h, MUMMU_ERR_BLOCKS, "row width " + std::to_string(I) + " is not whole blocks of " + std::to_string(block_elems(down_type)));
-    if ((gate_type == T_Q4_K || gate_type == T_Q8_0) && H / 32 > 256)
+    if (is_quant_type(gate_type) && H / 32 > 256)
         return fail(h, MUMMU_ERR_CONFIG, "quantized rows wider than 8192 are not supported");
-    if ((down_type == T_Q4_K || down_type == T_Q8_0) && I / 32 > 256)
+    if (is_quant_type(down_type) && I / 32 > 256)
         return fail(h, MUMMU_ERR_CONFIG, "quantized rows wider than 8192 are not supported");
 
     Layer &L = h->layers[layer];

@@ -22,7 +22,8 @@ from typing import List, Optional, Sequence, Tuple
 import numpy as np
 
 from . import _lib
-from ._lib import BF16, F16, F32, Q4_K, Q8_0, ROUTER_QWEN4EXP, ROUTER_SPARSE_MOE  # noqa: F401
+from ._lib import (BF16, F16, F32, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, ROUTER_QWEN4EXP,  # noqa: F401
+                   ROUTER_SPARSE_MOE)
 
 
 class MoeError(RuntimeError):
@@ -121,7 +122,7 @@ class SparseMoe:
         router, gate, up, down = _bytes(router), _bytes(gate), _bytes(up), _bytes(down)
 
         def want(t, in_dim, out_dim):
-            bs = {F32: (1, 4), F16: (1, 2), BF16: (1, 2), Q8_0: (32, 34), Q4_K: (256, 144)}.get(t)
+            bs = _lib.BLOCKS.get(t)
             if bs is None or in_dim % bs[0]:
                 return None  # the library reports the precise error
             return c.num_experts * out_dim * (in_dim // bs[0]) * bs[1]
@@ -380,7 +381,7 @@ def device_name() -> str:
 def dequantize(dtype: int, data) -> np.ndarray:
     """gguf::dequantize (gguf.rs:1403) on the GPU, bit-exact."""
     b = _bytes(data)
-    geom = {F32: (1, 4), F16: (1, 2), BF16: (1, 2), Q8_0: (32, 34), Q4_K: (256, 144)}.get(dtype, (1, 1))
+    geom = _lib.BLOCKS.get(dtype, (1, 1))
     out = np.empty(max(b.size // geom[1], 1) * geom[0], dtype=np.float32)
     lib = _lib.load()
     rc = lib.mummu_dequantize(dtype, _ptr(b), b.size, _ptr(out))

@@ -19,10 +19,24 @@ _M1 = np.uint64(0xBF58476D1CE4E5B9)
 _M2 = np.uint64(0x94D049BB133111EB)
 
 # ggml type ids (gguf.rs:298-324)
-F32, F16, Q5_1, Q8_0, Q4_K, Q5_K, BF16 = 0, 1, 7, 8, 12, 13, 30
+F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 2, 3, 6, 7, 8, 12, 13, 14, 30
 
-BLOCK_SIZE = {F32: 1, F16: 1, BF16: 1, Q5_1: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256}
-BLOCK_BYTES = {F32: 4, F16: 2, BF16: 2, Q5_1: 24, Q8_0: 34, Q4_K: 144, Q5_K: 176}
+BLOCK_SIZE = {F32: 1, F16: 1, BF16: 1, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256}
+BLOCK_BYTES = {F32: 4, F16: 2, BF16: 2, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+
+# f16 header fields of a synthetic block: (byte offset, low, high).  Q8_0, Q5_1, Q4_K and Q5_K are
+# the reference's ranges (experts.rs:1209-1237); the others are this package's own, chosen to give
+# weights of the same magnitude.
+SCALE_FIELDS = {
+    Q8_0: [(0, 0.002, 0.02)],
+    Q5_1: [(0, 0.005, 0.05), (2, -0.4, 0.0)],
+    Q4_K: [(0, 0.0005, 0.003), (2, 0.0005, 0.003)],
+    Q5_K: [(0, 0.0003, 0.002), (2, 0.0003, 0.002)],
+    Q4_0: [(0, 0.005, 0.05)],
+    Q4_1: [(0, 0.005, 0.05), (2, -0.4, 0.0)],
+    Q5_0: [(0, 0.003, 0.03)],
+    Q6_K: [(208, 0.00002, 0.0002)],
+}
 
 
 def row_bytes(dtype: int, in_dim: int) -> int:
@@ -85,28 +99,25 @@ def synth_blocks(dtype: int, blocks: int, rng: SplitMix64) -> np.ndarray:
     """``blocks`` sane blocks of ``dtype``: finite, modest f16 scales and random quant bits
     (experts.rs:1209-1237).  Draws are consumed block by block in the reference's order:
     the scale uniform(s) first, then one draw per payload byte."""
-    if dtype == Q8_0:
-        heads, ranges, payload = 1, [(0.002, 0.02)], 32
-    elif dtype == Q5_1:
-        heads, ranges, payload = 2, [(0.005, 0.05), (-0.4, 0.0)], 20
-    elif dtype == Q4_K:
-        heads, ranges, payload = 2, [(0.0005, 0.003), (0.0005, 0.003)], 140
-    elif dtype == Q5_K:
-        heads, ranges, payload = 2, [(0.0003, 0.002), (0.0003, 0.002)], 172
-    else:
+    if dtype not in SCALE_FIELDS:
         raise ValueError(f"no synthetic blocks for ggml type {dtype}")
-    per = heads + payload
-    out = np.empty((blocks, BLOCK_BYTES[dtype]), dtype=np.uint8)
+    fields = SCALE_FIELDS[dtype]
+    bb = BLOCK_BYTES[dtype]
+    heads = len(fields)
+    head_bytes = {o + i for o, _, _ in fields for i in (0, 1)}
+    body = np.array([i for i in range(bb) if i not in head_bytes])
+    per = heads + len(body)
+    out = np.empty((blocks, bb), dtype=np.uint8)
     # Generate in slabs so a multi-hundred-MB bank never holds 8x its size in u64 draws.
     slab = max(1, (1 << 22) // per)
     for b0 in range(0, blocks, slab):
         nb = min(slab, blocks - b0)
         draws = rng.next_u64(nb * per).reshape(nb, per)
-        for h, (lo, hi) in enumerate(ranges):
+        for h, (off, lo, hi) in enumerate(fields):
             bits = f16_bits(SplitMix64._to_uniform(draws[:, h], lo, hi))
-            out[b0:b0 + nb, 2 * h] = (bits & 0xFF).astype(np.uint8)
-            out[b0:b0 + nb, 2 * h + 1] = (bits >> 8).astype(np.uint8)
-        out[b0:b0 + nb, 2 * heads:] = SplitMix64._to_byte(draws[:, heads:])
+            out[b0:b0 + nb, off] = (bits & 0xFF).astype(np.uint8)
+            out[b0:b0 + nb, off + 1] = (bits >> 8).astype(np.uint8)
+        out[b0:b0 + nb, body] = SplitMix64._to_byte(draws[:, heads:])
     return out.reshape(-1)
 
 
@@ -151,14 +162,10 @@ def random_bank_fast(dtype: int, ne, seed: int) -> np.ndarray:
     blocks = in_dim // BLOCK_SIZE[dtype] * out_dim * n_experts
     bb = BLOCK_BYTES[dtype]
     out = g.integers(0, 256, size=(blocks, bb), dtype=np.uint8)
-    if dtype == Q8_0:
-        ranges = [(0.002, 0.02)]
-    elif dtype == Q4_K:
-        ranges = [(0.0005, 0.003), (0.0005, 0.003)]
-    else:
+    if dtype not in SCALE_FIELDS:
         raise ValueError(f"no fast bank for ggml type {dtype}")
-    for h, (lo, hi) in enumerate(ranges):
+    for off, lo, hi in SCALE_FIELDS[dtype]:
         bits = f16_bits(g.uniform(lo, hi, size=blocks).astype(np.float32))
-        out[:, 2 * h] = (bits & 0xFF).astype(np.uint8)
-        out[:, 2 * h + 1] = (bits >> 8).astype(np.uint8)
+        out[:, off] = (bits & 0xFF).astype(np.uint8)
+        out[:, off + 1] = (bits >> 8).astype(np.uint8)
     return out.reshape(-1)

@@ -89,10 +89,10 @@ def test_a_split_set_loads_each_bank_from_its_own_shard(tmp_path):
 
 
 def test_a_bank_type_without_a_kernel_is_refused_with_the_tensor_named(tmp_path):
-    case = dict(CASE, down_type=14)  # Q6_K parses as a container type but has no expert kernel here
+    case = dict(CASE, down_type=10)  # Q2_K (84-byte super-blocks) parses as a container type but has no expert kernel here
     lw = weights(CASE, 1, 8)
-    lw[0]["down"] = np.zeros(CASE["experts"] * CASE["hidden"] * (CASE["inter"] // 256) * 210, np.uint8)
-    with GgufFile.open(W.moe_gguf(case, lw).write(tmp_path / "q6.gguf")) as f:
+    lw[0]["down"] = np.zeros(CASE["experts"] * CASE["hidden"] * (CASE["inter"] // 256) * 84, np.uint8)
+    with GgufFile.open(W.moe_gguf(case, lw).write(tmp_path / "q2.gguf")) as f:
         with pytest.raises(GgufError, match="blk.0") as e:
             f.load_moe(max_tokens=8)
         assert e.value.code == M._lib.ERR_TYPE

@@ -213,12 +213,12 @@ def test_routed_equals_run_local_and_hits_count_rows(toy):
 
 
 # ---------------------------------------------------------------------------------------------
-# quantized toy layers (experts.rs:1429-1563): gate/up Q4_K, down Q8_0
+# quantized toy layers (experts.rs:1429-1563): gate/up Q4_K, down Q5_1 (layer 0) / Q8_0 (layer 1)
 # ---------------------------------------------------------------------------------------------
 
-@pytest.fixture(scope="module")
-def toy_q():
-    raw = toy_d_layers(11)[1]
+@pytest.fixture(scope="module", params=[0, 1], ids=["down_q5_1", "down_q8_0"])
+def toy_q(request):
+    raw = toy_d_layers(11)[request.param]
     H, F, E = TOY_D["hidden"], TOY_D["ffn"], TOY_D["experts"]
     m = M.SparseMoe(M.SparseMoeConfig(H, F, E, 2), max_tokens=16, router_flavour=M.ROUTER_QWEN4EXP, norm_topk_prob=True)
     router = synth.SplitMix64(5).normal(E * H, 0.0, 0.05).reshape(E, H)
@@ -284,12 +284,16 @@ def test_expert_run_is_the_single_expert_swiglu(toy_q):
 
 
 def test_unsupported_bank_types_and_ragged_rows_are_refused():
-    raw = toy_d_layers(11)[0]  # down bank is Q5_1: no kernel yet
+    raw = toy_d_layers(11)[0]
     H, F, E = TOY_D["hidden"], TOY_D["ffn"], TOY_D["experts"]
     with M.SparseMoe(M.SparseMoeConfig(H, F, E, 2)) as m:
         router = np.zeros((E, H), np.float32)
-        with pytest.raises(M.MoeError, match="type"):
-            m.load_layer(0, router, M.F32, raw["gate"], raw["gate_type"], raw["up"], raw["up_type"], raw["down"], 7)
+        for no_kernel in (10, 11, 15, 20):  # Q2_K, Q3_K, Q8_K, IQ4_NL: container types without an expert kernel
+            with pytest.raises(M.MoeError, match="type"):
+                m.load_layer(0, router, M.F32, raw["gate"], raw["gate_type"], raw["up"], raw["up_type"], raw["down"], no_kernel)
+        with pytest.raises(M.MoeError, match="share one type"):
+            m.load_layer(0, router, M.F32, raw["gate"], M.Q4_K, np.zeros(E * F * (H // 256) * 176, np.uint8), M.Q5_K,
+                         raw["down"], raw["down_type"])
         with pytest.raises(M.MoeError):
             m.forward(np.zeros((1, H), np.float32), 2, False)  # nothing loaded
     # experts.rs:1355-1363: 640-wide rows cannot be K-quant
