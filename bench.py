@@ -45,7 +45,13 @@ WORKLOADS = {
     "olmoe_q8_0_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q8_0", router="F16"),
     "olmoe_f16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F16", router="F16"),
     "qwen3_a3b_q4k": dict(hidden=2048, inter=768, experts=128, top_k=8, norm=True, bank="Q4_K", router="F16"),
+    # mixed bank types: llama.cpp's Q4_K_M recipe stores part of ffn_down as Q6_K; the shipped qwen4exp file has
+    # Q4_K gate/up with Q5_1 downs, 512 experts, top-10 (models/qwen4exp/mod.rs:18-20, experts.rs:1838-1879)
+    "olmoe_q4km_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q4_K", down="Q6_K", router="F16"),
+    "qwen4exp_decode": dict(hidden=2560, inter=640, experts=512, top_k=10, norm=True, bank="Q4_K", down="Q5_1", router="F16",
+                            flavour=1),
 }
+BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "Q6_K": 14, "Q5_1": 7, "Q5_K": 13}
 
 
 def main() -> int:
@@ -75,7 +81,8 @@ def main() -> int:
 
     w = WORKLOADS[args.workload]
     H, I, E, k, norm = w["hidden"], w["inter"], w["experts"], w["top_k"], w["norm"]
-    bank_t = {"Q4_K": M.Q4_K, "Q8_0": M.Q8_0, "F16": M.F16}[w["bank"]]
+    bank_t = BANK_TYPES[w["bank"]]
+    down_t = BANK_TYPES[w.get("down", w["bank"])]
     router_t = M.F16
     n = args.tokens
     L = args.layers
@@ -85,22 +92,24 @@ def main() -> int:
 
     g = np.random.Generator(np.random.PCG64(args.seed))
 
-    def make_bank(in_dim, out_dim, seed):
-        if bank_t in (M.Q4_K, M.Q8_0):
-            return synth.random_bank_fast(bank_t, [in_dim, out_dim, E], seed)
+    def make_bank(in_dim, out_dim, seed, t=None):
+        t = bank_t if t is None else t
+        if t != M.F16:
+            return synth.random_bank_fast(t, [in_dim, out_dim, E], seed)
         gg = np.random.Generator(np.random.PCG64(seed))
         return (gg.standard_normal(E * out_dim * in_dim, dtype=np.float32) * np.float32(0.02)).astype(np.float16).view(np.uint8)
 
     t_setup = time.time()
-    moe = M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=max(n, 8), norm_topk_prob=norm)
+    moe = M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=max(n, 8), norm_topk_prob=norm,
+                      router_flavour=w.get("flavour", 0))
     routers = []
     keep_layer0 = None
     for l in range(L):
         router = (g.standard_normal((E, H), dtype=np.float32) * np.float32(0.02)).astype(np.float16)
         gate = make_bank(H, I, args.seed * 1000 + 3 * l)
         up = make_bank(H, I, args.seed * 1000 + 3 * l + 1)
-        down = make_bank(I, H, args.seed * 1000 + 3 * l + 2)
-        moe.load_layer(l, router, router_t, gate, bank_t, up, bank_t, down, bank_t)
+        down = make_bank(I, H, args.seed * 1000 + 3 * l + 2, down_t)
+        moe.load_layer(l, router, router_t, gate, bank_t, up, bank_t, down, down_t)
         routers.append(router)
         if l == 0:
             keep_layer0 = (router, gate, up, down)
@@ -111,7 +120,7 @@ def main() -> int:
     out_dev = M.DeviceBuffer(n * H * 4)
     setup_s = time.time() - t_setup
 
-    expert_bytes = 2 * I * synth.row_bytes(bank_t, H) + H * synth.row_bytes(bank_t, I)
+    expert_bytes = 2 * I * synth.row_bytes(bank_t, H) + H * synth.row_bytes(down_t, I)
     gate_up_expert_bytes = 2 * I * synth.row_bytes(bank_t, H)
     router_bytes = E * H * 2
 
@@ -184,6 +193,7 @@ def main() -> int:
     # the dominant kernel and the bytes one launch of it has to move
     kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes + n * E * 4,
                     "down_combine": mean_distinct * (expert_bytes - gate_up_expert_bytes),
+                    "down": mean_distinct * (expert_bytes - gate_up_expert_bytes),
                     "gemm_gate_up": mean_distinct * gate_up_expert_bytes}
     timed = {name: us for name, us in per_kernel_us.items() if us is not None and name in kernel_bytes}
     dom = max(timed, key=lambda name: timed[name] * kt[name][1]) if timed else None
@@ -213,10 +223,10 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"Q4_K": "u4*i16->i32 (v_dot4_i32_i8), f32 scales", "Q8_0": "i8*i16->i32 (v_dot4_i32_i8), f32 scales",
-                  "F16": "f32"}[w["bank"]],
+        "dtype": "f32" if w["bank"] == "F16" else ("i8*i16->i32" if w["bank"] == "Q8_0" else "u4*i16->i32") +
+                 " (v_dot4_i32_i8), f32 scales",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts, "
+        "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
                    "tokens_per_step": n, "layers": L, "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
                    "mean_distinct_experts_per_step": round(mean_distinct, 3)},
@@ -237,26 +247,26 @@ def main() -> int:
     }
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(keep_layer0, w, bank_t, xs, n, args.cpu_seconds)
+        out["cpu_baseline"] = cpu_baseline(keep_layer0, w, bank_t, down_t, xs, n, args.cpu_seconds)
     print(json.dumps(out))
     return 0
 
 
-def cpu_baseline(layer0, w, bank_t, xs, n, budget_s):
+def cpu_baseline(layer0, w, bank_t, down_t, xs, n, budget_s):
     """The oracle's routed path (the reference's qwen4exp algorithm: per hit expert, dequantize
     row chunks and dot them in the fixed 8-lane order; OpenMP over rows where the reference
     uses rayon) on layer 0 of the same banks, same token batches, for about budget_s seconds."""
     from oracle import binding as orc
     router, gate, up, down = layer0
     H, I, E, k, norm = w["hidden"], w["inter"], w["experts"], w["top_k"], w["norm"]
-    t = {"Q4_K": orc.Q4_K, "Q8_0": orc.Q8_0, "F16": orc.F16}[w["bank"]]
-    banks = orc.LayerBanks(H, I, E, gate, up, down, t)
+    banks = orc.LayerBanks(H, I, E, gate, up, down, bank_t, bank_t, down_t)  # the oracle uses the same ggml type ids
+    flavour = w.get("flavour", 0)
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    orc.moe_forward(banks, router, orc.F16, xs[0], k, norm)  # warm
+    orc.moe_forward(banks, router, orc.F16, xs[0], k, norm, flavour)  # warm
     done, t0, best = 0, time.perf_counter(), None
     while time.perf_counter() - t0 < budget_s:
         t1 = time.perf_counter()
-        orc.moe_forward(banks, router, orc.F16, xs[done % xs.shape[0]], k, norm)
+        orc.moe_forward(banks, router, orc.F16, xs[done % xs.shape[0]], k, norm, flavour)
         dt = time.perf_counter() - t1
         best = dt if best is None else min(best, dt)
         done += 1

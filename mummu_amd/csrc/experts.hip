@@ -63,15 +63,18 @@ static hipError_t with_bank_type(int type, F &&f) {
 // rows_per_block = waves*NIT*rows_per_it output rows are a whole number of 16-element
 // activation blocks, quantized for the down projection in the epilogue.
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int NIT, bool ACTQ, bool ROUTE = false>
+// RJN > 0: the kernel routes by itself, RJN experts per lane of the routing wave (see RouteInline).
+template <int WT, int UPL, int NIT, bool ACTQ, int RJN = 0>
 __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restrict__ gate,
                                                          const uint8_t *__restrict__ up, QAct xq,
                                                          const int32_t *__restrict__ ids, int k, int fixed_expert,
                                                          int hidden, int inter, int n_experts,
                                                          float *__restrict__ act, QAct actq,
                                                          int32_t *__restrict__ flags, RouteInline route) {
+    constexpr bool ROUTE = RJN > 0;
+    constexpr int JN = ROUTE ? RJN : 1;
     extern __shared__ float s_act[];  // rows_per_block floats
-    __shared__ __attribute__((aligned(16))) RouteScratch<1> s_route;
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> s_route;
     __shared__ int s_ids[64];
     __shared__ float s_w[64];
     MUMMU_PHASE(0);
@@ -85,8 +88,10 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     if (ROUTE) {
         // wave 0 routes token t from its logits; everybody else already has the activations coming
         if (wave == 0) {
-            float l[1] = {lane < n_experts ? route.logits[(size_t)t * n_experts + lane] : 0.0f};
-            route_token<1>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
+            float l[JN];
+#pragma unroll
+            for (int j = 0; j < JN; j++) l[j] = lane + 64 * j < n_experts ? route.logits[(size_t)t * n_experts + lane + 64 * j] : 0.0f;
+            route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
             wave_lds_sync();
             if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
                 const int id = s_ids[lane];
@@ -302,14 +307,12 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_f_kernel(const uint8_t *
 }
 
 // ------------------------------------------------------------------------------------------
-// down + combine in one launch (quantized down bank, top_k <= 4*KPW): blockIdx.x = token,
-// blockIdx.y = tile of NIT*rows_per_it output rows.  The 4 waves split the token's experts
+// down + combine in one launch (quantized down bank, top_k <= kDcWaves*KPW <= 16): blockIdx.x = token,
+// blockIdx.y = tile of NIT*rows_per_it output rows.  The kDcWaves waves split the token's experts
 // in ascending-id order, KPW each; their row sums meet in LDS and are combined in that same
 // order, multiply and add rounded separately.
 // ------------------------------------------------------------------------------------------
-constexpr int kDcWaves = 4;
-
-template <int WT, int UPL, int NIT, int KPW>
+template <int WT, int UPL, int NIT, int KPW, int kDcWaves = 4>
 __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
     const uint8_t *__restrict__ down, QAct actq, const int32_t *__restrict__ ids, const float *__restrict__ weights,
     int k, int hidden, int inter, int n_experts, const float *__restrict__ residual, float *__restrict__ out) {
@@ -475,27 +478,39 @@ hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const i
 
 bool gate_up_routes_inline(const ExpertBanks &b, int k) {
     const RowSplit rs = row_split(b.hidden);
-    return is_quant_type(b.gate_type) && b.gate_type == b.up_type && is_quant_type(b.down_type) && rs.units <= 64 &&
-           b.n_experts <= 64 && k >= 1 && k <= b.n_experts && k <= 64 && b.inter % 16 == 0;
+    return is_quant_type(b.gate_type) && b.gate_type == b.up_type && is_quant_type(b.down_type) && rs.units <= 128 &&
+           b.n_experts <= 512 && k >= 1 && k <= b.n_experts && k <= 16 && b.inter % 16 == 0;
+}
+
+template <int WT, int UPL, int NIT>
+static hipError_t launch_gate_up_routed_t(const ExpertBanks &b, QAct xq, const RouteInline &route, int n_tokens, int k,
+                                          QAct actq, int32_t *flags, hipStream_t s) {
+    const RowSplit rs = row_split(b.hidden);
+    int waves = 4;
+    while (waves * NIT * rs.rows_per_it < 16) waves *= 2;
+    const int rpb = waves * NIT * rs.rows_per_it;
+    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(64 * waves);
+    const size_t lds = sizeof(float) * (size_t)rpb;
+#define MUMMU_GUR(JN)                                                                                                    \
+    launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true, JN>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, \
+                  k, -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route)
+    if (b.n_experts <= 64) MUMMU_GUR(1);
+    else if (b.n_experts <= 128) MUMMU_GUR(2);
+    else MUMMU_GUR(8);
+#undef MUMMU_GUR
+    return hipGetLastError();
 }
 
 hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInline &route, int n_tokens, int k, QAct actq,
                                  int32_t *flags, hipStream_t s) {
     if (n_tokens <= 0) return hipSuccess;
     if (!gate_up_routes_inline(b, k) || n_tokens > 65535) return hipErrorInvalidValue;
-    const RowSplit rs = row_split(b.hidden);
-    constexpr int NIT = 4;
-    int waves = 4;
-    while (waves * NIT * rs.rows_per_it < 16) waves *= 2;
-    const int rpb = waves * NIT * rs.rows_per_it;
-    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(64 * waves);
-    const size_t lds = sizeof(float) * (size_t)rpb;
+    const bool wide = row_split(b.hidden).units > 64;
     return with_bank_type(b.gate_type, [&](auto tag) {
         constexpr int WT = decltype(tag)::value;
         if constexpr (is_quant_type(WT)) {
-            launch_kernel(gate_up_q_kernel<WT, 1, NIT, true, true>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, k,
-                          -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route);
-            return hipGetLastError();
+            return wide ? launch_gate_up_routed_t<WT, 2, 2>(b, xq, route, n_tokens, k, actq, flags, s)
+                        : launch_gate_up_routed_t<WT, 1, 4>(b, xq, route, n_tokens, k, actq, flags, s);
         } else {
             return hipErrorInvalidValue;
         }
@@ -544,7 +559,7 @@ hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const 
 }
 
 bool down_combine_supported(const ExpertBanks &b, int k) {
-    return is_quant_type(b.down_type) && k <= 8 && (row_split(b.inter).units + 63) / 64 <= 2;
+    return is_quant_type(b.down_type) && k <= 16 && (row_split(b.inter).units + 63) / 64 <= 2;
 }
 
 template <int WT>
@@ -552,21 +567,25 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
                                         int k, const float *residual, float *out, hipStream_t s) {
     const RowSplit rs = row_split(b.inter);
     const int upl = (rs.units + 63) / 64;
-    dim3 block(64 * kDcWaves);
-#define MUMMU_DC(UPL, NIT, KPW)                                                                                    \
+#define MUMMU_DC(UPL, NIT, KPW, WAVES)                                                                             \
     do {                                                                                                           \
         const int rpb = (NIT)*rs.rows_per_it;                                                                      \
-        dim3 grid(n, (b.hidden + rpb - 1) / rpb);                                                                  \
-        const size_t lds = sizeof(float) * (size_t)(kDcWaves * (KPW)) * (size_t)(rpb + 1);                         \
-        launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW>, grid, block, lds, s, b.down, actq, ids, weights, k, b.hidden, \
-                                                                          b.inter, b.n_experts, residual, out);    \
+        dim3 grid(n, (b.hidden + rpb - 1) / rpb), block(64 * (WAVES));                                             \
+        const size_t lds = sizeof(float) * (size_t)((WAVES) * (KPW)) * (size_t)(rpb + 1);                          \
+        launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW, WAVES>, grid, block, lds, s, b.down, actq, ids, weights, k, \
+                      b.hidden, b.inter, b.n_experts, residual, out);                                              \
     } while (0)
+    // two experts per wave (one for top_k <= 4), as many waves as that takes
     if (upl == 1) {
-        if (k <= 4) MUMMU_DC(1, 4, 1);
-        else MUMMU_DC(1, 2, 2);
+        if (k <= 4) MUMMU_DC(1, 4, 1, 4);
+        else if (k <= 8) MUMMU_DC(1, 2, 2, 4);
+        else if (k <= 10) MUMMU_DC(1, 2, 2, 5);
+        else if (k <= 12) MUMMU_DC(1, 2, 2, 6);
+        else MUMMU_DC(1, 2, 2, 8);
     } else {
-        if (k <= 4) MUMMU_DC(2, 2, 1);
-        else MUMMU_DC(2, 2, 2);
+        if (k <= 4) MUMMU_DC(2, 2, 1, 4);
+        else if (k <= 8) MUMMU_DC(2, 2, 2, 4);
+        else MUMMU_DC(2, 2, 2, 8);
     }
 #undef MUMMU_DC
     return hipGetLastError();

@@ -55,7 +55,7 @@ hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const i
 // the routing (same arithmetic as route_topk, so the same bits in every workgroup) instead of
 // waiting for a separate launch to publish it; the workgroup of (slot 0, row tile 0) writes
 // ids / weights / hit counters for the kernels that follow.  Quantized gate/up banks feeding a
-// quantized down bank, hidden <= 2048, at most 64 experts.
+// quantized down bank, hidden <= 4096, at most 512 experts.
 struct RouteInline {
     const float *logits = nullptr;  // [n, n_experts]
     int flavour = 0, norm = 0;
@@ -74,7 +74,7 @@ hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const 
 // inv (nullable): y row of assignment a is inv[a] instead of a (dispatch-sorted layout).
 hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, const int32_t *inv, int n, int k,
                           int hidden, const float *residual, float *out, hipStream_t s);
-// down + combine in one launch (no y round trip): quantized down bank and top_k <= 8.
+// down + combine in one launch (no y round trip): quantized down bank and top_k <= 16.
 bool down_combine_supported(const ExpertBanks &b, int k);
 hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,
                                const float *residual, float *out, hipStream_t s);

@@ -65,8 +65,9 @@ struct RouteScratch {
 };
 
 // One wave routes one token whose logits sit in l[j] (expert lane + 64*j).  JN = experts held
-// per lane (num_experts <= 64 * JN).
-template <int JN>
+// per lane (num_experts <= 64 * JN).  ANY_K = false leaves out the ranking path of k > 16 (the
+// caller guarantees k <= 16), which is most of the code and of the registers.
+template <int JN, bool ANY_K = true>
 __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts, int k, int flavour, int norm,
                                    int32_t *__restrict__ ids, float *__restrict__ weights,
                                    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags,
@@ -107,12 +108,14 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
     }
     wave_lds_sync();
 
-    // normaliser: sequential over ascending expert id (every lane computes the same sum)
+    // normaliser: sequential over ascending expert id (every lane computes the same sum); the
+    // slots past n_experts hold +0 and are skipped in whole chunks of four
     const float4 *bp = (const float4 *)sc.p;
+    const int chunks = JN == 1 ? 16 : (n_experts + 3) >> 2;
     if (flavour == 0) {
         float total = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 16 * JN; c++) {
+#pragma unroll 16
+        for (int c = 0; c < chunks; c++) {
             const float4 v = bp[c];
             total = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(total, v.x), v.y), v.z), v.w);
         }
@@ -120,17 +123,31 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         for (int j = 0; j < JN; j++) p[j] = __fdiv_rn(p[j], total);
     } else {
         double total = 0.0;
+        // The f64 sum of at most 512 values in [0, 1] is EXACT, whatever the order, when every
+        // non-zero value is at least 2^-20: such an f32 is a multiple of 2^-43, and a sum of those
+        // that stays <= 2^9 fits f64's 53 bits.  Then a tree over the lanes gives the bits of the
+        // sequential sum; otherwise (a probability below 2^-20) add in expert order as written.
+        bool exact = JN > 1;
 #pragma unroll
-        for (int c = 0; c < 16 * JN; c++) {
-            const float4 v = bp[c];
-            total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
+        for (int j = 0; j < JN; j++) exact = exact && (p[j] == 0.0f || p[j] >= 0x1p-20f);
+        if (JN > 1 && __all(exact)) {
+#pragma unroll
+            for (int j = 0; j < JN; j++) total = __dadd_rn(total, (double)p[j]);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) total = __dadd_rn(total, __shfl_xor(total, off, 64));
+        } else {
+#pragma unroll 16
+            for (int c = 0; c < chunks; c++) {
+                const float4 v = bp[c];
+                total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
+            }
         }
         const float scale = (float)__ddiv_rn(1.0, total);
 #pragma unroll
         for (int j = 0; j < JN; j++) p[j] = __fmul_rn(p[j], scale);
     }
 
-    if (k <= 16) {
+    if (!ANY_K || k <= 16) {
         // k rounds of "largest remaining probability, lowest id on a tie": the wave maximum,
         // then the first lane (and, within a lane, the first expert) that holds it
         float cand[JN];
@@ -147,9 +164,12 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
             for (int j = JN - 1; j >= 0; j--)
                 if (cand[j] == best) my = lane + 64 * j;
             int win = my;
+            const unsigned long long m = __ballot(my != 0x7FFFFFFF);
             if (JN == 1) {
-                const unsigned long long m = __ballot(my != 0x7FFFFFFF);
                 win = (int)__builtin_ctzll(m);
+            } else if ((m & (m - 1)) == 0ull) {
+                // one lane holds the maximum (the usual case): its lowest such expert wins
+                win = __builtin_amdgcn_readlane(my, (int)__builtin_ctzll(m));
             } else {
                 // minimum id over the wave
                 float f = -(float)win;  // ids < 2^24: exact in f32, negated so that max finds the minimum

@@ -113,12 +113,15 @@ def test_router_refuses_non_finite_logits_and_bad_k(toy):
 
 
 @pytest.mark.parametrize("flavour,norm", [(M.ROUTER_QWEN4EXP, True), (M.ROUTER_SPARSE_MOE, False), (M.ROUTER_SPARSE_MOE, True)])
-@pytest.mark.parametrize("n_experts,k", [(8, 3), (64, 8), (128, 8), (130, 130), (512, 5)])
-def test_routing_of_random_logits_is_bit_exact(toy, flavour, norm, n_experts, k):
+@pytest.mark.parametrize("n_experts,k", [(8, 3), (64, 8), (128, 8), (130, 130), (512, 5), (512, 10), (300, 16)])
+@pytest.mark.parametrize("spread", [4.0, 14.0])
+def test_routing_of_random_logits_is_bit_exact(toy, flavour, norm, n_experts, k, spread):
+    # spread 4: every probability stays above 2^-20 of the largest (the f64 normaliser may be
+    # summed as a tree); spread 14: some fall below it (the sum must run in expert order)
     m = toy[0]
     rng = synth.SplitMix64(n_experts * 31 + k)
     n = 37
-    lg = rng.uniform(-4.0, 4.0, n * n_experts).reshape(n, n_experts)
+    lg = rng.uniform(-spread, spread, n * n_experts).reshape(n, n_experts)
     lg[::5, 1] = lg[::5, n_experts - 1]  # exact ties, some at the selection boundary
     lg[3] = 0.25                        # a fully tied row
     ids, w = M.route(m, lg, n, n_experts, k, flavour, norm)
