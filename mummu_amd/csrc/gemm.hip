@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// Q8_0 / Q4_K banks
+// block-quantized banks (Q8_0, Q4_K, Q5_K, Q6_K, Q4_0, Q4_1, Q5_0, Q5_1)
 // ---------------------------------------------------------------------------------------
 
 // Raw bytes of one thread's share of a weight tile: one 32-element block of one row.
@@ -240,6 +240,34 @@ struct RawQ<T_Q4_K> {
     uint4 hdr;
     uint4 q[2];
 };
+template <>
+struct RawQ<T_Q5_K> {
+    uint4 hdr;
+    uint4 qh[2];  // fifth bits of the 32 byte positions (all four chunks)
+    uint4 q[2];
+};
+template <>
+struct RawQ<T_Q6_K> {
+    uint32_t ql[8];  // 32 bytes of low 4 bits (one nibble of each is this block's)
+    uint32_t qh[8];  // 32 bytes of high 2 bits (one field of each is this block's)
+    uint32_t sc;     // the block's two int8 scales (16 elements each)
+    uint32_t d;
+};
+struct RawLegacyQ {
+    uint32_t dm;  // f16 d | f16 m << 16
+    uint32_t qh;  // fifth bits (Q5_0, Q5_1)
+    uint32_t q[4];
+};
+template <> struct RawQ<T_Q4_0> : RawLegacyQ {};
+template <> struct RawQ<T_Q4_1> : RawLegacyQ {};
+template <> struct RawQ<T_Q5_0> : RawLegacyQ {};
+template <> struct RawQ<T_Q5_1> : RawLegacyQ {};
+
+constexpr bool gemm_legacy32(int t) { return t == T_Q4_0 || t == T_Q4_1 || t == T_Q5_0 || t == T_Q5_1; }
+// weight = scale * code + offset with a non-zero offset (the offset term rides on an f32 MFMA)
+constexpr bool gemm_has_offset(int t) { return t != T_Q8_0 && t != T_Q6_K; }
+// one scale per 16 elements instead of per 32 (the integer products are split at 16)
+constexpr bool gemm_sub16(int t) { return t == T_Q6_K; }
 
 // rowp: start of the weight row; k0: first element of the K step (multiple of 64); half: which
 // 32-element block of the step.
@@ -252,48 +280,122 @@ __device__ inline void load_q(const uint8_t *__restrict__ rowp, int k0, int half
         r.d = db;
 #pragma unroll
         for (int w = 0; w < 8; w++) __builtin_memcpy(&r.q[w], blk + 2 + 4 * w, 4);
-    } else {
+    } else if constexpr (WT == T_Q4_K) {
         const uint8_t *blk = rowp + (size_t)(k0 >> 8) * 144;
         r.hdr = *(const uint4 *)blk;
         const uint4 *q = (const uint4 *)(blk + 16 + ((k0 & 255) >> 6) * 32);
         r.q[0] = q[0];
         r.q[1] = q[1];
+    } else if constexpr (WT == T_Q5_K) {
+        const uint8_t *blk = rowp + (size_t)(k0 >> 8) * 176;
+        r.hdr = *(const uint4 *)blk;
+        r.qh[0] = *(const uint4 *)(blk + 16);
+        r.qh[1] = *(const uint4 *)(blk + 32);
+        const uint4 *q = (const uint4 *)(blk + 48 + ((k0 & 255) >> 6) * 32);
+        r.q[0] = q[0];
+        r.q[1] = q[1];
+    } else if constexpr (WT == T_Q6_K) {
+        const uint8_t *blk = rowp + (size_t)(k0 >> 8) * 210;  // 2-byte aligned only
+        const int within = (k0 & 255) + 32 * half, n = within >> 7, j = (within & 127) >> 5;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            __builtin_memcpy(&r.ql[w], blk + 64 * n + 32 * (j & 1) + 4 * w, 4);
+            __builtin_memcpy(&r.qh[w], blk + 128 + 32 * n + 4 * w, 4);
+        }
+        uint16_t sb, db;
+        __builtin_memcpy(&sb, blk + 192 + 8 * n + 2 * j, 2);
+        __builtin_memcpy(&db, blk + 208, 2);
+        r.sc = sb;
+        r.d = db;
+    } else {
+        constexpr bool has_m = WT == T_Q4_1 || WT == T_Q5_1;
+        constexpr bool has_h = WT == T_Q5_0 || WT == T_Q5_1;
+        const uint8_t *blk = rowp + (size_t)(k0 / 32 + half) * block_bytes(WT);
+        uint16_t db, mb = 0;
+        __builtin_memcpy(&db, blk, 2);
+        if constexpr (has_m) __builtin_memcpy(&mb, blk + 2, 2);
+        r.dm = (uint32_t)db | ((uint32_t)mb << 16);
+        const uint8_t *p = blk + (has_m ? 4 : 2);
+        r.qh = 0u;
+        if constexpr (has_h) {
+            __builtin_memcpy(&r.qh, p, 4);
+            p += 4;
+        }
+#pragma unroll
+        for (int w = 0; w < 4; w++) __builtin_memcpy(&r.q[w], p + 4 * w, 4);
     }
 }
 
-// The block's 32 integers as bytes in element order, its scale, and minus its offset.
+// ggml get_scale_min_k4 on the 12 scale bytes held in three words.
+__device__ inline void k4_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j, uint32_t &sc, uint32_t &mn) {
+    auto byte_of = [&](int k) -> uint32_t {
+        const uint32_t w = k < 4 ? s0 : (k < 8 ? s1 : s2);
+        return (w >> (8 * (k & 3))) & 0xFFu;
+    };
+    if (j < 4) {
+        sc = byte_of(j) & 63u;
+        mn = byte_of(j + 4) & 63u;
+    } else {
+        const uint32_t hi = byte_of(j + 4);
+        sc = (hi & 0x0Fu) | ((byte_of(j - 4) >> 6) << 4);
+        mn = (hi >> 4) | ((byte_of(j) >> 6) << 4);
+    }
+}
+
+// The block's 32 integers as bytes in element order, with weight = scale * byte + offset.
+// Types with one scale per 16 elements return the second half's scale in scale1 (else scale1 =
+// scale).  Bytes are codes 0..31 (unsigned) or, for Q8_0 / Q6_K, signed values.
 template <int WT>
-__device__ inline void expand_q(const RawQ<WT> &r, int k0, int half, uint32_t (&q)[8], float &scale, float &neg_min) {
+__device__ inline void expand_q(const RawQ<WT> &r, int k0, int half, uint32_t (&q)[8], float &scale, float &scale1,
+                                float &offset) {
     if constexpr (WT == T_Q8_0) {
 #pragma unroll
         for (int w = 0; w < 8; w++) q[w] = r.q[w];
-        scale = half_bits_to_float((uint16_t)r.d);
-        neg_min = 0.0f;
-    } else {
+        scale = scale1 = half_bits_to_float((uint16_t)r.d);
+        offset = 0.0f;
+    } else if constexpr (WT == T_Q4_K || WT == T_Q5_K) {
         const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFFu));
         const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
-        const int j = 2 * ((k0 & 255) >> 6) + half;  // sub-block: low nibbles first, then high
+        const int c = (k0 & 255) >> 6;
+        const int j = 2 * c + half;  // sub-block: low nibbles first, then high
         uint32_t sc, mn;
-        {
-            const uint32_t s0 = r.hdr.y, s1 = r.hdr.z, s2 = r.hdr.w;
-            auto byte_of = [&](int k) -> uint32_t {
-                const uint32_t w = k < 4 ? s0 : (k < 8 ? s1 : s2);
-                return (w >> (8 * (k & 3))) & 0xFFu;
-            };
-            if (j < 4) {
-                sc = byte_of(j) & 63u;
-                mn = byte_of(j + 4) & 63u;
-            } else {
-                const uint32_t hi = byte_of(j + 4);
-                sc = (hi & 0x0Fu) | ((byte_of(j - 4) >> 6) << 4);
-                mn = (hi >> 4) | ((byte_of(j) >> 6) << 4);
-            }
-        }
-        scale = __fmul_rn(d, (float)sc);
-        neg_min = -__fmul_rn(dmin, (float)mn);
+        k4_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, j, sc, mn);
+        scale = scale1 = __fmul_rn(d, (float)sc);
+        offset = -__fmul_rn(dmin, (float)mn);
         const uint32_t qw[8] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w, r.q[1].x, r.q[1].y, r.q[1].z, r.q[1].w};
 #pragma unroll
         for (int w = 0; w < 8; w++) q[w] = half ? (qw[w] >> 4) & 0x0F0F0F0Fu : qw[w] & 0x0F0F0F0Fu;
+        if constexpr (WT == T_Q5_K) {
+            const uint32_t hw[8] = {r.qh[0].x, r.qh[0].y, r.qh[0].z, r.qh[0].w, r.qh[1].x, r.qh[1].y, r.qh[1].z, r.qh[1].w};
+#pragma unroll
+            for (int w = 0; w < 8; w++) q[w] |= ((hw[w] >> j) & 0x01010101u) << 4;
+        }
+    } else if constexpr (WT == T_Q6_K) {
+        const int within = (k0 & 255) + 32 * half, j = (within & 127) >> 5;
+        const float d = half_bits_to_float((uint16_t)r.d);
+        scale = __fmul_rn(d, (float)(int)(int8_t)(r.sc & 0xFFu));
+        scale1 = __fmul_rn(d, (float)(int)(int8_t)((r.sc >> 8) & 0xFFu));
+        offset = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const uint32_t nib = j < 2 ? r.ql[w] & 0x0F0F0F0Fu : (r.ql[w] >> 4) & 0x0F0F0F0Fu;
+            const uint32_t code = nib | (((r.qh[w] >> (2 * j)) & 0x03030303u) << 4);   // 0..63 per byte
+            q[w] = ((code | 0x80808080u) - 0x20202020u) ^ 0x80808080u;                  // minus 32, byte-wise
+        }
+    } else {  // Q4_0, Q4_1, Q5_0, Q5_1
+        const float d = half_bits_to_float((uint16_t)(r.dm & 0xFFFFu));
+        const float m = half_bits_to_float((uint16_t)(r.dm >> 16));
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            q[w] = r.q[w] & 0x0F0F0F0Fu;
+            q[4 + w] = (r.q[w] >> 4) & 0x0F0F0F0Fu;
+            if constexpr (WT == T_Q5_0 || WT == T_Q5_1) {
+                q[w] |= (((r.qh >> (4 * w)) & 0xFu) * 0x02040810u) & 0x10101010u;
+                q[4 + w] |= (((r.qh >> (16 + 4 * w)) & 0xFu) * 0x02040810u) & 0x10101010u;
+            }
+        }
+        scale = scale1 = d;
+        offset = WT == T_Q4_0 ? __fmul_rn(-8.0f, d) : (WT == T_Q5_0 ? __fmul_rn(-16.0f, d) : m);
     }
 }
 
@@ -320,8 +422,10 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
     __shared__ __attribute__((aligned(16))) uint8_t s_raw[L::kBytes];
     __shared__ __attribute__((aligned(16))) float s_as[BM];       // activation scale of this K step, per tile row
     __shared__ float s_am[BM][2];                                 // activation ssum of its two blocks
-    __shared__ float s_bd[NB][kBN][2];                            // weight block scales
-    __shared__ float s_bm[NB][kBN][2];                            // minus the weight block offsets (Q4_K)
+    constexpr bool OFFSET = gemm_has_offset(WT), SUB16 = gemm_sub16(WT);
+    constexpr int NSC = SUB16 ? 4 : 2;
+    __shared__ float s_bd[NB][kBN][NSC];                          // weight scales of the K step (per 32 or per 16 elements)
+    __shared__ float s_bm[NB][kBN][2];                            // weight block offsets (types that have one)
     auto s_a = [&](int plane, int row) -> uint8_t * { return s_raw + ((size_t)plane * BM + row) * kLdsQ; };
     auto s_b = [&](int b, int row) -> uint8_t * { return s_raw + L::kA + ((size_t)b * kBN + row) * kLdsQ; };
 
@@ -377,7 +481,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 #pragma unroll
         for (int p = 0; p < MT; p++) ra[p] = a_src[p] ? *(const uint4 *)(a_src[p] + k0) : make_uint4(0, 0, 0, 0);
         ras = as_ptr ? as_ptr[k0 >> 6] : 0.0f;
-        if (WT == T_Q4_K) ram = am_ptr ? am_ptr[k0 >> 5] : 0.0f;
+        if (OFFSET) ram = am_ptr ? am_ptr[k0 >> 5] : 0.0f;
     };
     fetch(0);
 
@@ -389,18 +493,23 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             uint32_t q[8];
-            float sc, nm;
-            expand_q<WT>(rb[b], k0, b_half, q, sc, nm);
+            float sc, sc1, nm;
+            expand_q<WT>(rb[b], k0, b_half, q, sc, sc1, nm);
             uint4 *dst = (uint4 *)(s_b(b, b_row) + b_half * 32);
             dst[0] = make_uint4(q[0], q[1], q[2], q[3]);
             dst[1] = make_uint4(q[4], q[5], q[6], q[7]);
-            s_bd[b][b_row][b_half] = sc;
-            if (WT == T_Q4_K) s_bm[b][b_row][b_half] = nm;
+            if (SUB16) {
+                s_bd[b][b_row][(2 * b_half) % NSC] = sc;
+                s_bd[b][b_row][(2 * b_half + 1) % NSC] = sc1;
+            } else {
+                s_bd[b][b_row][b_half] = sc;
+            }
+            if (OFFSET) s_bm[b][b_row][b_half] = nm;
         }
 #pragma unroll
         for (int p = 0; p < MT; p++) *(uint4 *)(s_a(a_plane, a_row[p]) + a_chunk * 16) = ra[p];
         if (tid < BM) s_as[tid] = ras;
-        if (WT == T_Q4_K && tid < 2 * BM) s_am[tid >> 1][tid & 1] = ram;
+        if (OFFSET && tid < 2 * BM) s_am[tid >> 1][tid & 1] = ram;
         MUMMU_TIMER_MARK(1);
         __syncthreads();
         MUMMU_TIMER_MARK(2);
@@ -408,36 +517,74 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
         MUMMU_TIMER_MARK(3);
 
         // multiply: wave owns columns 32*wave .. +31
+        if constexpr (!SUB16) {
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const int4v bq0 = *(const int4v *)(s_b(b, col) + 16 * g);
-            const int4v bq1 = *(const int4v *)(s_b(b, col) + 32 + 16 * g);
-            const float d0 = s_bd[b][col][0], d1 = s_bd[b][col][1];
+            for (int b = 0; b < NB; b++) {
+                const int4v bq0 = *(const int4v *)(s_b(b, col) + 16 * g);
+                const int4v bq1 = *(const int4v *)(s_b(b, col) + 32 + 16 * g);
+                const float d0 = s_bd[b][col][0], d1 = s_bd[b][col][1];
 #pragma unroll
-            for (int m = 0; m < MT; m++) {
-                const int arow = 32 * m + (lane & 31);
-                const int4v ah0 = *(const int4v *)(s_a(0, arow) + 16 * g), al0 = *(const int4v *)(s_a(1, arow) + 16 * g);
-                const int4v ah1 = *(const int4v *)(s_a(0, arow) + 32 + 16 * g), al1 = *(const int4v *)(s_a(1, arow) + 32 + 16 * g);
-                const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                const int16v ch0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah0, bq0, zero, 0, 0, 0);
-                const int16v cl0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al0, bq0, zero, 0, 0, 0);
-                const int16v ch1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah1, bq1, zero, 0, 0, 0);
-                const int16v cl1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al1, bq1, zero, 0, 0, 0);
+                for (int m = 0; m < MT; m++) {
+                    const int arow = 32 * m + (lane & 31);
+                    const int4v ah0 = *(const int4v *)(s_a(0, arow) + 16 * g), al0 = *(const int4v *)(s_a(1, arow) + 16 * g);
+                    const int4v ah1 = *(const int4v *)(s_a(0, arow) + 32 + 16 * g), al1 = *(const int4v *)(s_a(1, arow) + 32 + 16 * g);
+                    const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    const int16v ch0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah0, bq0, zero, 0, 0, 0);
+                    const int16v cl0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al0, bq0, zero, 0, 0, 0);
+                    const int16v ch1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah1, bq1, zero, 0, 0, 0);
+                    const int16v cl1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al1, bq1, zero, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
+                        const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int r = 4 * j + i;
+                            const float f0 = (float)((ch0[r] << 8) + cl0[r]);
+                            const float f1 = (float)((ch1[r] << 8) + cl1[r]);
+                            const float t = fmaf(d1, f1, __fmul_rn(d0, f0));
+                            acc[b][m][r] = fmaf(t, sr[i], acc[b][m][r]);
+                        }
+                    }
+                    if (OFFSET)
+                        acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][g], s_bm[b][col][g], acc[b][m], 0, 0, 0);
+                }
+            }
+        } else {
+            // one weight scale per 16 elements: the K step is four 16-deep integer products
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                long bq[4];
+                float dj[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
-                    const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+                    bq[j] = *(const long *)(s_b(b, col) + 16 * j + 8 * g);
+                    dj[j] = s_bd[b][col][j];
+                }
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int r = 4 * j + i;
-                        const float f0 = (float)((ch0[r] << 8) + cl0[r]);
-                        const float f1 = (float)((ch1[r] << 8) + cl1[r]);
-                        const float t = fmaf(d1, f1, __fmul_rn(d0, f0));
-                        acc[b][m][r] = fmaf(t, sr[i], acc[b][m][r]);
+                for (int m = 0; m < MT; m++) {
+                    const int arow = 32 * m + (lane & 31);
+                    float t[16];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const long ah = *(const long *)(s_a(0, arow) + 16 * j + 8 * g), al = *(const long *)(s_a(1, arow) + 16 * j + 8 * g);
+                        const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        const int16v ch = __builtin_amdgcn_mfma_i32_32x32x16_i8(ah, bq[j], zero, 0, 0, 0);
+                        const int16v cl = __builtin_amdgcn_mfma_i32_32x32x16_i8(al, bq[j], zero, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const float f = (float)((ch[r] << 8) + cl[r]);
+                            t[r] = j == 0 ? __fmul_rn(dj[0], f) : fmaf(dj[j], f, t[r]);
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
+                        const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc[b][m][4 * j + i] = fmaf(t[4 * j + i], sr[i], acc[b][m][4 * j + i]);
                     }
                 }
-                if (WT == T_Q4_K)
-                    acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][g], s_bm[b][col][g], acc[b][m], 0, 0, 0);
             }
         }
         MUMMU_TIMER_MARK(4);
@@ -495,7 +642,7 @@ hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStr
     return hipGetLastError();
 }
 
-static bool gemm_q_type(int t) { return t == T_Q8_0 || t == T_Q4_K; }
+static bool gemm_q_type(int t) { return is_quant_type(t); }
 
 bool grouped_gemm_quantized(const ExpertBanks &b) {
     return gemm_q_type(b.gate_type) && b.gate_type == b.up_type && gemm_q_type(b.down_type);
@@ -561,11 +708,22 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     if (b.gate_type == T_F16)
         return launch_gemm_f16<true>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
                                      b.inter, (_Float16 *)act16, nullptr, s);
-    if (b.gate_type == T_Q8_0)
-        return launch_gemm_q<T_Q8_0, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
-                                           b.inter, actq, nullptr, s);
-    return launch_gemm_q<T_Q4_K, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
-                                       b.inter, actq, nullptr, s);
+    switch (b.gate_type) {
+#define MUMMU_GU(T)                                                                                                          \
+    case T:                                                                                                                  \
+        return launch_gemm_q<T, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden, b.inter, \
+                                      actq, nullptr, s)
+        MUMMU_GU(T_Q8_0);
+        MUMMU_GU(T_Q4_K);
+        MUMMU_GU(T_Q4_0);
+        MUMMU_GU(T_Q4_1);
+        MUMMU_GU(T_Q5_0);
+        MUMMU_GU(T_Q5_1);
+        MUMMU_GU(T_Q5_K);
+        MUMMU_GU(T_Q6_K);
+#undef MUMMU_GU
+    default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, const int32_t *tiles,
@@ -574,11 +732,22 @@ hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq
     if (b.down_type == T_F16)
         return launch_gemm_f16<false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
                                       tile_rows, b.inter, b.hidden, nullptr, y, s);
-    if (b.down_type == T_Q8_0)
-        return launch_gemm_q<T_Q8_0, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter,
-                                            b.hidden, QAct64(), y, s);
-    return launch_gemm_q<T_Q4_K, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter,
-                                        b.hidden, QAct64(), y, s);
+    switch (b.down_type) {
+#define MUMMU_DN(T)                                                                                                      \
+    case T:                                                                                                              \
+        return launch_gemm_q<T, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter, b.hidden, \
+                                       QAct64(), y, s)
+        MUMMU_DN(T_Q8_0);
+        MUMMU_DN(T_Q4_K);
+        MUMMU_DN(T_Q4_0);
+        MUMMU_DN(T_Q4_1);
+        MUMMU_DN(T_Q5_0);
+        MUMMU_DN(T_Q5_1);
+        MUMMU_DN(T_Q5_K);
+        MUMMU_DN(T_Q6_K);
+#undef MUMMU_DN
+    default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace mummu

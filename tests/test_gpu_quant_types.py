@@ -101,20 +101,39 @@ def test_mixed_type_banks_match_the_oracle(gt, dt, H, I, E, k):
     assert np.array_equal(down_e.view(np.uint32), od.view(np.uint32))
 
 
-def test_many_tokens_with_a_type_the_matrix_core_path_does_not_cover_still_match():
-    # 300 tokens take the per-assignment kernels when a bank type has no grouped GEMM
-    gt, dt, H, I, E, k, n = M.Q5_K, M.Q6_K, 512, 256, 8, 2, 300
-    gate = synth.random_bank_fast(gt, [H, I, E], 1)
-    up = synth.random_bank_fast(gt, [H, I, E], 2)
-    down = synth.random_bank_fast(dt, [I, H, E], 3)
+# many tokens: dispatch + grouped GEMM on the int8 matrix cores, every block type on either side
+PREFILL = [
+    (M.Q5_K, M.Q6_K, 512, 256, 8, 2, 300),
+    (M.Q6_K, M.Q5_K, 512, 256, 8, 2, 300),
+    (M.Q4_0, M.Q4_1, 512, 256, 8, 2, 130),
+    (M.Q4_1, M.Q4_0, 512, 256, 8, 2, 77),
+    (M.Q5_0, M.Q5_1, 512, 256, 8, 4, 200),
+    (M.Q5_1, M.Q5_0, 512, 256, 8, 2, 515),
+    (M.Q4_K, M.Q6_K, 1024, 512, 16, 4, 1027),
+    (M.Q5_K, M.Q5_1, 2560, 640, 32, 10, 96),   # qwen4exp geometry, top-10
+    (M.Q4_K, M.Q5_1, 512, 96, 8, 2, 300),      # 96-wide rows are not whole 64-element K steps: per-assignment kernels
+]
+
+
+@pytest.mark.parametrize("gt,dt,H,I,E,k,n", PREFILL, ids=[f"{NAME[c[0]]}-{NAME[c[1]]}-{c[2]}x{c[3]}-{c[6]}" for c in PREFILL])
+def test_many_tokens_match_the_oracle_for_every_block_type(gt, dt, H, I, E, k, n):
+    gate = synth.random_bank_fast(gt, [H, I, E], 1 + gt)
+    up = synth.random_bank_fast(gt, [H, I, E], 2 + gt)
+    down = synth.random_bank_fast(dt, [I, H, E], 3 + dt)
     router = normal((E, H), 4, 0.05).astype(np.float16)
     x = normal((n, H), 5)
     with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=n) as m:
         m.load_layer(0, router, M.F16, gate, gt, up, gt, down, dt)
         got = m.forward(x, k, False)
         hits = m.take_hits()
+        ids, w = m.last_routing(n, k)
+        again = m.forward(x, k, False)
     banks = orc.LayerBanks(H, I, E, gate, up, down, gt, gt, dt)
     _, oids, ow, _ = orc.moe_forward(banks, router, orc.F16, x, k, False)
+    assert np.array_equal(ids, oids.astype(np.int32))
+    assert np.array_equal(w.view(np.uint32), ow.view(np.uint32))
     assert hits.tolist() == np.bincount(oids.reshape(-1), minlength=E).tolist()
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
     want, mag = orc.moe_ref_f64(banks, oids, ow, x)
-    assert orc.rel_err(got, want, mag).max() <= 2e-3
+    err = orc.rel_err(got, want, mag)
+    assert err.max() <= 2e-3, f"max relative error {err.max():.3e}"
