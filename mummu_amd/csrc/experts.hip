@@ -410,163 +410,6 @@ __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Expert-major kernels for a handful of tokens (quantized banks, rows of at most 64 units):
-// blockIdx.x = expert, blockIdx.y = tile of output rows.  The workgroup lists the assignments
-// routed to its expert, loads its rows of the expert's weights ONCE and multiplies them with every
-// listed token in turn, so an expert shared by several tokens is read once instead of once per
-// token.  Per (token, row) the lanes, the integer dots and the reduction are those of the
-// token-major kernels above: a token's result is bit-identical on either path.
-// ------------------------------------------------------------------------------------------
-constexpr int kXMaxAssign = 1024;
-
-// Ascending list of the assignments a (= token*k + slot) with ids[a] == e, by wave 0; returns the
-// count to every thread.  Ends with a workgroup barrier.
-__device__ inline int list_assignments(const int32_t *__restrict__ ids, int n_assign, int e, int n_experts, int *s_list,
-                                       int *s_count, int32_t *__restrict__ flags, bool check_ids) {
-    const int lane = threadIdx.x & 63;
-    if (threadIdx.x < 64) {
-        int v[kXMaxAssign / 64];
-#pragma unroll
-        for (int c = 0; c < kXMaxAssign / 64; c++) v[c] = 64 * c + lane < n_assign ? ids[64 * c + lane] : -1;
-        int cnt = 0;
-        bool bad = false;
-#pragma unroll
-        for (int c = 0; c < kXMaxAssign / 64; c++) {
-            if (64 * c < n_assign) {
-                const bool hit = v[c] == e;
-                bad = bad || (64 * c + lane < n_assign && (unsigned)v[c] >= (unsigned)n_experts);
-                const unsigned long long m = __ballot(hit);
-                if (hit) s_list[cnt + __popcll(m & ((1ull << lane) - 1ull))] = 64 * c + lane;
-                cnt += __popcll(m);
-            }
-        }
-        if (check_ids && __any(bad) && lane == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
-        if (lane == 0) *s_count = cnt;
-    }
-    __syncthreads();
-    return *s_count;
-}
-
-template <int WT, int NIT>
-__global__ __launch_bounds__(1024) void gate_up_xq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
-                                                          QAct xq, const int32_t *__restrict__ ids, int n_assign, int k,
-                                                          int hidden, int inter, int n_experts, QAct actq,
-                                                          int32_t *__restrict__ flags) {
-    extern __shared__ float s_act[];  // 2 * rows_per_block floats (double-buffered over the tokens)
-    __shared__ int s_list[kXMaxAssign];
-    __shared__ int s_count;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int e = blockIdx.x;
-    const int cnt = list_assignments(ids, n_assign, e, n_experts, s_list, &s_count, flags, blockIdx.x == 0 && blockIdx.y == 0);
-    if (cnt == 0) return;
-    const RowSplit rs = row_split(hidden);
-    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
-    const int rows_per_wave = NIT * rs.rows_per_it;
-    const int rows_per_block = rows_per_wave * (blockDim.x >> 6);
-    const int block_row0 = blockIdx.y * rows_per_block;
-    const int row0 = block_row0 + wave * rows_per_wave;
-    const size_t row_bytes = type_row_bytes(WT, hidden);
-    const uint8_t *ge = gate + (size_t)e * (size_t)inter * row_bytes;
-    const uint8_t *ue = up + (size_t)e * (size_t)inter * row_bytes;
-
-    LaneAct<1> la;
-    load_lane_act<WT, 1>(xq, (size_t)(s_list[0] / k), hidden, unit0, rs.units, la);
-    RawRow<WT, 1> rg[NIT], ru[NIT];
-#pragma unroll
-    for (int i = 0; i < NIT; i++) {
-        const int row = row0 + i * rs.rows_per_it + sub;
-        const bool ok = row < inter;
-        load_row<WT, 1>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
-        load_row<WT, 1>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
-    }
-    for (int j = 0; j < cnt; j++) {
-        const int a = s_list[j];
-        LaneAct<1> nxt = la;
-        if (j + 1 < cnt) load_lane_act<WT, 1>(xq, (size_t)(s_list[j + 1] / k), hidden, unit0, rs.units, nxt);
-        float part[2 * NIT];
-#pragma unroll
-        for (int i = 0; i < NIT; i++) {
-            part[2 * i] = dot_row<WT, 1>(rg[i], unit0, la);
-            part[2 * i + 1] = dot_row<WT, 1>(ru[i], unit0, la);
-        }
-        float *s_cur = s_act + (j & 1) * rows_per_block;
-        dispatch_group(rs.group, [&](auto group_tag) {
-            constexpr int GROUP = decltype(group_tag)::value;
-            constexpr int count = reduced_count<2 * NIT, GROUP>();
-            static_assert(count >= 2, "gate and up sums of a row must meet in one lane");
-            const int offset = reduce_partials<2 * NIT, GROUP>(part, lane);
-            constexpr int width = GROUP < 16 ? GROUP : 16;
-            if ((lane & (width - 1)) == 0) {
-#pragma unroll
-                for (int jj = 0; jj < count; jj += 2) {
-                    const int row = row0 + ((offset + jj) >> 1) * rs.rows_per_it + sub;
-                    if (row < inter) s_cur[row - block_row0] = __fmul_rn(det_silu(part[jj]), part[jj + 1]);
-                }
-            }
-        });
-        __syncthreads();  // one barrier per token: the buffer written two tokens ago is free again
-        for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
-            const int row = block_row0 + r;
-            const bool on = row < inter;
-            quantize_store16(on ? s_cur[r] : 0.0f, on, actq, (size_t)a, inter, on ? row : 0);
-        }
-        la = nxt;
-    }
-}
-
-template <int WT, int NIT>
-__global__ __launch_bounds__(64 * kGemvWaves) void down_xq_kernel(const uint8_t *__restrict__ down, QAct actq,
-                                                                  const int32_t *__restrict__ ids, int n_assign,
-                                                                  int hidden, int inter, int n_experts,
-                                                                  float *__restrict__ y) {
-    __shared__ int s_list[kXMaxAssign];
-    __shared__ int s_count;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int e = blockIdx.x;
-    const int cnt = list_assignments(ids, n_assign, e, n_experts, s_list, &s_count, nullptr, false);
-    if (cnt == 0) return;
-    const RowSplit rs = row_split(inter);
-    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
-    const int rows_per_wave = NIT * rs.rows_per_it;
-    const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
-    const size_t row_bytes = type_row_bytes(WT, inter);
-    const uint8_t *de = down + (size_t)e * (size_t)hidden * row_bytes;
-
-    LaneAct<1> la;
-    load_lane_act<WT, 1>(actq, (size_t)s_list[0], inter, unit0, rs.units, la);
-    RawRow<WT, 1> rd[NIT];
-#pragma unroll
-    for (int i = 0; i < NIT; i++) {
-        const int row = row0 + i * rs.rows_per_it + sub;
-        const bool ok = row < hidden;
-        load_row<WT, 1>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i]);
-    }
-    for (int j = 0; j < cnt; j++) {
-        const int a = s_list[j];
-        LaneAct<1> nxt = la;
-        if (j + 1 < cnt) load_lane_act<WT, 1>(actq, (size_t)s_list[j + 1], inter, unit0, rs.units, nxt);
-        float part[NIT];
-#pragma unroll
-        for (int i = 0; i < NIT; i++) part[i] = dot_row<WT, 1>(rd[i], unit0, la);
-        float *yrow = y + (size_t)a * (size_t)hidden;
-        dispatch_group(rs.group, [&](auto group_tag) {
-            constexpr int GROUP = decltype(group_tag)::value;
-            const int offset = reduce_partials<NIT, GROUP>(part, lane);
-            constexpr int count = reduced_count<NIT, GROUP>();
-            constexpr int width = GROUP < 16 ? GROUP : 16;
-            if ((lane & (width - 1)) == 0) {
-#pragma unroll
-                for (int jj = 0; jj < count; jj++) {
-                    const int row = row0 + (offset + jj) * rs.rows_per_it + sub;
-                    if (row < hidden) yrow[row] = part[jj];
-                }
-            }
-        });
-        la = nxt;
-    }
-}
-
-// ------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------
 // Float rows: rows per wave so that a launch has a few thousand waves without tiny tiles.
@@ -756,53 +599,6 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
         constexpr int WT = decltype(tag)::value;
         if constexpr (is_quant_type(WT)) return launch_down_combine_t<WT>(b, actq, ids, weights, n, k, residual, out, s);
         else return hipErrorInvalidValue;
-    });
-}
-
-bool expert_major_supported(const ExpertBanks &b, int n_assign) {
-    return is_quant_type(b.gate_type) && b.gate_type == b.up_type && is_quant_type(b.down_type) &&
-           row_split(b.hidden).units <= 64 && row_split(b.inter).units <= 64 && b.inter % 16 == 0 && n_assign <= kXMaxAssign &&
-           b.n_experts <= 65535;
-}
-
-hipError_t launch_gate_up_expert_major(const ExpertBanks &b, QAct xq, const int32_t *ids, int n_assign, int k, QAct actq,
-                                       int32_t *flags, hipStream_t s) {
-    if (n_assign <= 0) return hipSuccess;
-    if (!expert_major_supported(b, n_assign)) return hipErrorInvalidValue;
-    const RowSplit rs = row_split(b.hidden);
-    constexpr int NIT = 4;
-    int waves = 4;
-    while (waves * NIT * rs.rows_per_it < 16) waves *= 2;
-    const int rpb = waves * NIT * rs.rows_per_it;
-    dim3 grid(b.n_experts, (b.inter + rpb - 1) / rpb), block(64 * waves);
-    const size_t lds = sizeof(float) * 2 * (size_t)rpb;
-    return with_bank_type(b.gate_type, [&](auto tag) {
-        constexpr int WT = decltype(tag)::value;
-        if constexpr (is_quant_type(WT)) {
-            launch_kernel(gate_up_xq_kernel<WT, NIT>, grid, block, lds, s, b.gate, b.up, xq, ids, n_assign, k, b.hidden, b.inter,
-                          b.n_experts, actq, flags);
-            return hipGetLastError();
-        } else {
-            return hipErrorInvalidValue;
-        }
-    });
-}
-
-hipError_t launch_down_expert_major(const ExpertBanks &b, QAct actq, const int32_t *ids, int n_assign, float *y, hipStream_t s) {
-    if (n_assign <= 0) return hipSuccess;
-    if (!expert_major_supported(b, n_assign)) return hipErrorInvalidValue;
-    const RowSplit rs = row_split(b.inter);
-    constexpr int NIT = 4;
-    const int rpb = kGemvWaves * NIT * rs.rows_per_it;
-    dim3 grid(b.n_experts, (b.hidden + rpb - 1) / rpb), block(64 * kGemvWaves);
-    return with_bank_type(b.down_type, [&](auto tag) {
-        constexpr int WT = decltype(tag)::value;
-        if constexpr (is_quant_type(WT)) {
-            launch_kernel(down_xq_kernel<WT, NIT>, grid, block, 0, s, b.down, actq, ids, n_assign, b.hidden, b.inter, b.n_experts, y);
-            return hipGetLastError();
-        } else {
-            return hipErrorInvalidValue;
-        }
     });
 }
 

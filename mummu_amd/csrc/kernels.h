@@ -74,14 +74,6 @@ hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const 
 // inv (nullable): y row of assignment a is inv[a] instead of a (dispatch-sorted layout).
 hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, const int32_t *inv, int n, int k,
                           int hidden, const float *residual, float *out, hipStream_t s);
-// Expert-major gate/up and down for a handful of tokens: a launch covers every expert, each
-// workgroup finds the assignments of its expert in ids[n_assign] and reads the expert's rows once
-// for all of them.  Same bits per (token, expert) as the kernels above.  Quantized banks, rows of
-// at most 2048 elements, n_assign <= 1024.
-bool expert_major_supported(const ExpertBanks &b, int n_assign);
-hipError_t launch_gate_up_expert_major(const ExpertBanks &b, QAct xq, const int32_t *ids, int n_assign, int k, QAct actq,
-                                       int32_t *flags, hipStream_t s);
-hipError_t launch_down_expert_major(const ExpertBanks &b, QAct actq, const int32_t *ids, int n_assign, float *y, hipStream_t s);
 // down + combine in one launch (no y round trip): quantized down bank and top_k <= 16.
 bool down_combine_supported(const ExpertBanks &b, int k);
 hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,

@@ -68,7 +68,6 @@ struct mummu_moe {
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
     int gemm_min_tokens = 32;    // batches at least this large take the grouped GEMM
-    int xmajor_min_tokens = 3;   // batches at least this large (and below the GEMM's) take the expert-major kernels
 
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing = false;
@@ -273,13 +272,6 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
     }
     if (is_quant_type(b.gate_type) && !x_quantized)
         LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x, (int)n, b.hidden, h->xq, s));
-    if (n >= h->xmajor_min_tokens && expert_major_supported(b, na)) {
-        // a handful of tokens: every expert's rows are read once for all the tokens routed to it
-        LAUNCH(h, K_GATE_UP, s, launch_gate_up_expert_major(b, h->xq, h->ids, na, k, h->actq, h->flags, s));
-        LAUNCH(h, K_DOWN, s, launch_down_expert_major(b, h->actq, h->ids, na, h->y, s));
-        LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, nullptr, (int)n, k, b.hidden, residual, out, s));
-        return MUMMU_OK;
-    }
     LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x, h->xq, h->ids, na, k, -1, h->act, h->actq, h->flags, s));
     if (down_combine_supported(b, k)) {
         LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, k, residual, out, s));
@@ -309,8 +301,7 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
         // few tokens: the router rows are spread over as many CUs as there are experts
         LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s));
         const ExpertBanks b = banks_of(h, L);
-        const bool xmajor = n >= h->xmajor_min_tokens && expert_major_supported(b, (int)(n * k));
-        if (!xmajor && want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
+        if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
             // ... and the gate/up kernel routes by itself: one launch less on the decode path
             RouteInline route;
             route.logits = h->logits;
