@@ -70,6 +70,16 @@ static __device__ long long *g_trace_buf = nullptr;
 #define MUMMU_TIMER_STORE do { } while (0)
 #endif
 
+// Keeps code on either side where it was written: the compiler may not move memory accesses
+// across it (so a prefetch stays issued early instead of being sunk next to its first use) and
+// the instruction scheduler may not move anything across it.  Emits no instruction and waits for
+// nothing.
+#define MUMMU_CODE_FENCE()                      \
+    do {                                        \
+        asm volatile("" ::: "memory");          \
+        __builtin_amdgcn_sched_barrier(0);      \
+    } while (0)
+
 // ggml tensor type ids (the values stored in GGUF tensor tables).
 enum : int {
     T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8,

@@ -129,16 +129,16 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     constexpr int AHEAD = NIT < 2 ? NIT : 2;
 #pragma unroll
     for (int i = 0; i < AHEAD; i++) fetch(i);
-    __builtin_amdgcn_sched_barrier(0);
+    MUMMU_CODE_FENCE();
     MUMMU_PHASE(1);
     float part[2 * NIT];
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
         if (i + AHEAD < NIT) fetch(i + AHEAD);
-        __builtin_amdgcn_sched_barrier(0);
+        MUMMU_CODE_FENCE();
         part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
         part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
-        __builtin_amdgcn_sched_barrier(0);
+        MUMMU_CODE_FENCE();
     }
     MUMMU_PHASE(2);
     dispatch_group(rs.group, [&](auto group_tag) {
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_f_kernel(const uint8_t *
 // ------------------------------------------------------------------------------------------
 template <int WT, int UPL, int NIT, int KPW, int kDcWaves = 4>
 __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
-    const uint8_t *__restrict__ down, QAct actq, const int32_t *__restrict__ ids, const float *__restrict__ weights,
+    const uint8_t *down /* not __restrict__: the code fences below must order its loads */, QAct actq, const int32_t *__restrict__ ids, const float *__restrict__ weights,
     int k, int hidden, int inter, int n_experts, const float *__restrict__ residual, float *__restrict__ out) {
     constexpr int KMAX = kDcWaves * KPW;
     extern __shared__ float s_mem[];  // [KMAX][rows_per_block] row sums, then [KMAX] weights
@@ -371,14 +371,14 @@ __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
     for (int i = 0; i < KPW; i++) load_lane_act<WT, UPL>(actq, (size_t)(on_p[i] ? a_p[i] : 0), inter, unit0, rs.units, la[i]);
 #pragma unroll
     for (int st = 0; st < AHEAD; st++) fetch(st);
-    __builtin_amdgcn_sched_barrier(0);
+    MUMMU_CODE_FENCE();
     float part[KPW * NIT];
 #pragma unroll
     for (int st = 0; st < STEPS; st++) {
         if (st + AHEAD < STEPS) fetch(st + AHEAD);
-        __builtin_amdgcn_sched_barrier(0);
+        MUMMU_CODE_FENCE();
         part[st] = dot_row<WT, UPL>(rd[st / NIT][st % NIT], unit0, la[st / NIT]);
-        __builtin_amdgcn_sched_barrier(0);
+        MUMMU_CODE_FENCE();
     }
     MUMMU_PHASE(2);
     dispatch_group(rs.group, [&](auto group_tag) {

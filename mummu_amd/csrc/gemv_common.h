@@ -52,8 +52,9 @@ template <int UPL>
 struct LaneAct {
     int xh[UPL][8];   // hi bytes, 4 per word: words 0-3 first half, 4-7 second half
     int xl[UPL][8];   // lo bytes
-    float s[UPL][2];  // scale of each half
-    int sx[UPL][2];   // sum(xq) of each half
+    float s[UPL][2];    // scale of each half
+    int sx[UPL][2];     // sum(xq) of each half
+    float fsx[UPL][2];  // scale * sum(xq) of each half (what a block offset multiplies)
 };
 
 template <int WT, int UPL>
@@ -78,6 +79,8 @@ __device__ inline void load_lane_act(const QAct &q, size_t row, int d, int unit0
         a.s[i][1] = on ? sc[e1 >> 4] : 0.0f;
         a.sx[i][0] = on ? sm[e0 >> 4] : 0;
         a.sx[i][1] = on ? sm[e1 >> 4] : 0;
+        a.fsx[i][0] = __fmul_rn(a.s[i][0], (float)a.sx[i][0]);
+        a.fsx[i][1] = __fmul_rn(a.s[i][1], (float)a.sx[i][1]);
     }
 }
 
@@ -185,6 +188,19 @@ __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int
     }
 }
 
+// The 6-bit (scale, min) of sub-blocks 2c and 2c+1 of a Q4_K / Q5_K super-block (ggml
+// get_scale_min_k4), each pair packed as two bytes (sub-block 2c in byte 0), without a branch:
+// y, z, w are the three words of the 12 scale bytes.
+__device__ inline void k4_scale_min_pair(uint32_t y, uint32_t z, uint32_t w, int c, uint32_t &sc, uint32_t &mn) {
+    const int sh = 16 * (c & 1);
+    const uint32_t a = y >> sh, b = z >> sh, p = w >> sh;
+    const uint32_t lo_sc = a & 0x3F3Fu, lo_mn = b & 0x3F3Fu;                   // sub-blocks 0..3: bytes j and j+4
+    const uint32_t hi_sc = (p & 0x0F0Fu) | ((a >> 2) & 0x3030u);              // sub-blocks 4..7: low nibble of byte j+4,
+    const uint32_t hi_mn = ((p >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);       // top two bits of byte j-4 (scale) / j (min)
+    sc = c < 2 ? lo_sc : hi_sc;
+    mn = c < 2 ? lo_mn : hi_mn;
+}
+
 // The lane's partial of <row, activation> (formulas in the file comment).  A lane that loaded
 // nothing holds zero scales and contributes exactly 0.
 template <int WT, int UPL>
@@ -197,22 +213,11 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
             const uint4 hdr = r.hdr[i];
             const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFFu));
             const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
-            // 6-bit (scale, min) of sub-blocks 2c, 2c+1 (ggml get_scale_min_k4), c fixed per lane
-            const int c = (u & 7) >> 1;
-            const int sh = 16 * (c & 1);
-            int sc0, sc1, mn0, mn1;
-            if (c < 2) {
-                sc0 = (int)((hdr.y >> sh) & 63u);
-                sc1 = (int)((hdr.y >> (sh + 8)) & 63u);
-                mn0 = (int)((hdr.z >> sh) & 63u);
-                mn1 = (int)((hdr.z >> (sh + 8)) & 63u);
-            } else {
-                const uint32_t lo = hdr.w >> sh;
-                sc0 = (int)((lo & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4));
-                mn0 = (int)(((lo >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4));
-                sc1 = (int)(((lo >> 8) & 0xFu) | (((hdr.y >> (sh + 14)) & 3u) << 4));
-                mn1 = (int)(((lo >> 12) & 0xFu) | (((hdr.z >> (sh + 14)) & 3u) << 4));
-            }
+            // 6-bit (scale, min) of sub-blocks 2c, 2c+1, c fixed per lane
+            uint32_t scp, mnp;
+            k4_scale_min_pair(hdr.y, hdr.z, hdr.w, (u & 7) >> 1, scp, mnp);
+            const float sc0 = (float)(scp & 0xFFu), sc1 = (float)((scp >> 8) & 0xFFu);
+            const float mn0 = (float)(mnp & 0xFFu), mn1 = (float)((mnp >> 8) & 0xFFu);
             const uint32_t q[4] = {r.q[i].x, r.q[i].y, r.q[i].z, r.q[i].w};
             int lh = 0, ll = 0, hh = 0, hl = 0;
 #pragma unroll
@@ -224,12 +229,12 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
                 hh = __builtin_amdgcn_sdot4(hi, a.xh[i][4 + w], hh, false);
                 hl = __builtin_amdgcn_sdot4(hi, a.xl[i][4 + w], hl, false);
             }
-            // |sum(q*xq)| <= 15*32512*16 < 2^23 and |sum(xq)| <= 16*32512: 24-bit multiplies are exact
-            const float p0 = (float)__mul24(sc0, lh * 256 + ll), p1 = (float)__mul24(sc1, hh * 256 + hl);
-            const float n0 = (float)__mul24(mn0, a.sx[i][0]), n1 = (float)__mul24(mn1, a.sx[i][1]);
-            const float pos = __builtin_fmaf(a.s[i][0], p0, __fmul_rn(a.s[i][1], p1));
-            const float neg = __builtin_fmaf(a.s[i][0], n0, __fmul_rn(a.s[i][1], n1));
-            acc = __fadd_rn(acc, __builtin_fmaf(-dmin, neg, __fmul_rn(d, pos)));
+            // |sum(q*xq)| <= 15*32512*16 < 2^23: exact in f32
+            const float p0 = (float)(lh * 256 + ll), p1 = (float)(hh * 256 + hl);
+            const float pos = __builtin_fmaf(__fmul_rn(a.s[i][1], sc1), p1, __fmul_rn(__fmul_rn(a.s[i][0], sc0), p0));
+            const float neg = __builtin_fmaf(a.fsx[i][1], mn1, __fmul_rn(a.fsx[i][0], mn0));
+            acc = __builtin_fmaf(d, pos, acc);
+            acc = __builtin_fmaf(-dmin, neg, acc);
         } else if constexpr (WT != T_Q8_0) {
             // Every other type: the two 16-element halves as non-negative byte codes c0, c1 with
             //     weight = A_h * code + B_h,
@@ -257,20 +262,10 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
                 const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFFu));
                 const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
                 const int c = (u & 7) >> 1;
-                const int sh = 16 * (c & 1);
-                int sc0, sc1, mn0, mn1;
-                if (c < 2) {
-                    sc0 = (int)((hdr.y >> sh) & 63u);
-                    sc1 = (int)((hdr.y >> (sh + 8)) & 63u);
-                    mn0 = (int)((hdr.z >> sh) & 63u);
-                    mn1 = (int)((hdr.z >> (sh + 8)) & 63u);
-                } else {
-                    const uint32_t lo = hdr.w >> sh;
-                    sc0 = (int)((lo & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4));
-                    mn0 = (int)(((lo >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4));
-                    sc1 = (int)(((lo >> 8) & 0xFu) | (((hdr.y >> (sh + 14)) & 3u) << 4));
-                    mn1 = (int)(((lo >> 12) & 0xFu) | (((hdr.z >> (sh + 14)) & 3u) << 4));
-                }
+                uint32_t scp, mnp;
+                k4_scale_min_pair(hdr.y, hdr.z, hdr.w, c, scp, mnp);
+                const float sc0 = (float)(scp & 0xFFu), sc1 = (float)((scp >> 8) & 0xFFu);
+                const float mn0 = (float)(mnp & 0xFFu), mn1 = (float)((mnp >> 8) & 0xFFu);
                 const uint32_t q[4] = {r.q[i].x, r.q[i].y, r.q[i].z, r.q[i].w};
                 const uint32_t h[4] = {r.qh[i].x, r.qh[i].y, r.qh[i].z, r.qh[i].w};
 #pragma unroll
@@ -278,10 +273,10 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
                     c0[w] = (q[w] & 0x0F0F0F0Fu) | (((h[w] >> (2 * c)) & 0x01010101u) << 4);
                     c1[w] = ((q[w] >> 4) & 0x0F0F0F0Fu) | (((h[w] >> (2 * c + 1)) & 0x01010101u) << 4);
                 }
-                A0 = __fmul_rn(d, (float)sc0);
-                A1 = __fmul_rn(d, (float)sc1);
-                B0 = -__fmul_rn(dmin, (float)mn0);
-                B1 = -__fmul_rn(dmin, (float)mn1);
+                A0 = __fmul_rn(d, sc0);
+                A1 = __fmul_rn(d, sc1);
+                B0 = -__fmul_rn(dmin, mn0);
+                B1 = -__fmul_rn(dmin, mn1);
             } else {  // Q6_K
                 const int u = unit0 + 64 * i;
                 const int jj = ((u & 7) >> 1) & 1;  // which pair of 2-bit fields of qh: (0, 4) or (2, 6)
@@ -305,10 +300,10 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
                 l1 = __builtin_amdgcn_sdot4((int)c1[w], a.xl[i][4 + w], l1, false);
             }
             // codes <= 63 and |xq| <= 32512: every integer sum fits 32 bits
-            const float t0 = __builtin_fmaf(A0, (float)(h0 * 256 + l0), __fmul_rn(B0, (float)a.sx[i][0]));
-            const float t1 = __builtin_fmaf(A1, (float)(h1 * 256 + l1), __fmul_rn(B1, (float)a.sx[i][1]));
-            acc = __builtin_fmaf(a.s[i][0], t0, acc);
-            acc = __builtin_fmaf(a.s[i][1], t1, acc);
+            acc = __builtin_fmaf(__fmul_rn(a.s[i][0], A0), (float)(h0 * 256 + l0), acc);
+            acc = __builtin_fmaf(__fmul_rn(a.s[i][1], A1), (float)(h1 * 256 + l1), acc);
+            acc = __builtin_fmaf(a.fsx[i][0], B0, acc);
+            acc = __builtin_fmaf(a.fsx[i][1], B1, acc);
         } else {  // Q8_0
             const float d = half_bits_to_float((uint16_t)r.d[i]);
             int h0 = 0, l0 = 0, h1 = 0, l1 = 0;
