@@ -57,7 +57,8 @@ enum mummu_status {
     MUMMU_ERR_DEVICE = 10,    /* no HIP device / a HIP call failed */
     MUMMU_ERR_ARG = 11,       /* null pointer or otherwise unusable argument */
     MUMMU_ERR_IO = 12,        /* a file cannot be opened, read or mapped, or ends inside its header */
-    MUMMU_ERR_GGUF = 13       /* the GGUF container breaks one of the reader's rules (gguf.rs:1226-1376) */
+    MUMMU_ERR_GGUF = 13,      /* the GGUF container breaks one of the reader's rules (gguf.rs:1226-1376) */
+    MUMMU_ERR_SAFETENSORS = 14 /* a safetensors header, index or expert group breaks a rule (safetensors.rs:180-320, 600-740) */
 };
 
 /* Router arithmetic.  0: SparseMoe / SparseMoePerExpert (nn/moe.rs:144-150: f32 softmax,
@@ -230,6 +231,51 @@ MUMMU_API int mummu_gguf_locate_moe_layer(const mummu_gguf *g, int layer, mummu_
  * handle's layers 0..n_layers through mummu_moe_load_layer, payload bytes unchanged (mapped
  * read-only from their shard, offsets relative to that shard's own payload base). */
 MUMMU_API int mummu_moe_load_gguf(mummu_moe *h, mummu_gguf *g, int first_layer, int n_layers);
+
+/* ---- HF safetensors checkpoint directories (host side) -----------------------------------
+ * checkpoint_shards + SafetensorsHeader::open (safetensors.rs:180-320, 377-430): a single
+ * `model.safetensors` or the shards `model.safetensors.index.json` names (at most 256, each
+ * checked to be on disk); every header entry checked against the payload it claims (header
+ * <= 64 MiB, <= 2^20 entries, known dtype, integer dims, offsets inside the payload, shape
+ * bytes == claimed bytes).  `config.json` of the same directory is parsed as OlmoeConfig. */
+typedef struct mummu_st mummu_st;
+
+/* TensorEntry (safetensors.rs:122-148) plus where its payload lies. */
+typedef struct mummu_st_tensor {
+    const char *name;
+    const char *dtype;    /* "F32", "F16", "BF16", ... */
+    int32_t n_dims;
+    int64_t dims[8];      /* row-major, outermost first, padded with 1 */
+    int32_t shard;
+    uint64_t file_offset; /* absolute offset in that shard's file */
+    uint64_t nbytes;
+    const char *path;
+} mummu_st_tensor;
+
+MUMMU_API const char *mummu_st_last_error(void);
+MUMMU_API int mummu_st_open(const char *dir, mummu_st **out);
+MUMMU_API void mummu_st_close(mummu_st *st);
+MUMMU_API int mummu_st_shard_count(const mummu_st *st);
+MUMMU_API int mummu_st_tensor_count(const mummu_st *st);
+MUMMU_API int mummu_st_find_tensor(const mummu_st *st, const char *name);
+MUMMU_API int mummu_st_tensor_info(const mummu_st *st, int index, mummu_st_tensor *out);
+/* OlmoeConfig::from_json_bytes (models/olmoe.rs:52-115, validation :180-226), the fields the MoE
+ * block reads: hidden_size, intermediate_size, num_experts, num_experts_per_tok, norm_topk_prob
+ * (default false), rms_norm_eps, num_hidden_layers; refuses E < 2, top-k outside 1..=E, zero
+ * layers or vocab, heads that do not divide.  (Rope scaling and sliding windows belong to the
+ * attention side and are not judged here.) */
+MUMMU_API int mummu_olmoe_config_from_json(const char *json, size_t len, mummu_moe_config *cfg);
+/* The same from the directory's config.json. */
+MUMMU_API int mummu_st_moe_config(const mummu_st *st, mummu_moe_config *cfg);
+/* olmoe_hf_fuse (models/olmoe.rs:405-430) as a check, no payload read: layer L has
+ * `model.layers.L.mlp.gate.weight` [E,H], optional `post_attention_layernorm.weight` [H], and for
+ * each of gate/up/down exactly the members `mlp.experts.{0..E-1}.*_proj.weight`, all of one float
+ * dtype and of the shape the config implies (group rules of safetensors.rs:600-740). */
+MUMMU_API int mummu_st_check_moe_layer(const mummu_st *st, int layer);
+/* load_from_dir's fuse for the MoE block (models/olmoe.rs:432-500, safetensors.rs:450-600):
+ * the members are stacked in numeric expert order into [E, out, in] banks of the source dtype
+ * (BF16 / F16 / F32 kept as stored) and loaded into the handle's layers 0..n_layers. */
+MUMMU_API int mummu_moe_load_safetensors(mummu_moe *h, mummu_st *st, int first_layer, int n_layers);
 
 /* ---- plumbing for harnesses that do not link HIP themselves -----------------------------*/
 MUMMU_API void *mummu_device_alloc(size_t bytes);

@@ -22,6 +22,10 @@
 //   OlmoeConfig::from_gguf (MoE fields) models/olmoe.rs:116-179   mummu::GgufFile::moe_config
 //   RoutedExperts::open (bank locator) experts.rs:869-911         mummu::GgufFile::locate_moe_layer,
 //                                                                  mummu::SparseMoe::from_gguf
+//   OlmoeConfig::from_json_bytes  models/olmoe.rs:104-108          mummu::olmoe_config_from_json
+//   checkpoint_shards, SafetensorsHeader::open, olmoe_hf_fuse, load_from_dir
+//                              safetensors.rs:180-430; models/olmoe.rs:405-500
+//                                                      mummu::Checkpoint, mummu::SparseMoe::from_checkpoint
 //
 // Error behaviour: the reference panics on contract violations of SparseMoe (assert!) and
 // returns Err(String) from the qwen4exp functions.  Both surface here as mummu::MoeError (a
@@ -212,6 +216,70 @@ class GgufFile {
     std::shared_ptr<mummu_gguf> g_;
 };
 
+// SafetensorsError (safetensors.rs:62-118) and the config errors of OlmoeConfig::from_json_bytes.
+class SafetensorsError : public MoeError {
+  public:
+    using MoeError::MoeError;
+};
+
+inline SparseMoeConfig moe_config_of(const mummu_moe_config &k) {
+    SparseMoeConfig c;
+    c.hidden_size = k.hidden_size;
+    c.expert_intermediate_size = k.expert_intermediate_size;
+    c.num_experts = k.num_experts;
+    c.num_experts_per_tok = k.num_experts_per_tok;
+    c.norm_topk_prob = k.norm_topk_prob != 0;
+    c.router_flavour = k.router_flavour;
+    c.num_layers = k.num_layers;
+    c.max_tokens = k.max_tokens;
+    c.rms_norm_eps = k.rms_norm_eps;
+    return c;
+}
+
+// OlmoeConfig::from_json_bytes (models/olmoe.rs:104-108): the MoE block's fields, validated.
+inline SparseMoeConfig olmoe_config_from_json(const std::string &json) {
+    mummu_moe_config k{};
+    const int rc = mummu_olmoe_config_from_json(json.data(), json.size(), &k);
+    if (rc != MUMMU_OK) throw SafetensorsError(rc, mummu_st_last_error());
+    return moe_config_of(k);
+}
+
+// An HF safetensors checkpoint directory (safetensors.rs:180-430): shards discovered and every
+// header entry validated on open.
+class Checkpoint {
+  public:
+    static Checkpoint open(const std::string &dir) {
+        mummu_st *st = nullptr;
+        const int rc = mummu_st_open(dir.c_str(), &st);
+        if (rc != MUMMU_OK) throw SafetensorsError(rc, mummu_st_last_error());
+        return Checkpoint(st);
+    }
+    mummu_st *handle() const { return st_.get(); }
+    size_t shard_count() const { return (size_t)mummu_st_shard_count(st_.get()); }
+    size_t tensor_count() const { return (size_t)mummu_st_tensor_count(st_.get()); }
+    std::optional<mummu_st_tensor> tensor(const std::string &name) const {
+        const int i = mummu_st_find_tensor(st_.get(), name.c_str());
+        if (i < 0) return std::nullopt;
+        mummu_st_tensor t{};
+        check(mummu_st_tensor_info(st_.get(), i, &t));
+        return t;
+    }
+    SparseMoeConfig moe_config() const {
+        mummu_moe_config k{};
+        check(mummu_st_moe_config(st_.get(), &k));
+        return moe_config_of(k);
+    }
+    // The fuse's planning pass for one layer (olmoe_hf_fuse + the group rules), nothing read.
+    void check_moe_layer(int layer) const { check(mummu_st_check_moe_layer(st_.get(), layer)); }
+
+  private:
+    explicit Checkpoint(mummu_st *st) : st_(st, mummu_st_close) {}
+    static void check(int rc) {
+        if (rc != MUMMU_OK) throw SafetensorsError(rc, mummu_st_last_error());
+    }
+    std::shared_ptr<mummu_st> st_;
+};
+
 // The block, resident on the MI355X.  One object holds every MoE layer of a model.
 class SparseMoe {
   public:
@@ -255,6 +323,19 @@ class SparseMoe {
         SparseMoe m(c);
         const int rc = mummu_moe_load_gguf(m.handle(), f.handle(), first_layer, n_layers);
         if (rc != MUMMU_OK) throw GgufError(rc, mummu_gguf_last_error());
+        return m;
+    }
+
+    // The same from an HF checkpoint directory: per-expert projections fused into [E, out, in]
+    // banks of the stored dtype (load_from_dir, models/olmoe.rs:432-500).
+    static SparseMoe from_checkpoint(const Checkpoint &ck, int first_layer = 0, int n_layers = -1, int max_tokens = 512) {
+        SparseMoeConfig c = ck.moe_config();
+        if (n_layers < 0) n_layers = c.num_layers - first_layer;
+        c.num_layers = n_layers > 0 ? n_layers : 1;
+        c.max_tokens = max_tokens;
+        SparseMoe m(c);
+        const int rc = mummu_moe_load_safetensors(m.handle(), ck.handle(), first_layer, n_layers);
+        if (rc != MUMMU_OK) throw SafetensorsError(rc, mummu_st_last_error());
         return m;
     }
 

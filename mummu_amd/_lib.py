@@ -19,10 +19,10 @@ BLOCKS = {F32: (1, 4), F16: (1, 2), BF16: (1, 2), Q4_0: (32, 18), Q4_1: (32, 20)
 ROUTER_SPARSE_MOE, ROUTER_QWEN4EXP = 0, 1
 
 (OK, ERR_CONFIG, ERR_TYPE, ERR_BLOCKS, ERR_TOPK, ERR_SHAPE, ERR_NONFINITE, ERR_RANGE, ERR_NOT_LOADED, ERR_TOKENS,
- ERR_DEVICE, ERR_ARG, ERR_IO, ERR_GGUF) = range(14)
+ ERR_DEVICE, ERR_ARG, ERR_IO, ERR_GGUF, ERR_SAFETENSORS) = range(15)
 
 STATUS_NAMES = ["ok", "config", "type", "blocks", "topk", "shape", "nonfinite", "range", "not_loaded", "tokens",
-                "device", "arg", "io", "gguf"]
+                "device", "arg", "io", "gguf", "safetensors"]
 
 
 class Config(C.Structure):
@@ -39,6 +39,14 @@ class GgufTensor(C.Structure):
     _fields_ = [
         ("name", C.c_char_p), ("n_dims", C.c_int32), ("dims", C.c_int64 * 4), ("ggml_type", C.c_int32),
         ("shard", C.c_int32), ("file_offset", C.c_uint64), ("nbytes", C.c_uint64), ("path", C.c_char_p),
+    ]
+
+
+class StTensor(C.Structure):
+    """mummu_st_tensor."""
+    _fields_ = [
+        ("name", C.c_char_p), ("dtype", C.c_char_p), ("n_dims", C.c_int32), ("dims", C.c_int64 * 8), ("shard", C.c_int32),
+        ("file_offset", C.c_uint64), ("nbytes", C.c_uint64), ("path", C.c_char_p),
     ]
 
 
@@ -101,6 +109,17 @@ SIGNATURES = {
     "mummu_gguf_moe_config": (_I, [_P, C.POINTER(Config)]),
     "mummu_gguf_locate_moe_layer": (_I, [_P, _I, C.POINTER(GgufMoeLayer)]),
     "mummu_moe_load_gguf": (_I, [_P, _P, _I, _I]),
+    "mummu_st_last_error": (C.c_char_p, []),
+    "mummu_st_open": (_I, [C.c_char_p, C.POINTER(_P)]),
+    "mummu_st_close": (None, [_P]),
+    "mummu_st_shard_count": (_I, [_P]),
+    "mummu_st_tensor_count": (_I, [_P]),
+    "mummu_st_find_tensor": (_I, [_P, C.c_char_p]),
+    "mummu_st_tensor_info": (_I, [_P, _I, C.POINTER(StTensor)]),
+    "mummu_olmoe_config_from_json": (_I, [C.c_char_p, _SZ, C.POINTER(Config)]),
+    "mummu_st_moe_config": (_I, [_P, C.POINTER(Config)]),
+    "mummu_st_check_moe_layer": (_I, [_P, _I]),
+    "mummu_moe_load_safetensors": (_I, [_P, _P, _I, _I]),
     "mummu_moe_kernel_timing": (_I, [_P, _I]),
     "mummu_moe_kernel_times": (_I, [_P, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(C.c_int64), _I]),
 }

@@ -268,6 +268,21 @@ int main(int argc, char **argv) {
                                  d = sin_fill(3.3f, E * H * I);
         gguf_host_checks(r, g, u, d);
     }
+    // OlmoeConfig::from_json_bytes: fields, default, refusals (models/olmoe.rs:52-226)
+    {
+        const std::string ok = R"({"vocab_size": 50304, "hidden_size": 2048, "intermediate_size": 1024, "num_hidden_layers": 16,
+            "num_attention_heads": 16, "num_key_value_heads": 16, "num_experts": 64, "num_experts_per_tok": 8,
+            "rms_norm_eps": 1e-05, "rope_theta": 10000.0})";
+        const mummu::SparseMoeConfig c = mummu::olmoe_config_from_json(ok);
+        EXPECT(c.hidden_size == 2048 && c.expert_intermediate_size == 1024 && c.num_experts == 64 && c.num_experts_per_tok == 8 &&
+                   c.num_layers == 16 && !c.norm_topk_prob,
+               "config.json fields, norm_topk_prob defaults to false");
+        std::string one = ok;
+        one.replace(one.find("\"num_experts\": 64"), 17, "\"num_experts\": 1 ");
+        EXPECT(throws([&] { mummu::olmoe_config_from_json(one); }, MUMMU_ERR_CONFIG, "num_experts (1) must be >= 2"), "one expert is refused");
+        EXPECT(throws([&] { mummu::olmoe_config_from_json("{\"hidden_size\": 4"); }, MUMMU_ERR_CONFIG, "config.json"), "broken JSON is refused");
+        EXPECT(throws([&] { mummu::Checkpoint::open("/nonexistent-dir"); }, MUMMU_ERR_IO, "neither"), "a directory without a checkpoint");
+    }
     if (no_gpu) {
         std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror (no gpu): ok\n", failures);
         return failures ? 1 : 0;
