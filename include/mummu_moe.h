@@ -103,6 +103,18 @@ MUMMU_API int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, 
                                    int gate_type, const void *up, int up_type, const void *down, int down_type,
                                    const float *rms_gamma);
 
+/* The Qwen-style block's shared expert and its sigmoid gate (models/qwen4exp/model.rs:786-804;
+ * tensors `ffn_{gate,up,down}_shexp`, `ffn_gate_inp_shexp`, :228-231): once loaded, forward and
+ * stack_forward of that layer return
+ *     routed + shared_ffn(x) * sigmoid(<gate_vec, x>)
+ * (product and sums rounded separately, in that grouping).  gate/up [inter, hidden] and down
+ * [hidden, inter] in any bank type, `inter` free; gate_vec [hidden] F32 / F16 / BF16, or NULL for
+ * an ungated shared expert.  The routed-only entry points (route, apply_routing, routed) are not
+ * affected.  Call after mummu_moe_load_layer of the same layer. */
+MUMMU_API int mummu_moe_load_shared_expert(mummu_moe *h, int layer, int inter, const void *gate, int gate_type, const void *up,
+                                           int up_type, const void *down, int down_type, const void *gate_vec,
+                                           int gate_vec_type);
+
 /* Bytes resident on the device for weights (ExpertExec::resident_bytes, nn/moe.rs:352). */
 MUMMU_API uint64_t mummu_moe_resident_bytes(const mummu_moe *h);
 
@@ -229,7 +241,10 @@ MUMMU_API int mummu_gguf_locate_moe_layer(const mummu_gguf *g, int layer, mummu_
 /* RoutedExperts::open (experts.rs:869-911) + Olmoe's MoE-block load (models/olmoe.rs:338-345):
  * locates layers [first_layer, first_layer + n_layers) as above and loads them into the
  * handle's layers 0..n_layers through mummu_moe_load_layer, payload bytes unchanged (mapped
- * read-only from their shard, offsets relative to that shard's own payload base). */
+ * read-only from their shard, offsets relative to that shard's own payload base).  A layer that
+ * also holds `blk.L.ffn_{gate,up,down}_shexp.weight` (2 dims) gets its shared expert loaded too,
+ * gated by `blk.L.ffn_gate_inp_shexp.weight` [H] when that is present
+ * (models/qwen4exp/model.rs:228-231). */
 MUMMU_API int mummu_moe_load_gguf(mummu_moe *h, mummu_gguf *g, int first_layer, int n_layers);
 
 /* ---- HF safetensors checkpoint directories (host side) -----------------------------------

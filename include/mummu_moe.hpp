@@ -339,6 +339,14 @@ class SparseMoe {
         return m;
     }
 
+    // The shared expert of a Qwen-style block and its sigmoid gate vector (may be null)
+    // (models/qwen4exp/model.rs:786-804): forward then returns routed + shared(x) * sigmoid(<gate_vec, x>).
+    void load_shared_expert(int layer, int inter, TensorBytes gate, TensorBytes up, TensorBytes down,
+                            TensorBytes gate_vec = TensorBytes()) {
+        check(mummu_moe_load_shared_expert(h_.get(), layer, inter, gate.data, gate.ggml_type, up.data, up.ggml_type, down.data,
+                                           down.ggml_type, gate_vec.data, gate_vec.ggml_type));
+    }
+
     uint64_t resident_bytes() const { return mummu_moe_resident_bytes(h_.get()); }
 
     // SparseMoe::forward (nn/moe.rs:116): x [tokens, hidden] -> [tokens, hidden].

@@ -63,6 +63,7 @@ SIGNATURES = {
     "mummu_moe_create": (_I, [C.POINTER(Config), C.POINTER(_P)]),
     "mummu_moe_destroy": (None, [_P]),
     "mummu_moe_load_layer": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P]),
+    "mummu_moe_load_shared_expert": (_I, [_P, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I]),
     "mummu_moe_resident_bytes": (C.c_uint64, [_P]),
     "mummu_moe_forward": (_I, [_P, _I, _P, _I64, _I, _I, _P]),
     "mummu_moe_route": (_I, [_P, _I, _P, _I64, _I, _I, _P, _P, _P]),

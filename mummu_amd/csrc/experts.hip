@@ -653,4 +653,29 @@ hipError_t launch_combine(const float *y, const int32_t *ids, const float *weigh
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------
+// shared expert: out = [residual +] (out + y * sigmoid(logit)), each operation rounded on its own
+// (models/qwen4exp/model.rs:786-804).  logit null: the shared expert is not gated.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void shared_add_kernel(float *__restrict__ out, const float *__restrict__ y,
+                                                         const float *__restrict__ logit, const float *__restrict__ residual,
+                                                         int hidden) {
+    const int t = blockIdx.x;
+    float g = 1.0f;
+    if (logit) g = __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-logit[t])));
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < hidden; c += gridDim.y * blockDim.x) {
+        const size_t o = (size_t)t * (size_t)hidden + c;
+        const float shared = logit ? __fmul_rn(y[o], g) : y[o];
+        const float v = __fadd_rn(out[o], shared);
+        out[o] = residual ? __fadd_rn(residual[o], v) : v;
+    }
+}
+
+hipError_t launch_shared_add(float *out, const float *y, const float *logit, const float *residual, int n, int hidden, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    int ysplit = n >= 64 ? 1 : (hidden + 255) / 256;
+    launch_kernel(shared_add_kernel, dim3(n, ysplit), dim3(256), 0, s, out, y, logit, residual, hidden);
+    return hipGetLastError();
+}
+
 }  // namespace mummu

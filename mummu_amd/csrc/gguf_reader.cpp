@@ -574,6 +574,31 @@ int mummu_moe_load_gguf(mummu_moe *h, mummu_gguf *g, int first_layer, int n_laye
         }
         rc = mummu_moe_load_layer(h, l, data[0], type[0], data[1], type[1], data[2], type[2], data[3], type[3], (const float *)data[4]);
         if (rc) return fail(rc, "blk." + std::to_string(first_layer + l) + ": " + mummu_moe_last_error(h));
+        // the shared expert of a Qwen-style block, when the file has one (models/qwen4exp/model.rs:228-231)
+        const std::string blk = "blk." + std::to_string(first_layer + l) + ".";
+        const int sg = g->find(blk + "ffn_gate_shexp.weight"), su = g->find(blk + "ffn_up_shexp.weight"),
+                  sd = g->find(blk + "ffn_down_shexp.weight"), sv = g->find(blk + "ffn_gate_inp_shexp.weight");
+        if (sg >= 0 || su >= 0 || sd >= 0) {
+            if (sg < 0 || su < 0 || sd < 0) return fail(MUMMU_ERR_GGUF, blk + "ffn_*_shexp.weight: the shared expert needs its gate, up and down tensors");
+            const Tensor &tg = g->header.tensors[(size_t)sg], &tu = g->header.tensors[(size_t)su], &td = g->header.tensors[(size_t)sd];
+            mummu_moe_config want;
+            if ((rc = mummu_gguf_moe_config(g, &want))) return rc;
+            const uint64_t H = (uint64_t)want.hidden_size;
+            if (tg.dims.size() != 2 || tu.dims.size() != 2 || td.dims.size() != 2 || tg.dims[0] != H || tu.dims != tg.dims ||
+                td.dims[0] != tg.dims[1] || td.dims[1] != H || tg.dims[1] > (1u << 30))
+                return fail(MUMMU_ERR_SHAPE, blk + "ffn_*_shexp.weight: want gate/up [hidden, width] and down [width, hidden]");
+            const void *pg, *pu, *pd, *pv = nullptr;
+            int vt = MUMMU_F32;
+            if ((rc = g->payload(sg, &pg)) || (rc = g->payload(su, &pu)) || (rc = g->payload(sd, &pd))) return rc;
+            if (sv >= 0) {
+                const Tensor &tv = g->header.tensors[(size_t)sv];
+                if (tv.dims.size() != 1 || tv.dims[0] != H) return fail(MUMMU_ERR_SHAPE, blk + "ffn_gate_inp_shexp.weight: want [hidden]");
+                vt = (int)tv.type;
+                if ((rc = g->payload(sv, &pv))) return rc;
+            }
+            rc = mummu_moe_load_shared_expert(h, l, (int)tg.dims[1], pg, (int)tg.type, pu, (int)tu.type, pd, (int)td.type, pv, vt);
+            if (rc) return fail(rc, blk + "ffn_*_shexp: " + mummu_moe_last_error(h));
+        }
     }
     g_gguf_error.clear();
     return MUMMU_OK;

@@ -80,6 +80,11 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
                                const float *residual, float *out, hipStream_t s);
 
 
+// out[t, :] = [residual[t, :] +] (out[t, :] + y[t, :] * sigmoid(logit[t])), every operation rounded on
+// its own; logit null: no gate.
+hipError_t launch_shared_add(float *out, const float *y, const float *logit, const float *residual, int n, int hidden,
+                             hipStream_t s);
+
 // dispatch.hip ------------------------------------------------------------------------
 // Stable counting sort of the assignments by expert (ranks, histograms and scans in LDS, three
 // small launches): offsets[E+1], sorted[A] (position -> assignment), inv[A] (assignment ->

@@ -23,9 +23,9 @@ namespace {
 thread_local std::string g_error;  // failures of calls that have no handle
 
 enum KernelSlot { K_ROUTER, K_ROUTER_LOGITS, K_ROUTE_TOPK, K_QUANTIZE, K_GATE_UP, K_DOWN_COMBINE, K_DOWN, K_COMBINE, K_RMSNORM,
-                  K_DISPATCH, K_GEMM_GATE_UP, K_GEMM_DOWN, K_SLOTS };
+                  K_DISPATCH, K_GEMM_GATE_UP, K_GEMM_DOWN, K_SHARED, K_SLOTS };
 const char *const kSlotNames[K_SLOTS] = {"router", "router_logits", "route_topk", "quantize", "gate_up", "down_combine",
-                                         "down", "combine", "rmsnorm", "dispatch", "gemm_gate_up", "gemm_down"};
+                                         "down", "combine", "rmsnorm", "dispatch", "gemm_gate_up", "gemm_down", "shared_expert"};
 
 struct Layer {
     void *router = nullptr;
@@ -36,6 +36,13 @@ struct Layer {
     unsigned long long *hits = nullptr;
     size_t bytes = 0;
     bool loaded = false;
+    // optional shared expert (always active) and its per-token sigmoid gate vector
+    uint8_t *sh_gate = nullptr, *sh_up = nullptr, *sh_down = nullptr;
+    int sh_gate_type = 0, sh_up_type = 0, sh_down_type = 0, sh_inter = 0;
+    void *sh_gatevec = nullptr;  // [hidden], router-type floats; null: the shared expert is added ungated
+    int sh_gatevec_type = 0;
+    size_t sh_bytes = 0;
+    bool sh_loaded = false;
 };
 
 struct TimedLaunch {
@@ -68,6 +75,11 @@ struct mummu_moe {
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
     int gemm_min_tokens = 32;    // batches at least this large take the grouped GEMM
+    // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
+    int sh_inter_max = 0;
+    int64_t sh_ws_tokens = 0;
+    float *sh_act = nullptr, *sh_y = nullptr, *sh_logit = nullptr;
+    QAct sh_actq;
 
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing = false;
@@ -108,6 +120,34 @@ void free_ws(mummu_moe *h) {
     h->act16 = nullptr;
     h->ws_tokens = h->ws_assign = 0;
     h->ws_experts = 0;
+    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum};
+    for (void *p : sh)
+        if (p) (void)hipFree(p);
+    h->sh_act = h->sh_y = h->sh_logit = nullptr;
+    h->sh_actq = QAct();
+    h->sh_ws_tokens = 0;
+}
+
+// The shared expert's own buffers, sized for the main workspace's token count.
+int ensure_shared_ws(mummu_moe *h) {
+    if (h->sh_inter_max == 0 || h->sh_ws_tokens >= h->ws_tokens) return MUMMU_OK;
+    HIPCHK(h, hipDeviceSynchronize());
+    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum};
+    for (void *p : sh)
+        if (p) (void)hipFree(p);
+    h->sh_act = h->sh_y = h->sh_logit = nullptr;
+    h->sh_actq = QAct();
+    const size_t nt = (size_t)h->ws_tokens, H = (size_t)h->cfg.hidden_size, I = (size_t)h->sh_inter_max;
+    const size_t ae = nt * ((I + 15) / 16 * 16);
+    HIPCHK(h, hipMalloc(&h->sh_act, sizeof(float) * nt * I));
+    HIPCHK(h, hipMalloc(&h->sh_y, sizeof(float) * nt * H));
+    HIPCHK(h, hipMalloc(&h->sh_logit, sizeof(float) * nt));
+    HIPCHK(h, hipMalloc(&h->sh_actq.hi, ae));
+    HIPCHK(h, hipMalloc(&h->sh_actq.lo, ae));
+    HIPCHK(h, hipMalloc(&h->sh_actq.scale, sizeof(float) * (ae / 16)));
+    HIPCHK(h, hipMalloc(&h->sh_actq.sum, sizeof(int32_t) * (ae / 16)));
+    h->sh_ws_tokens = h->ws_tokens;
+    return MUMMU_OK;
 }
 
 // Grow the workspace to hold n tokens and n_assign (token, expert) pairs.  Host entry points
@@ -153,7 +193,7 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     h->ws_tokens = nt;
     h->ws_assign = na;
     h->ws_experts = n_experts;
-    return MUMMU_OK;
+    return ensure_shared_ws(h);
 }
 
 // Device error flags back to idle.
@@ -282,8 +322,8 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
     return MUMMU_OK;
 }
 
-int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
-                 hipStream_t s) {
+int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
+                hipStream_t s) {
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
@@ -318,6 +358,38 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
                launch_route_topk(h->logits, (int)n, E, k, h->cfg.router_flavour, norm, h->ids, h->weights, L.hits, h->flags, s));
     }
     return run_experts(h, L, x, want_xq, n, k, residual, out, s);
+}
+
+// The block: the routed experts, plus (when the layer has one) the shared expert every token
+// takes, scaled by its sigmoid gate (models/qwen4exp/model.rs:786-804):
+//     out = [residual +] (routed + shared_ffn(x) * sigmoid(<gate_vec, x>))
+// with the product and the two sums rounded separately, in that grouping.
+int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
+                 hipStream_t s) {
+    const Layer &L = h->layers[layer];
+    if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s);
+    int rc = routed_impl(h, layer, x, n, k, norm, nullptr, out, s);
+    if (rc) return rc;
+    if (n > h->sh_ws_tokens) return fail(h, MUMMU_ERR_TOKENS, "shared-expert workspace is smaller than the call");
+    const int H = h->cfg.hidden_size;
+    ExpertBanks b;
+    b.gate = L.sh_gate;
+    b.up = L.sh_up;
+    b.down = L.sh_down;
+    b.gate_type = L.sh_gate_type;
+    b.up_type = L.sh_up_type;
+    b.down_type = L.sh_down_type;
+    b.hidden = H;
+    b.inter = L.sh_inter;
+    b.n_experts = 1;
+    // the routed path may have left the 16-bit activations in the batched layout (or not made them)
+    if (is_quant_type(b.gate_type)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x, (int)n, H, h->xq, s));
+    LAUNCH(h, K_SHARED, s, launch_gate_up(b, x, h->xq, nullptr, (int)n, 1, 0, h->sh_act, h->sh_actq, h->flags, s));
+    LAUNCH(h, K_SHARED, s, launch_down(b, h->sh_act, h->sh_actq, nullptr, (int)n, 1, 0, h->sh_y, s));
+    if (L.sh_gatevec)
+        LAUNCH(h, K_SHARED, s, launch_router_logits(x, L.sh_gatevec, L.sh_gatevec_type, h->sh_logit, (int)n, H, 1, QAct(), s));
+    LAUNCH(h, K_SHARED, s, launch_shared_add(out, h->sh_y, L.sh_gatevec ? h->sh_logit : nullptr, residual, (int)n, H, s));
+    return MUMMU_OK;
 }
 
 int check_device_call(mummu_moe *h, int64_t n, int k, const void *a, const void *b) {
@@ -407,7 +479,7 @@ void mummu_moe_destroy(mummu_moe *h) {
     if (!h) return;
     (void)hipDeviceSynchronize();
     for (Layer &L : h->layers) {
-        void *ptrs[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits};
+        void *ptrs[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits, L.sh_gate, L.sh_up, L.sh_down, L.sh_gatevec};
         for (void *p : ptrs)
             if (p) (void)hipFree(p);
     }
@@ -448,7 +520,7 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
 
     Layer &L = h->layers[layer];
     HIPCHK(h, hipDeviceSynchronize());
-    void *old[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits};
+    void *old[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits, L.sh_gate, L.sh_up, L.sh_down, L.sh_gatevec};
     for (void *p : old)
         if (p) (void)hipFree(p);
     L = Layer();
@@ -479,10 +551,66 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
     return MUMMU_OK;
 }
 
+int mummu_moe_load_shared_expert(mummu_moe *h, int layer, int inter, const void *gate, int gate_type, const void *up, int up_type,
+                                 const void *down, int down_type, const void *gate_vec, int gate_vec_type) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);  // the routed part of the layer comes first
+    if (rc) return rc;
+    if (!gate || !up || !down) return fail(h, MUMMU_ERR_ARG, "null weight pointer");
+    for (int t : {gate_type, up_type, down_type})
+        if (!bank_type_ok(t)) return fail(h, MUMMU_ERR_TYPE, "no expert kernel for ggml type " + std::to_string(t));
+    if (gate_type != up_type) return fail(h, MUMMU_ERR_TYPE, "gate and up banks must share one type");
+    if (gate_vec && !router_type_ok(gate_vec_type))
+        return fail(h, MUMMU_ERR_TYPE, "the shared expert's gate vector must be F32, F16 or BF16 (got ggml type " + std::to_string(gate_vec_type) + ")");
+    const int H = h->cfg.hidden_size;
+    if (inter < 1) return fail(h, MUMMU_ERR_CONFIG, "shared expert width must be >= 1");
+    if (H % block_elems(gate_type))
+        return fail(h, MUMMU_ERR_BLOCKS, "row width " + std::to_string(H) + " is not whole blocks of " + std::to_string(block_elems(gate_type)));
+    if (inter % block_elems(down_type))
+        return fail(h, MUMMU_ERR_BLOCKS, "row width " + std::to_string(inter) + " is not whole blocks of " + std::to_string(block_elems(down_type)));
+    if ((is_quant_type(gate_type) && H / 32 > 256) || (is_quant_type(down_type) && inter / 32 > 256))
+        return fail(h, MUMMU_ERR_CONFIG, "quantized rows wider than 8192 are not supported");
+    if (is_quant_type(down_type) && inter % 16) return fail(h, MUMMU_ERR_BLOCKS, "shared expert width must be a multiple of 16 for a quantized down matrix");
+    Layer &L = h->layers[layer];
+    HIPCHK(h, hipDeviceSynchronize());
+    void *old[] = {L.sh_gate, L.sh_up, L.sh_down, L.sh_gatevec};
+    for (void *p : old)
+        if (p) (void)hipFree(p);
+    L.sh_gate = L.sh_up = L.sh_down = nullptr;
+    L.sh_gatevec = nullptr;
+    L.sh_loaded = false;
+    L.sh_bytes = 0;
+    const size_t gb = (size_t)inter * row_bytes_of(gate_type, H), db = (size_t)H * row_bytes_of(down_type, inter);
+    const size_t vb = gate_vec ? (size_t)H * (size_t)block_bytes(gate_vec_type) : 0;
+    HIPCHK(h, hipMalloc(&L.sh_gate, gb));
+    HIPCHK(h, hipMalloc(&L.sh_up, gb));
+    HIPCHK(h, hipMalloc(&L.sh_down, db));
+    HIPCHK(h, hipMemcpy(L.sh_gate, gate, gb, hipMemcpyHostToDevice));
+    HIPCHK(h, hipMemcpy(L.sh_up, up, gb, hipMemcpyHostToDevice));
+    HIPCHK(h, hipMemcpy(L.sh_down, down, db, hipMemcpyHostToDevice));
+    if (gate_vec) {
+        HIPCHK(h, hipMalloc(&L.sh_gatevec, vb));
+        HIPCHK(h, hipMemcpy(L.sh_gatevec, gate_vec, vb, hipMemcpyHostToDevice));
+    }
+    L.sh_gate_type = gate_type;
+    L.sh_up_type = up_type;
+    L.sh_down_type = down_type;
+    L.sh_gatevec_type = gate_vec_type;
+    L.sh_inter = inter;
+    L.sh_bytes = 2 * gb + db + vb;
+    L.sh_loaded = true;
+    if (inter > h->sh_inter_max) {
+        h->sh_inter_max = inter;
+        h->sh_ws_tokens = 0;  // regrow for the wider expert
+    }
+    return ensure_shared_ws(h);
+}
+
 uint64_t mummu_moe_resident_bytes(const mummu_moe *h) {
     if (!h) return 0;
     uint64_t total = 0;
-    for (const Layer &L : h->layers) total += L.bytes;
+    for (const Layer &L : h->layers) total += L.bytes + L.sh_bytes;
     return total;
 }
 

@@ -142,6 +142,25 @@ class SparseMoe:
         self._check(self._lib.mummu_moe_load_layer(self._h, layer, _ptr(router), router_type, _ptr(gate), gate_type,
                                                    _ptr(up), up_type, _ptr(down), down_type, _ptr(g)))
 
+    def load_shared_expert(self, layer: int, inter: int, gate, gate_type: int, up, up_type: int, down, down_type: int,
+                           gate_vec=None, gate_vec_type: int = F32):
+        """The always-on shared expert of a Qwen-style block and its sigmoid gate vector
+        (models/qwen4exp/model.rs:786-804): gate/up [inter, hidden], down [hidden, inter] as GGUF
+        payload bytes, gate_vec [hidden] or None."""
+        c = self.config
+        gate, up, down = _bytes(gate), _bytes(up), _bytes(down)
+        for name, arr, t, i, o in (("gate", gate, gate_type, c.hidden_size, inter), ("up", up, up_type, c.hidden_size, inter),
+                                   ("down", down, down_type, inter, c.hidden_size)):
+            bs = _lib.BLOCKS.get(t)
+            if bs is not None and i % bs[0] == 0 and arr.size != o * (i // bs[0]) * bs[1]:
+                raise MoeError(_lib.ERR_SHAPE, f"shared expert {name} is {o * (i // bs[0]) * bs[1]} bytes, got {arr.size}")
+        gv = None if gate_vec is None else _bytes(gate_vec)
+        vw = {F32: 4, F16: 2, BF16: 2}.get(gate_vec_type)
+        if gv is not None and vw is not None and gv.size != c.hidden_size * vw:
+            raise MoeError(_lib.ERR_SHAPE, f"shared expert gate vector is {c.hidden_size * vw} bytes, got {gv.size}")
+        self._check(self._lib.mummu_moe_load_shared_expert(self._h, layer, inter, _ptr(gate), gate_type, _ptr(up), up_type,
+                                                           _ptr(down), down_type, _ptr(gv), gate_vec_type))
+
     def resident_bytes(self) -> int:
         return int(self._lib.mummu_moe_resident_bytes(self._h))
 

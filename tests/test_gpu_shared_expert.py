@@ -1,0 +1,160 @@
+"""The Qwen-style block (models/qwen4exp/model.rs:786-804): routed experts plus the shared expert
+every token takes, scaled by sigmoid(<gate_vec, x>).  Checked against the oracle's pieces composed
+the way the reference composes them - routed (+) shared_ffn(x) * sigmoid(logit) - within 2e-3 for
+quantized banks and 1e-5 for f32, for one token, a few, and enough for the batched path; the
+routed-only entry points stay routed-only; a GGUF file with ffn_*_shexp tensors loads it by itself."""
+import numpy as np
+import pytest
+
+from mummu_amd import moe as M
+from mummu_amd import synth
+from mummu_amd.gguf import GgufFile
+from oracle import binding as orc
+from tests import gguf_writer as W
+
+pytestmark = pytest.mark.gpu
+
+
+def normal(shape, seed, std=1.0):
+    g = np.random.Generator(np.random.PCG64(seed))
+    return (g.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+
+def bank(t, ne, seed, std=0.05):
+    if t == M.F32:
+        return normal((ne[2], ne[1], ne[0]), seed, std)
+    return synth.random_bank_fast(t, ne, seed)
+
+
+def reference(banks, shared, router, rt, gate_vec, x, k, norm, flavour):
+    """(routed, full): routed from the oracle's block, full = routed + shared * sigmoid (f64 for the tolerance)."""
+    _, ids, w, _ = orc.moe_forward(banks, router, rt, x, k, norm, flavour)
+    routed, mag = orc.moe_ref_f64(banks, ids, w, x)
+    n = x.shape[0]
+    sh, smag = orc.moe_ref_f64(shared, np.zeros((n, 1), np.uint32), np.ones((n, 1), np.float32), x)
+    if gate_vec is None:
+        g = np.ones((n, 1))
+    else:
+        z = orc.router_logits(x, gate_vec, orc.F32, 1).astype(np.float64).reshape(n, 1)
+        g = 1.0 / (1.0 + np.exp(-z))
+    return ids, w, routed, routed + sh * g, np.maximum(mag, smag * g)
+
+
+CASES = [
+    # routed gate/up, routed down, shared gate/up, shared down, H, I, I_shared, E, k, flavour
+    (M.Q4_K, M.Q5_1, M.Q4_K, M.Q8_0, 512, 128, 128, 16, 4, M.ROUTER_QWEN4EXP),
+    (M.Q4_K, M.Q4_K, M.Q8_0, M.Q8_0, 512, 256, 512, 8, 2, M.ROUTER_SPARSE_MOE),  # shared expert wider than the routed ones
+    (M.F32, M.F32, M.F32, M.F32, 64, 48, 80, 4, 2, M.ROUTER_SPARSE_MOE),
+    (M.Q8_0, M.Q8_0, M.F32, M.F32, 256, 64, 96, 8, 2, M.ROUTER_QWEN4EXP),       # quantized routed, float shared
+]
+
+
+@pytest.mark.parametrize("gt,dt,sgt,sdt,H,I,IS,E,k,flavour", CASES)
+@pytest.mark.parametrize("gated", [True, False])
+def test_shared_expert_and_sigmoid_gate_match_the_composition(gt, dt, sgt, sdt, H, I, IS, E, k, flavour, gated):
+    gate, up, down = bank(gt, [H, I, E], 1), bank(gt, [H, I, E], 2), bank(dt, [I, H, E], 3)
+    sgate, sup, sdown = bank(sgt, [H, IS, 1], 4), bank(sgt, [H, IS, 1], 5), bank(sdt, [IS, H, 1], 6)
+    router = normal((E, H), 7, 0.05)
+    gate_vec = normal((H,), 8, 0.2) if gated else None
+    n = 70
+    x = normal((n, H), 9)
+    norm = flavour == M.ROUTER_QWEN4EXP
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=n, router_flavour=flavour) as m:
+        m.load_layer(0, router, M.F32, gate, gt, up, gt, down, dt)
+        before = m.resident_bytes()
+        routed_only = m.forward(x, k, norm)
+        routed5 = m.forward(x[:5], k, norm)
+        m.load_shared_expert(0, IS, sgate, sgt, sup, sgt, sdown, sdt, gate_vec)
+        assert m.resident_bytes() > before
+        outs = {c: m.forward(x[:c], k, norm) for c in (1, 5, n)}
+        r = m.route(x[:5], k, norm)
+        local = m.run_local(x[:5], r)   # routed experts only, as in the reference
+    banks = orc.LayerBanks(H, I, E, gate, up, down, gt, gt, dt)
+    shared = orc.LayerBanks(H, IS, 1, sgate, sup, sdown, sgt, sgt, sdt)
+    ids, w, routed, full, mag = reference(banks, shared, router, orc.F32, gate_vec, x, k, norm, flavour)
+    tol = 1e-5 if gt == M.F32 else 2e-3
+    for c, got in outs.items():
+        assert orc.rel_err(got, full[:c], mag[:c]).max() <= tol, c
+    assert np.array_equal(outs[1].view(np.uint32), outs[n][:1].view(np.uint32)) or n >= 32  # same kernels below the batched path
+    assert np.array_equal(outs[1].view(np.uint32), outs[5][:1].view(np.uint32))
+    assert np.array_equal(local.view(np.uint32), routed5.view(np.uint32))
+    assert orc.rel_err(local, routed[:5], mag[:5]).max() <= tol
+    # the shared expert really contributes
+    assert np.abs(outs[n] - routed_only).max() > 1e-3
+
+
+def test_stack_forward_adds_the_residual_last_and_graph_replay_agrees():
+    H, I, IS, E, k, L, n = 256, 64, 64, 8, 2, 1, 4
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=8, router_flavour=M.ROUTER_QWEN4EXP) as m:
+        layers = []
+        for l in range(L):
+            w = dict(router=normal((E, H), 10 + l, 0.05), gate=bank(M.Q8_0, [H, I, E], 20 + l), up=bank(M.Q8_0, [H, I, E], 30 + l),
+                     down=bank(M.Q8_0, [I, H, E], 40 + l), sg=bank(M.Q8_0, [H, IS, 1], 50 + l), su=bank(M.Q8_0, [H, IS, 1], 60 + l),
+                     sd=bank(M.Q8_0, [IS, H, 1], 70 + l), gv=normal((H,), 80 + l, 0.2), gamma=np.ones(H, np.float32))
+            m.load_layer(l, w["router"], M.F32, w["gate"], M.Q8_0, w["up"], M.Q8_0, w["down"], M.Q8_0, w["gamma"])
+            m.load_shared_expert(l, IS, w["sg"], M.Q8_0, w["su"], M.Q8_0, w["sd"], M.Q8_0, w["gv"])
+            layers.append(w)
+        x = normal((n, H), 99, 0.5)
+        got = m.stack_forward(x, k, True)
+        # layer by layer on the host: x <- x + block(rmsnorm(x))
+        cur = x.copy()
+        for l, w in enumerate(layers):
+            hn = orc.rmsnorm(cur, w["gamma"], 1e-5)
+            cur = (cur + m.forward(hn, k, True, layer=l)).astype(np.float32)
+        # one layer: the device's RmsNorm may differ from the oracle's in the last place, which the
+        # experts pass on; no routing decision hangs on it here
+        assert np.abs(got - cur).max() <= 1e-5 * np.abs(cur).max()
+        # the device entry point inside a captured graph, replayed with eager work in between
+        xd, od = M.DeviceBuffer.from_array(x), M.DeviceBuffer(n * H * 4)
+        m.forward_device(0, xd, n, k, True, od)
+        M.synchronize()
+        eager = od.download(np.float32, (n, H))
+        m.graph_begin()
+        m.forward_device(0, xd, n, k, True, od)
+        graph = m.graph_end()
+        for _ in range(3):
+            m.forward(x[:2], k, True, layer=0)
+            graph.launch()
+            M.synchronize()
+            assert np.array_equal(od.download(np.float32, (n, H)).view(np.uint32), eager.view(np.uint32))
+        graph.close()
+
+
+def test_a_gguf_file_with_shexp_tensors_loads_the_shared_expert(tmp_path):
+    case = dict(hidden=256, inter=64, experts=8, top_k=2, router_type=0, gate_type=8, up_type=8, down_type=8, norm=True)
+    H, I, E, IS = 256, 64, 8, 96
+    lw = [dict(router=normal((E, H), 1, 0.05), gate=bank(M.Q8_0, [H, I, E], 2), up=bank(M.Q8_0, [H, I, E], 3), down=bank(M.Q8_0, [I, H, E], 4))]
+    sg, su, sd, gv = bank(M.Q8_0, [H, IS, 1], 5), bank(M.Q8_0, [H, IS, 1], 6), bank(M.Q4_0, [IS, H, 1], 7), normal((H,), 8, 0.2)
+    w = W.moe_gguf(case, lw, arch="qwen2moe")
+    w.add("blk.0.ffn_gate_shexp.weight", [H, IS], 8, sg).add("blk.0.ffn_up_shexp.weight", [H, IS], 8, su)
+    w.add("blk.0.ffn_down_shexp.weight", [IS, H], 2, sd).add("blk.0.ffn_gate_inp_shexp.weight", [H], 0, gv)
+    x = normal((6, H), 11)
+    with GgufFile.open(w.write(tmp_path / "q.gguf")) as f, f.load_moe(max_tokens=8) as m, \
+            M.SparseMoe(M.SparseMoeConfig(H, I, E, 2), max_tokens=8) as ref:
+        ref.load_layer(0, lw[0]["router"], M.F32, lw[0]["gate"], M.Q8_0, lw[0]["up"], M.Q8_0, lw[0]["down"], M.Q8_0)
+        ref.load_shared_expert(0, IS, sg, M.Q8_0, su, M.Q8_0, sd, M.Q4_0, gv)
+        assert m.resident_bytes() == ref.resident_bytes()
+        assert np.array_equal(m.forward(x, 2, True).view(np.uint32), ref.forward(x, 2, True).view(np.uint32))
+    # a file with only part of the shared expert is refused
+    w2 = W.moe_gguf(case, lw, arch="qwen2moe").add("blk.0.ffn_gate_shexp.weight", [H, IS], 8, sg)
+    with GgufFile.open(w2.write(tmp_path / "half.gguf")) as f:
+        with pytest.raises(M.MoeError, match="needs its gate, up and down"):
+            f.load_moe(max_tokens=8)
+
+
+def test_shared_expert_arguments_are_checked():
+    H, I, E = 256, 64, 4
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, 2)) as m:
+        z = np.zeros
+        with pytest.raises(M.MoeError, match="no weights"):
+            m.load_shared_expert(0, 64, z(64 * H, np.float32), M.F32, z(64 * H, np.float32), M.F32, z(64 * H, np.float32), M.F32)
+        m.load_layer(0, z((E, H), np.float32), M.F32, z(E * I * H, np.float32), M.F32, z(E * I * H, np.float32), M.F32,
+                     z(E * I * H, np.float32), M.F32)
+        with pytest.raises(M.MoeError, match="bytes"):
+            m.load_shared_expert(0, 64, z(10, np.uint8), M.Q8_0, z(10, np.uint8), M.Q8_0, z(10, np.uint8), M.Q8_0)
+        with pytest.raises(M.MoeError, match="whole blocks"):
+            m.load_shared_expert(0, 48, z(48 * H // 32 * 34, np.uint8), M.Q8_0, z(48 * H // 32 * 34, np.uint8), M.Q8_0,
+                                 z(10, np.uint8), M.Q4_K)
+        with pytest.raises(M.MoeError, match="share one type"):
+            m.load_shared_expert(0, 64, z(64 * H // 32 * 34, np.uint8), M.Q8_0, z(64 * H, np.float32), M.F32,
+                                 z(H * 64, np.float32), M.F32)
