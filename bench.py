@@ -44,6 +44,7 @@ WORKLOADS = {
     "olmoe_q4k_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q4_K", router="F16"),
     "olmoe_q8_0_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q8_0", router="F16"),
     "olmoe_f16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F16", router="F16"),
+    "olmoe_f32_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F32", router="F16"),
     "qwen3_a3b_q4k": dict(hidden=2048, inter=768, experts=128, top_k=8, norm=True, bank="Q4_K", router="F16"),
     # mixed bank types: llama.cpp's Q4_K_M recipe stores part of ffn_down as Q6_K; the shipped qwen4exp file has
     # Q4_K gate/up with Q5_1 downs, 512 experts, top-10 (models/qwen4exp/mod.rs:18-20, experts.rs:1838-1879)
@@ -51,7 +52,7 @@ WORKLOADS = {
     "qwen4exp_decode": dict(hidden=2560, inter=640, experts=512, top_k=10, norm=True, bank="Q4_K", down="Q5_1", router="F16",
                             flavour=1),
 }
-BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "Q6_K": 14, "Q5_1": 7, "Q5_K": 13}
+BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "F32": 0, "Q6_K": 14, "Q5_1": 7, "Q5_K": 13}
 
 
 def main() -> int:
@@ -63,6 +64,8 @@ def main() -> int:
     ap.add_argument("--tokens", type=int, default=1, help="tokens per step (decode batch)")
     ap.add_argument("--layers", type=int, default=16, help="distinct layer banks the steps rotate over")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--stack", action="store_true",
+                    help="a step is x <- x + MoE_l(RmsNorm_l(x)) through all --layers layers (reported per layer)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--seed", type=int, default=1234)
@@ -94,10 +97,11 @@ def main() -> int:
 
     def make_bank(in_dim, out_dim, seed, t=None):
         t = bank_t if t is None else t
-        if t != M.F16:
+        if t not in (M.F16, M.F32):
             return synth.random_bank_fast(t, [in_dim, out_dim, E], seed)
         gg = np.random.Generator(np.random.PCG64(seed))
-        return (gg.standard_normal(E * out_dim * in_dim, dtype=np.float32) * np.float32(0.02)).astype(np.float16).view(np.uint8)
+        w32 = gg.standard_normal(E * out_dim * in_dim, dtype=np.float32) * np.float32(0.02)
+        return (w32 if t == M.F32 else w32.astype(np.float16)).view(np.uint8)
 
     t_setup = time.time()
     moe = M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=max(n, 8), norm_topk_prob=norm,
@@ -109,7 +113,7 @@ def main() -> int:
         gate = make_bank(H, I, args.seed * 1000 + 3 * l)
         up = make_bank(H, I, args.seed * 1000 + 3 * l + 1)
         down = make_bank(I, H, args.seed * 1000 + 3 * l + 2, down_t)
-        moe.load_layer(l, router, router_t, gate, bank_t, up, bank_t, down, down_t)
+        moe.load_layer(l, router, router_t, gate, bank_t, up, bank_t, down, down_t, np.ones(H, np.float32) if args.stack else None)
         routers.append(router)
         if l == 0:
             keep_layer0 = (router, gate, up, down)
@@ -136,13 +140,18 @@ def main() -> int:
     mean_distinct = float(np.mean(list(distinct.values())))
 
     def step(s):
-        moe.forward_device(s % L, x_dev[s % pool], n, k, norm, out_dev)
+        if args.stack:
+            moe.stack_forward_device(x_dev[s % pool], n, k, norm, out_dev)
+        else:
+            moe.forward_device(s % L, x_dev[s % pool], n, k, norm, out_dev)
 
     use_graph = not args.no_graph
     graph = None
     steps_per_launch = 1
     if use_graph:
         steps_per_launch = period if period <= 1024 else L
+        if args.stack:
+            steps_per_launch = min(pool, 16)
         moe.graph_begin()
         for s in range(steps_per_launch):
             step(s)
@@ -178,8 +187,9 @@ def main() -> int:
     wall = time.perf_counter() - t0
     moe.check()
 
-    ms_per_step = wall * 1e3 / args.steps
-    value = n * args.steps / wall
+    layers_per_step = L if args.stack else 1
+    ms_per_step = wall * 1e3 / args.steps / layers_per_step  # per layer
+    value = n * args.steps * layers_per_step / wall
 
     # per-kernel durations: eager launches bracketed by HIP events on the library's stream
     moe.kernel_timing(True)
@@ -205,7 +215,7 @@ def main() -> int:
     # batched calls: matrix-core rate of the two grouped GEMMs (2*H*I flops per assignment and projection)
     mfma = None
     if per_kernel_us.get("gemm_gate_up") and per_kernel_us.get("gemm_down"):
-        peak = 2500.0 if w["bank"] == "F16" else 5000.0  # dense f16 TFLOP/s, int8 TOP/s
+        peak = 2500.0 if w["bank"] in ("F16", "F32") else 5000.0  # dense f16 TFLOP/s, int8 TOP/s
         gu_t = n * k * 2 * 2 * H * I / (per_kernel_us["gemm_gate_up"] * 1e-6) / 1e12
         dn_t = n * k * 2 * H * I / (per_kernel_us["gemm_down"] * 1e-6) / 1e12
         mfma = {"unit": "TFLOP/s" if w["bank"] == "F16" else "TOP/s", "peak": peak, "gemm_gate_up": round(gu_t, 1),
@@ -223,15 +233,15 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if w["bank"] == "F16" else ("i8*i16->i32" if w["bank"] == "Q8_0" else "u4*i16->i32") +
+        "dtype": "f32" if w["bank"] in ("F16", "F32") else ("i8*i16->i32" if w["bank"] == "Q8_0" else "u4*i16->i32") +
                  " (v_dot4_i32_i8), f32 scales",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
-                   "tokens_per_step": n, "layers": L, "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
+                   "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
                    "mean_distinct_experts_per_step": round(mean_distinct, 3)},
         "us_per_layer": round(ms_per_step * 1e3, 3),
-        "event_ms_per_step": round(ev_ms / args.steps, 6),
+        "event_ms_per_step": round(ev_ms / args.steps / layers_per_step, 6),
         "layer_algorithmic_bytes": int(layer_bytes),
         "layer_hbm_gbs": round(layer_gbs, 1),
         "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4),

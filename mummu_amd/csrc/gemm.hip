@@ -535,6 +535,9 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                     const int16v cl1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al1, bq1, zero, 0, 0, 0);
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
+                        // accumulator rows 8j..8j+7 of this 32-row block: past the tile's rows there is
+                        // nothing to scale (ragged experts leave most of a tile empty at small batches)
+                        if (GATE_UP && 32 * m + 8 * j >= rows) continue;  // (the down kernel measures faster without the test)
                         const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
                         const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
@@ -564,7 +567,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     const int arow = 32 * m + (lane & 31);
-                    float t[16];
+                    float t[16] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const long ah = *(const long *)(s_a(0, arow) + 16 * j + 8 * g), al = *(const long *)(s_a(1, arow) + 16 * j + 8 * g);
@@ -573,6 +576,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                         const int16v cl = __builtin_amdgcn_mfma_i32_32x32x16_i8(al, bq[j], zero, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
+                            if (GATE_UP && 32 * m + 8 * (r >> 2) >= rows) continue;  // rows past the tile's: nothing to scale
                             const float f = (float)((ch[r] << 8) + cl[r]);
                             t[r] = j == 0 ? __fmul_rn(dj[0], f) : fmaf(dj[j], f, t[r]);
                         }
@@ -581,8 +585,10 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                     for (int j = 0; j < 4; j++) {
                         const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
                         const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+                        if (!GATE_UP || 32 * m + 8 * j < rows) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++) acc[b][m][4 * j + i] = fmaf(t[4 * j + i], sr[i], acc[b][m][4 * j + i]);
+                            for (int i = 0; i < 4; i++) acc[b][m][4 * j + i] = fmaf(t[4 * j + i], sr[i], acc[b][m][4 * j + i]);
+                        }
                     }
                 }
             }

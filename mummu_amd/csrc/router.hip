@@ -448,36 +448,60 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
 }
 
 // ---------------------------------------------------------------------------------------
-// RmsNorm, one wave per token: sum of squares in the router's 512-partial order, then
-// (x * (1/sqrt(mean + eps))) * gamma with every step rounded separately.
+// RmsNorm, one workgroup per token: sum of squares in the router's 512-partial order (every wave
+// computes it for itself, from the same loads in the same order, so all hold the same bits), then
+// (x * (1/sqrt(mean + eps))) * gamma with every step rounded separately, the row split over the
+// workgroup's threads in 16-byte pieces.
 // ---------------------------------------------------------------------------------------
+template <bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
-                                                      float eps, int n, int hidden, float *__restrict__ out) {
+                                                      float eps, int hidden, float *__restrict__ out) {
     const int lane = threadIdx.x & 63;
-    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (t >= n) return;
+    const int t = blockIdx.x;
     const float *row = x + (size_t)t * (size_t)hidden;
     float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 4
     for (int base = lane * 8; base < hidden; base += 512) {
+        float v[8];
+        if (VEC) {  // hidden % 8 == 0: the lane's 8 elements are all inside the row
+            const float4 p = *(const float4 *)(row + base), q = *(const float4 *)(row + base + 4);
+            v[0] = p.x; v[1] = p.y; v[2] = p.z; v[3] = p.w; v[4] = q.x; v[5] = q.y; v[6] = q.z; v[7] = q.w;
+        } else {
 #pragma unroll
-        for (int j = 0; j < 8; j++)
-            if (base + j < hidden) {
-                float v = row[base + j];
-                a[j] = __builtin_fmaf(v, v, a[j]);
-            }
+            for (int j = 0; j < 8; j++) v[j] = base + j < hidden ? row[base + j] : 0.0f;  // +0 leaves a partial unchanged
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) a[j] = __builtin_fmaf(v[j], v[j], a[j]);
     }
     float ss = __fadd_rn(__fadd_rn(__fadd_rn(a[0], a[4]), __fadd_rn(a[1], a[5])),
                          __fadd_rn(__fadd_rn(a[2], a[6]), __fadd_rn(a[3], a[7])));
     ss = wave_sum(ss);
-    float mean = __fdiv_rn(ss, (float)hidden);
-    float r = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, eps)));
-    for (int i = lane; i < hidden; i += 64) out[(size_t)t * hidden + i] = __fmul_rn(__fmul_rn(row[i], r), gamma[i]);
+    const float mean = __fdiv_rn(ss, (float)hidden);
+    const float r = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(mean, eps)));
+    float *orow = out + (size_t)t * (size_t)hidden;
+    if (VEC) {
+#pragma unroll 2
+        for (int i = threadIdx.x * 4; i < hidden; i += 4 * blockDim.x) {
+            const float4 xv = *(const float4 *)(row + i), g = *(const float4 *)(gamma + i);
+            float4 o;
+            o.x = __fmul_rn(__fmul_rn(xv.x, r), g.x);
+            o.y = __fmul_rn(__fmul_rn(xv.y, r), g.y);
+            o.z = __fmul_rn(__fmul_rn(xv.z, r), g.z);
+            o.w = __fmul_rn(__fmul_rn(xv.w, r), g.w);
+            *(float4 *)(orow + i) = o;
+        }
+    } else {
+#pragma unroll 4
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) orow[i] = __fmul_rn(__fmul_rn(row[i], r), gamma[i]);
+    }
 }
 
 hipError_t launch_rmsnorm(const float *x, const float *gamma, float eps, int n, int hidden, float *out, hipStream_t s) {
     if (n <= 0) return hipSuccess;
-    dim3 block(256), grid((n + 3) / 4);
-    launch_kernel(rmsnorm_kernel, grid, block, 0, s, x, gamma, eps, n, hidden, out);
+    const bool vec = hidden % 8 == 0 && (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)out) & 15) == 0;
+    dim3 block(256), grid(n);
+    if (vec) launch_kernel(rmsnorm_kernel<true>, grid, block, 0, s, x, gamma, eps, hidden, out);
+    else launch_kernel(rmsnorm_kernel<false>, grid, block, 0, s, x, gamma, eps, hidden, out);
     return hipGetLastError();
 }
 
