@@ -21,6 +21,7 @@ MUMMU_TRACE_UNIT(router)
 namespace mummu {
 
 constexpr int kRouterTokensPerBlock = 4;
+constexpr int kRouterChunks = 4;  // rows of up to 2048 elements take the all-loads-first form at one token
 
 // One wave per expert row; the wave walks the row in chunks of 512 elements and serves
 // kRouterTokensPerBlock tokens from each loaded weight chunk.
@@ -34,7 +35,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
     const int t0 = blockIdx.x * kRouterTokensPerBlock;
     // this wave's share of the activation quantization for the integer expert products:
     // 64-element slices of the tile's rows, dealt round-robin over the tile's waves
-    if (xq.hi != nullptr) {
+    auto quantize_share = [&]() {
+        if (xq.hi == nullptr) return;
         const int nwaves = blockDim.x >> 6;
         const int slices_per_row = hidden / 64;  // hidden % 64 == 0 is checked by the launcher
         const int tile_tokens = (n - t0) < kRouterTokensPerBlock ? (n - t0) : kRouterTokensPerBlock;
@@ -43,7 +45,9 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
             const int elem = (sl % slices_per_row) * 64 + lane;
             quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
         }
-    }
+    };
+    const bool one_token_fast = VEC && hidden <= 512 * kRouterChunks && n - t0 == 1 && e < n_experts;
+    if (!one_token_fast) quantize_share();  // (the fast form does it under its own loads, below)
     if (e >= n_experts) return;
     float acc[kRouterTokensPerBlock][8];
 #pragma unroll
@@ -52,30 +56,55 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
         for (int j = 0; j < 8; j++) acc[t][j] = 0.0f;
 
     const size_t wrow = (size_t)e * (size_t)hidden;
-    for (int base = lane * 8; base < hidden; base += 512) {
-        float wv[8];
-        int cnt = hidden - base < 8 ? hidden - base : 8;
-        if (VEC) {
-            load_w8<WT>(w, wrow + (size_t)base, wv);
-        } else {
+    if (one_token_fast) {
+        // one token, a row of at most kRouterChunks 512-element chunks: every load of the wave is issued
+        // before the first multiply (a loop would pay the memory latency once per chunk)
+        float wv[kRouterChunks][8];
+        float4 xa[kRouterChunks], xb[kRouterChunks];
+        const float *xr = x + (size_t)t0 * (size_t)hidden;
 #pragma unroll
-            for (int j = 0; j < 8; j++) wv[j] = j < cnt ? load_w<WT>(w, wrow + (size_t)(base + j)) : 0.0f;
+        for (int c = 0; c < kRouterChunks; c++) {
+            const int base = lane * 8 + 512 * c;
+            const bool on = base < hidden;
+            const int at = on ? base : 0;
+            load_w8<WT>(w, wrow + (size_t)at, wv[c]);
+            xa[c] = ((const float4 *)(xr + at))[0];
+            xb[c] = ((const float4 *)(xr + at))[1];
         }
+        quantize_share();  // its one load joins the ones above; its stores do not hold them back
 #pragma unroll
-        for (int t = 0; t < kRouterTokensPerBlock; t++) {
-            if (t0 + t >= n) break;
-            const float *xr = x + (size_t)(t0 + t) * (size_t)hidden + base;
-            float xv[8];
+        for (int c = 0; c < kRouterChunks; c++) {
+            if (lane * 8 + 512 * c >= hidden) continue;  // (never adds: keeps -0 partials impossible either way)
+            const float xv[8] = {xa[c].x, xa[c].y, xa[c].z, xa[c].w, xb[c].x, xb[c].y, xb[c].z, xb[c].w};
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[0][j] = __builtin_fmaf(xv[j], wv[c][j], acc[0][j]);
+        }
+    } else {
+        for (int base = lane * 8; base < hidden; base += 512) {
+            float wv[8];
+            int cnt = hidden - base < 8 ? hidden - base : 8;
             if (VEC) {
-                float4 a = ((const float4 *)xr)[0], b = ((const float4 *)xr)[1];
-                xv[0] = a.x; xv[1] = a.y; xv[2] = a.z; xv[3] = a.w; xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
+                load_w8<WT>(w, wrow + (size_t)base, wv);
             } else {
 #pragma unroll
-                for (int j = 0; j < 8; j++) xv[j] = j < cnt ? xr[j] : 0.0f;
+                for (int j = 0; j < 8; j++) wv[j] = j < cnt ? load_w<WT>(w, wrow + (size_t)(base + j)) : 0.0f;
             }
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                if (VEC || j < cnt) acc[t][j] = __builtin_fmaf(xv[j], wv[j], acc[t][j]);
+            for (int t = 0; t < kRouterTokensPerBlock; t++) {
+                if (t0 + t >= n) break;
+                const float *xr = x + (size_t)(t0 + t) * (size_t)hidden + base;
+                float xv[8];
+                if (VEC) {
+                    float4 a = ((const float4 *)xr)[0], b = ((const float4 *)xr)[1];
+                    xv[0] = a.x; xv[1] = a.y; xv[2] = a.z; xv[3] = a.w; xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) xv[j] = j < cnt ? xr[j] : 0.0f;
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (VEC || j < cnt) acc[t][j] = __builtin_fmaf(xv[j], wv[j], acc[t][j]);
+            }
         }
     }
 #pragma unroll
