@@ -75,10 +75,14 @@ __device__ inline void load_lane_act(const QAct &q, size_t row, int d, int unit0
         a.xh[i][4] = h1.x; a.xh[i][5] = h1.y; a.xh[i][6] = h1.z; a.xh[i][7] = h1.w;
         a.xl[i][0] = l0.x; a.xl[i][1] = l0.y; a.xl[i][2] = l0.z; a.xl[i][3] = l0.w;
         a.xl[i][4] = l1.x; a.xl[i][5] = l1.y; a.xl[i][6] = l1.z; a.xl[i][7] = l1.w;
-        a.s[i][0] = on ? sc[e0 >> 4] : 0.0f;
-        a.s[i][1] = on ? sc[e1 >> 4] : 0.0f;
-        a.sx[i][0] = on ? sm[e0 >> 4] : 0;
-        a.sx[i][1] = on ? sm[e1 >> 4] : 0;
+        // loaded whatever `on` says (the addresses are valid either way) and zeroed afterwards: a load
+        // under a condition becomes a branch with a full wait in front of the loads that follow it
+        const float s0 = sc[e0 >> 4], s1 = sc[e1 >> 4];
+        const int x0 = sm[e0 >> 4], x1 = sm[e1 >> 4];
+        a.s[i][0] = on ? s0 : 0.0f;
+        a.s[i][1] = on ? s1 : 0.0f;
+        a.sx[i][0] = on ? x0 : 0;
+        a.sx[i][1] = on ? x1 : 0;
         a.fsx[i][0] = __fmul_rn(a.s[i][0], (float)a.sx[i][0]);
         a.fsx[i][1] = __fmul_rn(a.s[i][1], (float)a.sx[i][1]);
     }
