@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
 # same command (profiles/olmoe_q4k_decode_hbm_traffic.txt), each scaled by what the counter
 # reads for the library's 256 MiB copy kernel.  Only for the workload/batch they were taken on.
-PROFILED_TRAFFIC = {("olmoe_q4k_decode", 1, "gate_up"): 19139427}
+PROFILED_TRAFFIC = {("olmoe_q4k_decode", 1, "gate_up"): 19146025}
 
 WORKLOADS = {
     # name: (hidden, inter, experts, top_k, norm, bank type, router type)

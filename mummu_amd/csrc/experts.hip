@@ -99,8 +99,10 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
                 route.weights[(size_t)t * k + lane] = s_w[lane];
                 if (route.hits) atomicAdd(&route.hits[id], 1ULL);
             }
+            MUMMU_PHASE(6);
         }
         __syncthreads();
+        MUMMU_PHASE(7);
     }
     const int e = ROUTE ? s_ids[blockIdx.x] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
     if ((unsigned)e >= (unsigned)n_experts) {
