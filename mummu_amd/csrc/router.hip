@@ -28,25 +28,26 @@ constexpr int kRouterChunks = 4;  // rows of up to 2048 elements take the all-lo
 template <int WT, bool VEC>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x, const void *__restrict__ w,
                                                             float *__restrict__ logits, int n, int hidden,
-                                                            int n_experts, QAct xq) {
+                                                            int n_experts, QAct xq, int tokens_per_block) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int e = blockIdx.y * (blockDim.x >> 6) + wave;
-    const int t0 = blockIdx.x * kRouterTokensPerBlock;
+    const int t0 = blockIdx.x * tokens_per_block;  // tokens_per_block <= kRouterTokensPerBlock
+    const int n_here = (n - t0) < tokens_per_block ? (n - t0) : tokens_per_block;
     // this wave's share of the activation quantization for the integer expert products:
     // 64-element slices of the tile's rows, dealt round-robin over the tile's waves
     auto quantize_share = [&]() {
         if (xq.hi == nullptr) return;
         const int nwaves = blockDim.x >> 6;
         const int slices_per_row = hidden / 64;  // hidden % 64 == 0 is checked by the launcher
-        const int tile_tokens = (n - t0) < kRouterTokensPerBlock ? (n - t0) : kRouterTokensPerBlock;
+        const int tile_tokens = n_here;
         for (int sl = blockIdx.y * nwaves + wave; sl < tile_tokens * slices_per_row; sl += gridDim.y * nwaves) {
             const int t = t0 + sl / slices_per_row;
             const int elem = (sl % slices_per_row) * 64 + lane;
             quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
         }
     };
-    const bool one_token_fast = VEC && hidden <= 512 * kRouterChunks && n - t0 == 1 && e < n_experts;
+    const bool one_token_fast = VEC && hidden <= 512 * kRouterChunks && n_here == 1 && e < n_experts;
     if (!one_token_fast) quantize_share();  // (the fast form does it under its own loads, below)
     if (e >= n_experts) return;
     float acc[kRouterTokensPerBlock][8];
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
             }
 #pragma unroll
             for (int t = 0; t < kRouterTokensPerBlock; t++) {
-                if (t0 + t >= n) break;
+                if (t >= n_here) break;
                 const float *xr = x + (size_t)(t0 + t) * (size_t)hidden + base;
                 float xv[8];
                 if (VEC) {
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
     }
 #pragma unroll
     for (int t = 0; t < kRouterTokensPerBlock; t++) {
-        if (t0 + t >= n) break;
+        if (t >= n_here) break;
         const float *a = acc[t];
         float s = __fadd_rn(__fadd_rn(__fadd_rn(a[0], a[4]), __fadd_rn(a[1], a[5])),
                             __fadd_rn(__fadd_rn(a[2], a[6]), __fadd_rn(a[3], a[7])));
@@ -125,12 +126,14 @@ hipError_t launch_router_logits(const float *x, const void *w, int wtype, float 
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
     // few tokens: one wave per workgroup so the expert rows spread over as many CUs as possible
     const int waves = n <= 8 ? 1 : 4;
+    // ... and one token per workgroup, which takes the all-loads-first form of the kernel
+    const int tpb = n <= 8 ? 1 : kRouterTokensPerBlock;
     dim3 block(64 * waves);
-    dim3 grid((n + kRouterTokensPerBlock - 1) / kRouterTokensPerBlock, (n_experts + waves - 1) / waves);
+    dim3 grid((n + tpb - 1) / tpb, (n_experts + waves - 1) / waves);
 #define MUMMU_LAUNCH_ROUTER(WT)                                                                          \
     do {                                                                                                 \
-        if (vec) launch_kernel(router_logits_kernel<WT, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq);  \
-        else launch_kernel(router_logits_kernel<WT, false>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq);     \
+        if (vec) launch_kernel(router_logits_kernel<WT, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb);  \
+        else launch_kernel(router_logits_kernel<WT, false>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb);     \
     } while (0)
     switch (wtype) {
     case T_F32: MUMMU_LAUNCH_ROUTER(T_F32); break;
