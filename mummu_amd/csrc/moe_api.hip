@@ -322,14 +322,27 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
     return MUMMU_OK;
 }
 
+// The three-launch decode form (router logits + quantization, gate/up with the routing inside,
+// down + combine): nothing but the first launch reads the float activations.
+bool decode_three_launches(const mummu_moe *h, const Layer &L, int64_t n, int k) {
+    const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
+    const ExpertBanks b = banks_of(h, L);
+    const bool batched = n >= h->gemm_min_tokens && grouped_gemm_supported(b);
+    const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0 && !batched;
+    return !(n > 8 && router_fused_supported(E)) && want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k);
+}
+
+// norm_gamma != nullptr (only where decode_three_launches holds): x is the raw residual stream and the
+// first launch applies the layer's RmsNorm itself.
 int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
-                hipStream_t s) {
+                hipStream_t s, const float *norm_gamma = nullptr) {
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
     const bool batched = n >= h->gemm_min_tokens && grouped_gemm_supported(banks_of(h, L));
     const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0 && !batched;
     const QAct xq = want_xq ? h->xq : QAct();
+    if (norm_gamma && !decode_three_launches(h, L, n, k)) return fail(h, MUMMU_ERR_ARG, "fused RmsNorm outside the decode form");
     if (n > 8 && router_fused_supported(E)) {
         // many tokens: one workgroup per token tile does logits, routing and quantization
         // on the batched path the dispatch adds the per-expert row counts to the hit counters
@@ -339,7 +352,8 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
         return run_experts(h, L, x, want_xq, n, k, residual, out, s, batched);
     } else {
         // few tokens: the router rows are spread over as many CUs as there are experts
-        LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s));
+        LAUNCH(h, K_ROUTER_LOGITS, s,
+               launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s, norm_gamma, h->cfg.rms_norm_eps));
         const ExpertBanks b = banks_of(h, L);
         if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
             // ... and the gate/up kernel routes by itself: one launch less on the decode path
@@ -365,9 +379,10 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
 //     out = [residual +] (routed + shared_ffn(x) * sigmoid(<gate_vec, x>))
 // with the product and the two sums rounded separately, in that grouping.
 int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
-                 hipStream_t s) {
+                 hipStream_t s, const float *norm_gamma = nullptr) {
     const Layer &L = h->layers[layer];
-    if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s);
+    if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s, norm_gamma);
+    if (norm_gamma) return fail(h, MUMMU_ERR_ARG, "fused RmsNorm with a shared expert");
     int rc = routed_impl(h, layer, x, n, k, norm, nullptr, out, s);
     if (rc) return rc;
     if (n > h->sh_ws_tokens) return fail(h, MUMMU_ERR_TOKENS, "shared-expert workspace is smaller than the call");
@@ -413,8 +428,15 @@ int stack_impl(mummu_moe *h, const float *x, int64_t n, int k, int norm, float *
     for (int l = 0; l < nl; l++) {
         const float *src = l == 0 ? x : h->resid[(l - 1) & 1];
         float *dst = l == nl - 1 ? out : h->resid[l & 1];
-        LAUNCH(h, K_RMSNORM, s, launch_rmsnorm(src, h->layers[l].gamma, h->cfg.rms_norm_eps, (int)n, H, h->h2, s));
-        int rc = forward_impl(h, l, h->h2, n, k, norm, src, dst, s);
+        const Layer &L = h->layers[l];
+        int rc;
+        if (!L.sh_loaded && decode_three_launches(h, L, n, k) && router_logits_can_norm(src, L.router, L.gamma, (int)n, H)) {
+            // decode: the router launch normalises the row it already holds; no launch of its own
+            rc = forward_impl(h, l, src, n, k, norm, src, dst, s, L.gamma);
+        } else {
+            LAUNCH(h, K_RMSNORM, s, launch_rmsnorm(src, L.gamma, h->cfg.rms_norm_eps, (int)n, H, h->h2, s));
+            rc = forward_impl(h, l, h->h2, n, k, norm, src, dst, s);
+        }
         if (rc) return rc;
         if (ids_host) {
             HIPCHK(h, hipStreamSynchronize(s));

@@ -25,10 +25,14 @@ constexpr int kRouterChunks = 4;  // rows of up to 2048 elements take the all-lo
 
 // One wave per expert row; the wave walks the row in chunks of 512 elements and serves
 // kRouterTokensPerBlock tokens from each loaded weight chunk.
-template <int WT, bool VEC>
+// NORM: x is the raw residual stream and the kernel works on RmsNorm(x) = (x * r) * gamma instead,
+// r from the sum of squares in the same 512-partial order the RmsNorm kernel uses - the wave already
+// holds the row in exactly that layout.  Only in the one-token form (the launcher sees to it).
+template <int WT, bool VEC, bool NORM = false>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x, const void *__restrict__ w,
                                                             float *__restrict__ logits, int n, int hidden,
-                                                            int n_experts, QAct xq, int tokens_per_block) {
+                                                            int n_experts, QAct xq, int tokens_per_block,
+                                                            const float *__restrict__ gamma, float eps) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int e = blockIdx.y * (blockDim.x >> 6) + wave;
@@ -36,7 +40,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
     const int n_here = (n - t0) < tokens_per_block ? (n - t0) : tokens_per_block;
     // this wave's share of the activation quantization for the integer expert products:
     // 64-element slices of the tile's rows, dealt round-robin over the tile's waves
-    auto quantize_share = [&]() {
+    auto quantize_share = [&](float r) {
         if (xq.hi == nullptr) return;
         const int nwaves = blockDim.x >> 6;
         const int slices_per_row = hidden / 64;  // hidden % 64 == 0 is checked by the launcher
@@ -44,11 +48,13 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
         for (int sl = blockIdx.y * nwaves + wave; sl < tile_tokens * slices_per_row; sl += gridDim.y * nwaves) {
             const int t = t0 + sl / slices_per_row;
             const int elem = (sl % slices_per_row) * 64 + lane;
-            quantize_store16(x[(size_t)t * (size_t)hidden + elem], true, xq, (size_t)t, hidden, elem);
+            float v = x[(size_t)t * (size_t)hidden + elem];
+            if (NORM) v = __fmul_rn(__fmul_rn(v, r), gamma[elem]);
+            quantize_store16(v, true, xq, (size_t)t, hidden, elem);
         }
     };
     const bool one_token_fast = VEC && hidden <= 512 * kRouterChunks && n_here == 1 && e < n_experts;
-    if (!one_token_fast) quantize_share();  // (the fast form does it under its own loads, below)
+    if (!one_token_fast) quantize_share(1.0f);  // (the fast form does it under its own loads, below)
     if (e >= n_experts) return;
     float acc[kRouterTokensPerBlock][8];
 #pragma unroll
@@ -72,7 +78,41 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
             xa[c] = ((const float4 *)(xr + at))[0];
             xb[c] = ((const float4 *)(xr + at))[1];
         }
-        quantize_share();  // its one load joins the ones above; its stores do not hold them back
+        float r = 1.0f;
+        if (NORM) {
+            float4 ga[kRouterChunks], gb[kRouterChunks];
+#pragma unroll
+            for (int c = 0; c < kRouterChunks; c++) {
+                const int base = lane * 8 + 512 * c;
+                const int at = base < hidden ? base : 0;
+                ga[c] = ((const float4 *)(gamma + at))[0];
+                gb[c] = ((const float4 *)(gamma + at))[1];
+            }
+            float a2[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int c = 0; c < kRouterChunks; c++) {
+                if (lane * 8 + 512 * c >= hidden) continue;
+                const float xv[8] = {xa[c].x, xa[c].y, xa[c].z, xa[c].w, xb[c].x, xb[c].y, xb[c].z, xb[c].w};
+#pragma unroll
+                for (int j = 0; j < 8; j++) a2[j] = __builtin_fmaf(xv[j], xv[j], a2[j]);
+            }
+            float ss = __fadd_rn(__fadd_rn(__fadd_rn(a2[0], a2[4]), __fadd_rn(a2[1], a2[5])),
+                                 __fadd_rn(__fadd_rn(a2[2], a2[6]), __fadd_rn(a2[3], a2[7])));
+            ss = wave_sum(ss);
+            r = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, (float)hidden), eps)));
+#pragma unroll
+            for (int c = 0; c < kRouterChunks; c++) {
+                xa[c].x = __fmul_rn(__fmul_rn(xa[c].x, r), ga[c].x);
+                xa[c].y = __fmul_rn(__fmul_rn(xa[c].y, r), ga[c].y);
+                xa[c].z = __fmul_rn(__fmul_rn(xa[c].z, r), ga[c].z);
+                xa[c].w = __fmul_rn(__fmul_rn(xa[c].w, r), ga[c].w);
+                xb[c].x = __fmul_rn(__fmul_rn(xb[c].x, r), gb[c].x);
+                xb[c].y = __fmul_rn(__fmul_rn(xb[c].y, r), gb[c].y);
+                xb[c].z = __fmul_rn(__fmul_rn(xb[c].z, r), gb[c].z);
+                xb[c].w = __fmul_rn(__fmul_rn(xb[c].w, r), gb[c].w);
+            }
+        }
+        quantize_share(r);  // its loads join the ones above; its stores do not hold them back
 #pragma unroll
         for (int c = 0; c < kRouterChunks; c++) {
             if (lane * 8 + 512 * c >= hidden) continue;  // (never adds: keeps -0 partials impossible either way)
@@ -119,10 +159,16 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
     }
 }
 
+bool router_logits_can_norm(const float *x, const void *w, const float *gamma, int n, int hidden) {
+    return n >= 1 && n <= 8 && hidden % 64 == 0 && hidden <= 512 * kRouterChunks &&
+           (((uintptr_t)x | (uintptr_t)w | (uintptr_t)gamma) & 15) == 0;
+}
+
 hipError_t launch_router_logits(const float *x, const void *w, int wtype, float *logits, int n, int hidden,
-                                int n_experts, QAct xq, hipStream_t s) {
+                                int n_experts, QAct xq, hipStream_t s, const float *norm_gamma, float norm_eps) {
     if (n <= 0) return hipSuccess;
     if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
+    if (norm_gamma && !router_logits_can_norm(x, w, norm_gamma, n, hidden)) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
     // few tokens: one wave per workgroup so the expert rows spread over as many CUs as possible
     const int waves = n <= 8 ? 1 : 4;
@@ -130,10 +176,17 @@ hipError_t launch_router_logits(const float *x, const void *w, int wtype, float 
     const int tpb = n <= 8 ? 1 : kRouterTokensPerBlock;
     dim3 block(64 * waves);
     dim3 grid((n + tpb - 1) / tpb, (n_experts + waves - 1) / waves);
-#define MUMMU_LAUNCH_ROUTER(WT)                                                                          \
-    do {                                                                                                 \
-        if (vec) launch_kernel(router_logits_kernel<WT, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb);  \
-        else launch_kernel(router_logits_kernel<WT, false>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb);     \
+#define MUMMU_LAUNCH_ROUTER(WT)                                                                                       \
+    do {                                                                                                              \
+        if (norm_gamma)                                                                                               \
+            launch_kernel(router_logits_kernel<WT, true, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb, \
+                          norm_gamma, norm_eps);                                                                      \
+        else if (vec)                                                                                                 \
+            launch_kernel(router_logits_kernel<WT, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb, \
+                          (const float *)nullptr, 0.0f);                                                              \
+        else                                                                                                          \
+            launch_kernel(router_logits_kernel<WT, false>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb, \
+                          (const float *)nullptr, 0.0f);                                                              \
     } while (0)
     switch (wtype) {
     case T_F32: MUMMU_LAUNCH_ROUTER(T_F32); break;

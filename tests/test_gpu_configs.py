@@ -234,6 +234,39 @@ def test_c4_q8_0_stack_prefill_256_tokens_two_layers():
     check_stack(*run_c4(2, 256, 500), tol=9e-3)
 
 
+@pytest.mark.parametrize("H,I,E,k,gt", [(2048, 256, 64, 8, M.Q4_K), (512, 128, 8, 2, M.Q8_0), (1280, 128, 16, 4, M.Q5_0),
+                                        (2560, 128, 16, 4, M.Q8_0)],
+                         ids=["2048", "512", "1280-ragged-chunk", "2560-too-wide-to-fuse"])
+def test_decode_stack_with_the_norm_inside_the_router_launch_equals_the_separate_norm(H, I, E, k, gt):
+    # up to 8 tokens the stack applies RmsNorm inside the router launch; from 9 on a kernel of its own
+    # writes the normalised rows first.  Both must give a token the same bits, layer after layer (the
+    # decode kernels serve both sizes, and a token's result does not depend on its batch), and the
+    # first layer must agree with the oracle's RmsNorm + routing exactly.
+    L = 3
+    g = np.random.Generator(np.random.PCG64(H + E))
+    layers = []
+    for l in range(L):
+        gate = synth.random_bank_fast(gt, [H, I, E], 10 * l + 1)
+        up = synth.random_bank_fast(gt, [H, I, E], 10 * l + 2)
+        down = synth.random_bank_fast(gt, [I, H, E], 10 * l + 3)
+        router = normal((E, H), 10 * l + 4, 0.05).astype(np.float16)
+        gamma = (1.0 + 0.2 * g.standard_normal(H)).astype(np.float32)
+        layers.append((router, gate, up, down, gamma))
+    x = normal((12, H), 77, 3.0)
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=12, rms_norm_eps=1e-6) as m:
+        for l, (router, gate, up, down, gamma) in enumerate(layers):
+            m.load_layer(l, router, M.F16, gate, gt, up, gt, down, gt, rms_gamma=gamma)
+        many, many_ids = m.stack_forward(x, k, True, return_ids=True)
+        for n in (1, 3, 8):
+            few, few_ids = m.stack_forward(x[:n], k, True, return_ids=True)
+            assert np.array_equal(few_ids, many_ids[:, :n])
+            assert np.array_equal(bits(few), bits(many[:n])), f"{n} tokens"
+    router, gate, up, down, gamma = layers[0]
+    h2 = orc.rmsnorm(x, gamma, 1e-6)
+    _, ids, _, _ = orc.moe_forward(orc.LayerBanks(H, I, E, gate, up, down, gt), router, orc.F16, h2, k, True)
+    assert np.array_equal(many_ids[0], ids.astype(np.int32))
+
+
 def test_c4_q8_0_prefill_layer_against_the_f64_reference():
     # one full-size Q8_0 layer at 256 tokens (grouped GEMM), per element, the reference's measure
     H, I, E, k = OLMOE["H"], OLMOE["I"], OLMOE["E"], OLMOE["k"]
