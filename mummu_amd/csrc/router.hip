@@ -339,18 +339,25 @@ constexpr int kRouterMaxChunks = 4;  // 512-element chunks of a row held in regi
 // flight while the current one is multiplied.  The wave-wide sum leaves logit e in lane e%64, which
 // is the layout the routing step wants, so nothing goes through LDS but the routing scratch and
 // nothing waits on another wave.  Same summation order as router_logits_kernel.
+// SPLIT > 1 (TT = 1), for batches too small to fill the chip with one wave per token: a workgroup
+// of SPLIT waves per token, wave w walking experts w, w + SPLIT, ...; the logits meet in LDS and
+// wave 0 routes.  The chain of dependent reductions a wave walks is SPLIT times shorter.
 constexpr int kStreamWaves = 4;
 
-template <int WT, int TT, int JN, int CHUNKS>
-__global__ __launch_bounds__(64 * kStreamWaves) void router_stream_kernel(
+template <int WT, int TT, int JN, int CHUNKS, int SPLIT = 1>
+__global__ __launch_bounds__(64 * (SPLIT > 1 ? SPLIT : kStreamWaves)) void router_stream_kernel(
     const float *__restrict__ x, const void *__restrict__ w, int n, int hidden, int n_experts, int k, int flavour,
     int norm, float *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ weights,
     unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
-    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[kStreamWaves];
+    static_assert(SPLIT == 1 || TT == 1, "a split token is one token");
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[SPLIT > 1 ? 1 : kStreamWaves];
+    __shared__ float s_logit[SPLIT > 1 ? 64 * JN : 1];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int t0 = (blockIdx.x * kStreamWaves + wave) * TT;
+    const int t0 = SPLIT > 1 ? (int)blockIdx.x : (blockIdx.x * kStreamWaves + wave) * TT;
     if (t0 >= n) return;
+    constexpr int ESTEP = SPLIT > 1 ? SPLIT : 1;
+    const int e_first = SPLIT > 1 ? wave : 0;
     MUMMU_PHASE(0);
 
     float xv[TT][CHUNKS][8];
@@ -385,9 +392,9 @@ __global__ __launch_bounds__(64 * kStreamWaves) void router_stream_kernel(
 #pragma unroll
         for (int j = 0; j < JN; j++) l[t][j] = 0.0f;
 
-    fetch_row(0);
+    fetch_row(e_first);
     MUMMU_PHASE(1);
-    for (int e = 0; e < n_experts; e++) {
+    for (int e = e_first; e < n_experts; e += ESTEP) {
         // take over the row that was in flight, start the next one, and only then touch the data:
         // the scheduling barriers keep the compiler from sinking the new loads' first use up here
 #pragma unroll
@@ -395,7 +402,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void router_stream_kernel(
 #pragma unroll
             for (int i = 0; i < WORDS; i++) cur[c][i] = raw[c][i];
         __builtin_amdgcn_sched_barrier(0);
-        fetch_row(e + 1);
+        fetch_row(e + ESTEP);
         __builtin_amdgcn_sched_barrier(0);
         float wv[CHUNKS][8];
 #pragma unroll
@@ -431,10 +438,20 @@ __global__ __launch_bounds__(64 * kStreamWaves) void router_stream_kernel(
 #pragma unroll
         for (int t = 0; t < TT; t++) {
             sum[t] = wave_sum(sum[t]);
+            if (SPLIT > 1) {
+                if (lane == 0) s_logit[e] = sum[t];
+            } else {
 #pragma unroll
-            for (int j = 0; j < JN; j++) l[t][j] = (e == lane + 64 * j) ? sum[t] : l[t][j];
+                for (int j = 0; j < JN; j++) l[t][j] = (e == lane + 64 * j) ? sum[t] : l[t][j];
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if (SPLIT > 1) {
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int j = 0; j < JN; j++) l[0][j] = (lane + 64 * j < n_experts) ? s_logit[lane + 64 * j] : 0.0f;
     }
     MUMMU_PHASE(2);
 #pragma unroll
@@ -443,7 +460,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void router_stream_kernel(
 #pragma unroll
         for (int j = 0; j < JN; j++)
             if (lane + 64 * j < n_experts) logits[(size_t)(t0 + t) * (size_t)n_experts + lane + 64 * j] = l[t][j];
-        route_token<JN>(l[t], t0 + t, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[wave]);
+        route_token<JN>(l[t], t0 + t, n_experts, k, flavour, norm, ids, weights, hits, flags, sc[SPLIT > 1 ? 0 : wave]);
         wave_lds_sync();
     }
     MUMMU_PHASE(3);
@@ -476,12 +493,23 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
     // enough tokens to fill the chip with independent waves: activations in registers, weight
     // rows streamed (on this path the caller quantizes x separately)
     if (n > 64 && vec && xq.hi == nullptr && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks) {
-        // two tokens per wave once there are enough waves to keep every SIMD busy, else one
+        // two tokens per wave once there are enough waves to keep every SIMD busy, else one; below a
+        // wave per SIMD a token gets a whole workgroup
         const int tt = n > 2048 ? 2 : 1;
+        const int split = n <= 512 ? 8 : (n <= 1024 ? 4 : (n <= 2048 ? 2 : 1));
         dim3 block(64 * kStreamWaves), grid((n + tt * kStreamWaves - 1) / (tt * kStreamWaves));
 #define MUMMU_RT3(WT, JN, CH)                                                                                            \
     do {                                                                                                                 \
-        if (tt == 2)                                                                                                     \
+        if (split == 8)                                                                                                  \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 8>, dim3(n), dim3(512), 0, s, x, w, n, hidden, n_experts, k, flavour, \
+                          norm, logits, ids, weights, hits, flags);                                                      \
+        else if (split == 4)                                                                                             \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 4>, dim3(n), dim3(256), 0, s, x, w, n, hidden, n_experts, k, flavour, \
+                          norm, logits, ids, weights, hits, flags);                                                      \
+        else if (split == 2)                                                                                             \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 2>, dim3(n), dim3(128), 0, s, x, w, n, hidden, n_experts, k, flavour, \
+                          norm, logits, ids, weights, hits, flags);                                                      \
+        else if (tt == 2)                                                                                                \
             launch_kernel(router_stream_kernel<WT, 2, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
                           logits, ids, weights, hits, flags);                                                            \
         else                                                                                                             \
