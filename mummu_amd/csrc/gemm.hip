@@ -37,7 +37,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kBN = 128;            // output rows per workgroup
 constexpr int kBK = 64;             // K step
 constexpr int kLds = kBK + 8;       // f16 LDS row (halfs): 144 B keeps 16-byte reads conflict-free
-constexpr int kLdsQ = kBK + 16;     // int8 LDS row (bytes): 80 B, likewise
 constexpr int kLdsC = kBN + 4;      // f32 staging row of the gate/up epilogue
 
 __device__ inline uint32_t pack_half2(float a, float b) {
@@ -399,12 +398,13 @@ __device__ inline void expand_q(const RawQ<WT> &r, int k0, int half, uint32_t (&
     }
 }
 
-template <bool GATE_UP, int MT>
+template <bool GATE_UP, int MT, int KS>
 struct QTileLds {
     static constexpr int NB = GATE_UP ? 2 : 1;
     static constexpr int BM = 32 * MT;
-    static constexpr int kA = 2 * BM * kLdsQ;                 // hi and lo planes
-    static constexpr int kB = NB * kBN * kLdsQ;
+    static constexpr int kRow = KS * kBK + 16;                // LDS row (bytes): 80 or 144 B keep 16-byte reads conflict-free
+    static constexpr int kA = 2 * BM * kRow;                  // hi and lo planes
+    static constexpr int kB = NB * kBN * kRow;
     static constexpr int kC = GATE_UP ? BM * kLdsC * 4 : 0;   // f32 staging of the epilogue (aliases A and B)
     static constexpr int kBytes = (kA + kB) > kC ? (kA + kB) : kC;
 };
@@ -412,22 +412,27 @@ struct QTileLds {
 // GATE_UP: A = xq rows gathered by token through `sorted`; epilogue quantizes silu(g)*u into
 //          act_out rows in sorted order.
 // else   : A = act_in rows in sorted order; y[pos, n] = f32 sum.
-template <int WT, bool GATE_UP, int MT>
+// KS: 64-element K steps staged per barrier pair.  With KS = 2 (in_dim a multiple of 128) the two
+// threads of a weight row each load and expand a whole step of their own instead of the two blocks
+// of one step: the same registers keep twice the bytes in flight, which is what a launch that
+// streams its weights with few rows per expert is short of; the arithmetic and its order per
+// output element are the same.
+template <int WT, bool GATE_UP, int MT, int KS>
 __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
     const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, QAct64 a_in, const int32_t *__restrict__ sorted,
     int k_slots, const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim,
     QAct64 act_out, float *__restrict__ y_out) {
-    using L = QTileLds<GATE_UP, MT>;
-    constexpr int NB = L::NB, BM = L::BM;
+    using L = QTileLds<GATE_UP, MT, KS>;
+    constexpr int NB = L::NB, BM = L::BM, kRow = L::kRow;
     __shared__ __attribute__((aligned(16))) uint8_t s_raw[L::kBytes];
-    __shared__ __attribute__((aligned(16))) float s_as[BM];       // activation scale of this K step, per tile row
-    __shared__ float s_am[BM][2];                                 // activation ssum of its two blocks
+    __shared__ __attribute__((aligned(16))) float s_as[KS][BM];   // activation scale of each K step, per tile row
+    __shared__ float s_am[BM][2 * KS];                            // activation ssum of their blocks
     constexpr bool OFFSET = gemm_has_offset(WT), SUB16 = gemm_sub16(WT);
     constexpr int NSC = SUB16 ? 4 : 2;
-    __shared__ float s_bd[NB][kBN][NSC];                          // weight scales of the K step (per 32 or per 16 elements)
-    __shared__ float s_bm[NB][kBN][2];                            // weight block offsets (types that have one)
-    auto s_a = [&](int plane, int row) -> uint8_t * { return s_raw + ((size_t)plane * BM + row) * kLdsQ; };
-    auto s_b = [&](int b, int row) -> uint8_t * { return s_raw + L::kA + ((size_t)b * kBN + row) * kLdsQ; };
+    __shared__ float s_bd[NB][kBN][NSC * KS];                     // weight scales of the K steps (per 32 or per 16 elements)
+    __shared__ float s_bm[NB][kBN][2 * KS];                       // weight block offsets (types that have one)
+    auto s_a = [&](int plane, int row) -> uint8_t * { return s_raw + ((size_t)plane * BM + row) * kRow; };
+    auto s_b = [&](int b, int row) -> uint8_t * { return s_raw + L::kA + ((size_t)b * kBN + row) * kRow; };
 
     int tile, slab;
     if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
@@ -436,8 +441,11 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t row_bytes = gemm_row_bytes(WT, in_dim);
 
-    // weight tile: thread -> (row, block of the K step)
+    // weight tile: thread -> (row, block of the K step), or with two steps per stage (row, step)
+    // and both blocks of that step
     const int b_row = tid >> 1, b_half = tid & 1;
+    constexpr bool SHARED = WT == T_Q4_K || WT == T_Q5_K;  // one load holds both blocks of a step
+    constexpr int NBLK = KS, NRAW = (KS == 2 && !SHARED) ? 2 : 1;
     const int b_out = n0 + b_row < out_dim ? n0 + b_row : out_dim - 1;  // clamped; never stored
     const uint8_t *b_ptr[NB];
     b_ptr[0] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes;
@@ -448,21 +456,23 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
         if (r >= rows) return -1;
         return GATE_UP ? sorted[p0 + r] / k_slots : p0 + r;
     };
-    // activation tile: thread -> (plane, row, 16-byte chunk), MT passes of 32 rows
-    const int a_plane = tid >> 7, a_chunk = tid & 3;
-    const int8_t *a_src[MT];
-    int a_row[MT];
+    // activation tile: thread -> (plane, row, 16-byte chunk), MT * KS passes of 32 / KS rows
+    constexpr int A_PASSES = MT * KS, A_CHUNKS = 4 * KS, A_ROWS = 32 / KS;
+    const int a_plane = tid >> 7, a_chunk = tid & (A_CHUNKS - 1);
+    const int8_t *a_src[A_PASSES];
+    int a_row[A_PASSES];
 #pragma unroll
-    for (int p = 0; p < MT; p++) {
-        a_row[p] = 32 * p + ((tid >> 2) & 31);
+    for (int p = 0; p < A_PASSES; p++) {
+        a_row[p] = A_ROWS * p + ((tid / A_CHUNKS) & (A_ROWS - 1));
         const int src = source_row(a_row[p]);
         a_src[p] = src < 0 ? nullptr : (a_plane ? a_in.lo : a_in.hi) + (size_t)src * (size_t)in_dim + a_chunk * 16;
     }
-    // its scales: thread t < BM -> scale of row t; thread t < 2*BM -> ssum of (row t/2, block t%2)
-    const int src_s = tid < BM ? source_row(tid) : -1;
-    const int src_m = tid < 2 * BM ? source_row(tid >> 1) : -1;
-    const float *as_ptr = src_s < 0 ? nullptr : a_in.scale + (size_t)src_s * (size_t)(in_dim / 64);
-    const float *am_ptr = src_m < 0 ? nullptr : a_in.ssum + (size_t)src_m * (size_t)(in_dim / 32) + (tid & 1);
+    // its scales: thread t < KS*BM -> scale of (row t % BM, step t / BM); thread t < 2*KS*BM -> ssum of
+    // (row t / (2 KS), block t % (2 KS))
+    const int src_s = tid < KS * BM ? source_row(tid % BM) : -1;
+    const int src_m = tid < 2 * KS * BM ? source_row(tid / (2 * KS)) : -1;
+    const float *as_ptr = src_s < 0 ? nullptr : a_in.scale + (size_t)src_s * (size_t)(in_dim / 64) + tid / BM;
+    const float *am_ptr = src_m < 0 ? nullptr : a_in.ssum + (size_t)src_m * (size_t)(in_dim / 32) + (tid & (2 * KS - 1));
 
     float16v acc[NB][MT];
 #pragma unroll
@@ -472,14 +482,21 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
 
-    RawQ<WT> rb[NB];
-    uint4 ra[MT];
+    RawQ<WT> rb[NB][NRAW];
+    uint4 ra[A_PASSES];
     float ras = 0.0f, ram = 0.0f;
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int b = 0; b < NB; b++) load_q<WT>(b_ptr[b], k0, b_half, rb[b]);
+        for (int b = 0; b < NB; b++) {
+            if constexpr (KS == 1) {
+                load_q<WT>(b_ptr[b], k0, b_half, rb[b][0]);
+            } else {
 #pragma unroll
-        for (int p = 0; p < MT; p++) ra[p] = a_src[p] ? *(const uint4 *)(a_src[p] + k0) : make_uint4(0, 0, 0, 0);
+                for (int hf = 0; hf < NRAW; hf++) load_q<WT>(b_ptr[b], k0 + kBK * b_half, hf, rb[b][hf]);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < A_PASSES; p++) ra[p] = a_src[p] ? *(const uint4 *)(a_src[p] + k0) : make_uint4(0, 0, 0, 0);
         ras = as_ptr ? as_ptr[k0 >> 6] : 0.0f;
         if (OFFSET) ram = am_ptr ? am_ptr[k0 >> 5] : 0.0f;
     };
@@ -487,47 +504,54 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 
     const int col = 32 * wave + (lane & 31), g = lane >> 5;
     MUMMU_TIMER_DECL;
-    for (int k0 = 0; k0 < in_dim; k0 += kBK) {
+    for (int k0 = 0; k0 < in_dim; k0 += KS * kBK) {
         MUMMU_TIMER_MARK(0);
         // registers -> LDS
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            uint32_t q[8];
-            float sc, sc1, nm;
-            expand_q<WT>(rb[b], k0, b_half, q, sc, sc1, nm);
-            uint4 *dst = (uint4 *)(s_b(b, b_row) + b_half * 32);
-            dst[0] = make_uint4(q[0], q[1], q[2], q[3]);
-            dst[1] = make_uint4(q[4], q[5], q[6], q[7]);
-            if (SUB16) {
-                s_bd[b][b_row][(2 * b_half) % NSC] = sc;
-                s_bd[b][b_row][(2 * b_half + 1) % NSC] = sc1;
-            } else {
-                s_bd[b][b_row][b_half] = sc;
+#pragma unroll
+            for (int hh = 0; hh < NBLK; hh++) {
+                // the block this pass stages: block `blk` (0 .. 2 KS - 1) of the stage
+                const int half = KS == 1 ? b_half : hh, blk = KS == 1 ? b_half : 2 * b_half + hh;
+                uint32_t q[8];
+                float sc, sc1, nm;
+                expand_q<WT>(rb[b][NRAW == 2 ? hh : 0], k0 + (KS == 1 ? 0 : kBK * b_half), half, q, sc, sc1, nm);
+                uint4 *dst = (uint4 *)(s_b(b, b_row) + blk * 32);
+                dst[0] = make_uint4(q[0], q[1], q[2], q[3]);
+                dst[1] = make_uint4(q[4], q[5], q[6], q[7]);
+                if (SUB16) {
+                    s_bd[b][b_row][2 * blk] = sc;
+                    s_bd[b][b_row][2 * blk + 1] = sc1;
+                } else {
+                    s_bd[b][b_row][blk] = sc;
+                }
+                if (OFFSET) s_bm[b][b_row][blk] = nm;
             }
-            if (OFFSET) s_bm[b][b_row][b_half] = nm;
         }
 #pragma unroll
-        for (int p = 0; p < MT; p++) *(uint4 *)(s_a(a_plane, a_row[p]) + a_chunk * 16) = ra[p];
-        if (tid < BM) s_as[tid] = ras;
-        if (OFFSET && tid < 2 * BM) s_am[tid >> 1][tid & 1] = ram;
+        for (int p = 0; p < A_PASSES; p++) *(uint4 *)(s_a(a_plane, a_row[p]) + a_chunk * 16) = ra[p];
+        if (tid < KS * BM) s_as[tid / BM][tid % BM] = ras;
+        if (OFFSET && tid < 2 * KS * BM) s_am[tid / (2 * KS)][tid & (2 * KS - 1)] = ram;
         MUMMU_TIMER_MARK(1);
         __syncthreads();
         MUMMU_TIMER_MARK(2);
-        if (k0 + kBK < in_dim) fetch(k0 + kBK);
+        if (k0 + KS * kBK < in_dim) fetch(k0 + KS * kBK);
         MUMMU_TIMER_MARK(3);
 
         // multiply: wave owns columns 32*wave .. +31
+#pragma unroll
+        for (int sub = 0; sub < KS; sub++) {
         if constexpr (!SUB16) {
 #pragma unroll
             for (int b = 0; b < NB; b++) {
-                const int4v bq0 = *(const int4v *)(s_b(b, col) + 16 * g);
-                const int4v bq1 = *(const int4v *)(s_b(b, col) + 32 + 16 * g);
-                const float d0 = s_bd[b][col][0], d1 = s_bd[b][col][1];
+                const int4v bq0 = *(const int4v *)(s_b(b, col) + 64 * sub + 16 * g);
+                const int4v bq1 = *(const int4v *)(s_b(b, col) + 64 * sub + 32 + 16 * g);
+                const float d0 = s_bd[b][col][2 * sub], d1 = s_bd[b][col][2 * sub + 1];
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     const int arow = 32 * m + (lane & 31);
-                    const int4v ah0 = *(const int4v *)(s_a(0, arow) + 16 * g), al0 = *(const int4v *)(s_a(1, arow) + 16 * g);
-                    const int4v ah1 = *(const int4v *)(s_a(0, arow) + 32 + 16 * g), al1 = *(const int4v *)(s_a(1, arow) + 32 + 16 * g);
+                    const int4v ah0 = *(const int4v *)(s_a(0, arow) + 64 * sub + 16 * g), al0 = *(const int4v *)(s_a(1, arow) + 64 * sub + 16 * g);
+                    const int4v ah1 = *(const int4v *)(s_a(0, arow) + 64 * sub + 32 + 16 * g), al1 = *(const int4v *)(s_a(1, arow) + 64 * sub + 32 + 16 * g);
                     const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                     const int16v ch0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah0, bq0, zero, 0, 0, 0);
                     const int16v cl0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(al0, bq0, zero, 0, 0, 0);
@@ -538,7 +562,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                         // accumulator rows 8j..8j+7 of this 32-row block: past the tile's rows there is
                         // nothing to scale (ragged experts leave most of a tile empty at small batches)
                         if (GATE_UP && 32 * m + 8 * j >= rows) continue;  // (the down kernel measures faster without the test)
-                        const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
+                        const float4 s4 = *(const float4 *)&s_as[sub][32 * m + 8 * j + 4 * g];
                         const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
@@ -550,7 +574,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                         }
                     }
                     if (OFFSET)
-                        acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][g], s_bm[b][col][g], acc[b][m], 0, 0, 0);
+                        acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][2 * sub + g], s_bm[b][col][2 * sub + g], acc[b][m], 0, 0, 0);
                 }
             }
         } else {
@@ -561,8 +585,8 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                 float dj[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    bq[j] = *(const long *)(s_b(b, col) + 16 * j + 8 * g);
-                    dj[j] = s_bd[b][col][j];
+                    bq[j] = *(const long *)(s_b(b, col) + 64 * sub + 16 * j + 8 * g);
+                    dj[j] = s_bd[b][col][4 * sub + j];
                 }
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
@@ -570,7 +594,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                     float t[16] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const long ah = *(const long *)(s_a(0, arow) + 16 * j + 8 * g), al = *(const long *)(s_a(1, arow) + 16 * j + 8 * g);
+                        const long ah = *(const long *)(s_a(0, arow) + 64 * sub + 16 * j + 8 * g), al = *(const long *)(s_a(1, arow) + 64 * sub + 16 * j + 8 * g);
                         const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                         const int16v ch = __builtin_amdgcn_mfma_i32_32x32x16_i8(ah, bq[j], zero, 0, 0, 0);
                         const int16v cl = __builtin_amdgcn_mfma_i32_32x32x16_i8(al, bq[j], zero, 0, 0, 0);
@@ -583,7 +607,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                     }
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const float4 s4 = *(const float4 *)&s_as[32 * m + 8 * j + 4 * g];
+                        const float4 s4 = *(const float4 *)&s_as[sub][32 * m + 8 * j + 4 * g];
                         const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
                         if (!GATE_UP || 32 * m + 8 * j < rows) {
 #pragma unroll
@@ -592,6 +616,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                     }
                 }
             }
+        }
         }
         MUMMU_TIMER_MARK(4);
         __syncthreads();
@@ -678,12 +703,17 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
                                 const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
                                 int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
     dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
-    if (tile_rows == 64)
-        launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, 2>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
-                                                                     out_dim, act_out, y_out);
-    else
-        launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, 1>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
-                                                                     out_dim, act_out, y_out);
+    // two K steps per stage where the launch streams its weights with few rows per expert (small
+    // tiles) and the row length allows
+    const bool ks2 = in_dim % (2 * kBK) == 0;
+#define MUMMU_Q(MT, KS)                                                                                                   \
+    launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, MT, KS>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, \
+                  in_dim, out_dim, act_out, y_out)
+    if (tile_rows == 64 && ks2) MUMMU_Q(2, 2);
+    else if (tile_rows == 64) MUMMU_Q(2, 1);
+    else if (ks2) MUMMU_Q(1, 2);
+    else MUMMU_Q(1, 1);
+#undef MUMMU_Q
     return hipGetLastError();
 }
 
