@@ -115,6 +115,13 @@ MUMMU_API int mummu_moe_load_shared_expert(mummu_moe *h, int layer, int inter, c
                                            int up_type, const void *down, int down_type, const void *gate_vec,
                                            int gate_vec_type);
 
+/* The smallest token count at which a call on this layer sorts the assignments by expert and runs
+ * one grouped GEMM per projection (the reference's per-expert batched form, nn/moe.rs:275-316)
+ * instead of the per-token decode kernels; INT32_MAX when the layer's banks never do (or the layer is
+ * not loaded).  Below it a token's result does not depend on the tokens sharing the call.  The
+ * environment variable MUMMU_GEMM_MIN_TOKENS overrides the built-in crossover. */
+MUMMU_API int mummu_moe_batched_from(const mummu_moe *h, int layer);
+
 /* Bytes resident on the device for weights (ExpertExec::resident_bytes, nn/moe.rs:352). */
 MUMMU_API uint64_t mummu_moe_resident_bytes(const mummu_moe *h);
 

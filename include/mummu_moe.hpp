@@ -348,6 +348,8 @@ class SparseMoe {
     }
 
     uint64_t resident_bytes() const { return mummu_moe_resident_bytes(h_.get()); }
+    /// Smallest token count that takes dispatch + grouped GEMM on this layer (INT32_MAX: never).
+    int batched_from(int layer = 0) const { return mummu_moe_batched_from(h_.get(), layer); }
 
     // SparseMoe::forward (nn/moe.rs:116): x [tokens, hidden] -> [tokens, hidden].
     std::vector<float> forward(const std::vector<float> &x, int top_k, bool norm_topk_prob, int layer = 0) {

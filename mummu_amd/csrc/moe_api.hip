@@ -74,7 +74,9 @@ struct mummu_moe {
     int32_t *offsets = nullptr, *sorted = nullptr, *inv = nullptr, *tiles = nullptr, *n_tiles = nullptr, *disp_scratch = nullptr;
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
-    int gemm_min_tokens = 32;    // batches at least this large take the grouped GEMM
+    // batches at least this large take dispatch + grouped GEMM (measured crossovers on the OLMoE shape:
+    // the float decode kernels lose from 4 tokens on, the integer ones from 19)
+    int gemm_min_f16 = 4, gemm_min_quant = 19;
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
@@ -289,11 +291,18 @@ int check_topk(mummu_moe *h, int top_k, int n_experts) {
 
 // experts of an already-made routing: gate/up -> down -> combine.  x_quantized says h->xq
 // already holds the 16-bit form of x (the fused router produced it).
+// Smallest batch of this layer that takes the batched path (INT_MAX: never).
+int batched_from(const mummu_moe *h, const Layer &L) {
+    const ExpertBanks b = banks_of(h, L);
+    if (!grouped_gemm_supported(b)) return 0x7fffffff;
+    return grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16;
+}
+
 int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, int64_t n, int k, const float *residual,
                 float *out, hipStream_t s, bool count_hits = false) {
     ExpertBanks b = banks_of(h, L);
     const int na = (int)(n * k);
-    if (n >= h->gemm_min_tokens && grouped_gemm_supported(b)) {
+    if (n >= batched_from(h, L)) {
         // batched: sort the assignments by expert, then one grouped GEMM per projection
         const int tile_rows = grouped_gemm_tile_rows(b, na, b.n_experts);
         // the 16-bit activation buffers, viewed in the batched path's 64-element-block layout
@@ -327,7 +336,7 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
 bool decode_three_launches(const mummu_moe *h, const Layer &L, int64_t n, int k) {
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     const ExpertBanks b = banks_of(h, L);
-    const bool batched = n >= h->gemm_min_tokens && grouped_gemm_supported(b);
+    const bool batched = n >= batched_from(h, L);
     const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0 && !batched;
     return !(n > 8 && router_fused_supported(E)) && want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k);
 }
@@ -339,7 +348,7 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
-    const bool batched = n >= h->gemm_min_tokens && grouped_gemm_supported(banks_of(h, L));
+    const bool batched = n >= batched_from(h, L);
     const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0 && !batched;
     const QAct xq = want_xq ? h->xq : QAct();
     if (norm_gamma && !decode_three_launches(h, L, n, k)) return fail(h, MUMMU_ERR_ARG, "fused RmsNorm outside the decode form");
@@ -478,6 +487,11 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
 
     mummu_moe *h = new mummu_moe();
     h->cfg = *cfg;
+    // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
+    if (const char *e = getenv("MUMMU_GEMM_MIN_TOKENS")) {
+        const int v = atoi(e);
+        if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = v;
+    }
     h->layers.resize((size_t)cfg->num_layers);
     auto bail = [&](int rc) {
         g_error = h->err;
@@ -627,6 +641,11 @@ int mummu_moe_load_shared_expert(mummu_moe *h, int layer, int inter, const void 
         h->sh_ws_tokens = 0;  // regrow for the wider expert
     }
     return ensure_shared_ws(h);
+}
+
+int mummu_moe_batched_from(const mummu_moe *h, int layer) {
+    if (!h || layer < 0 || layer >= (int)h->layers.size() || !h->layers[layer].loaded) return 0x7fffffff;
+    return batched_from(h, h->layers[layer]);
 }
 
 uint64_t mummu_moe_resident_bytes(const mummu_moe *h) {

@@ -164,6 +164,10 @@ class SparseMoe:
     def resident_bytes(self) -> int:
         return int(self._lib.mummu_moe_resident_bytes(self._h))
 
+    def batched_from(self, layer: int = 0) -> int:
+        """Smallest token count that takes dispatch + grouped GEMM on this layer (2**31 - 1: never)."""
+        return int(self._lib.mummu_moe_batched_from(self._h, layer))
+
     # -- the block -------------------------------------------------------------------------
     def _rows(self, x) -> Tuple[np.ndarray, tuple]:
         x = _f32(x)

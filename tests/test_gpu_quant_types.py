@@ -71,6 +71,7 @@ def test_mixed_type_banks_match_the_oracle(gt, dt, H, I, E, k):
     with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=n) as m:
         m.load_layer(0, router, M.F16, gate, gt, up, gt, down, dt)
         outs = {c: m.forward(x[:c], k, True) for c in (1, 5, n)}
+        batched_from = m.batched_from(0)
         ids, w = m.last_routing(n, k)
         hits_before = m.take_hits()
         e0 = int(ids[0, 0])
@@ -86,9 +87,11 @@ def test_mixed_type_banks_match_the_oracle(gt, dt, H, I, E, k):
     for c, got in outs.items():
         err = orc.rel_err(got, want[:c], mag[:c])
         assert err.max() <= 2e-3, f"{c} tokens: max relative error {err.max():.3e}"
-    # a token's result does not depend on how many tokens share the call
-    assert np.array_equal(outs[1].view(np.uint32), outs[n][:1].view(np.uint32))
-    assert np.array_equal(outs[5].view(np.uint32), outs[n][:5].view(np.uint32))
+    # below the batched path (the 21-token call takes it where the shape allows the grouped GEMM) a
+    # token's result does not depend on how many tokens share the call
+    assert np.array_equal(outs[1].view(np.uint32), outs[5][:1].view(np.uint32))
+    if n < batched_from:
+        assert np.array_equal(outs[5].view(np.uint32), outs[n][:5].view(np.uint32))
     # one expert alone (ExpertExec::run) is a top-1 routing to it with weight 1: same closeness
     want1, mag1 = orc.moe_ref_f64(banks, np.full((3, 1), e0, np.uint32), np.ones((3, 1), np.float32), x[:3])
     assert orc.rel_err(one, want1, mag1).max() <= 2e-3

@@ -67,6 +67,7 @@ def test_shared_expert_and_sigmoid_gate_match_the_composition(gt, dt, sgt, sdt, 
         m.load_shared_expert(0, IS, sgate, sgt, sup, sgt, sdown, sdt, gate_vec)
         assert m.resident_bytes() > before
         outs = {c: m.forward(x[:c], k, norm) for c in (1, 5, n)}
+        batched_from = m.batched_from(0)
         r = m.route(x[:5], k, norm)
         local = m.run_local(x[:5], r)   # routed experts only, as in the reference
     banks = orc.LayerBanks(H, I, E, gate, up, down, gt, gt, dt)
@@ -75,8 +76,8 @@ def test_shared_expert_and_sigmoid_gate_match_the_composition(gt, dt, sgt, sdt, 
     tol = 1e-5 if gt == M.F32 else 2e-3
     for c, got in outs.items():
         assert orc.rel_err(got, full[:c], mag[:c]).max() <= tol, c
-    assert np.array_equal(outs[1].view(np.uint32), outs[n][:1].view(np.uint32)) or n >= 32  # same kernels below the batched path
-    assert np.array_equal(outs[1].view(np.uint32), outs[5][:1].view(np.uint32))
+    assert n >= batched_from or np.array_equal(outs[1].view(np.uint32), outs[n][:1].view(np.uint32))  # same kernels below the batched path
+    assert 5 >= batched_from or np.array_equal(outs[1].view(np.uint32), outs[5][:1].view(np.uint32))
     assert np.array_equal(local.view(np.uint32), routed5.view(np.uint32))
     assert orc.rel_err(local, routed[:5], mag[:5]).max() <= tol
     # the shared expert really contributes
