@@ -208,14 +208,26 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_f_kernel(
     const float *xrow = x + (size_t)t * (size_t)hidden;
     float *arow = act + (size_t)a * (size_t)inter;
     const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
-    for (int r = 0; r < rows_per_wave; r++) {
-        const int row = row0 + r;
-        if (row >= inter) break;
-        float pg = row_partial_f<WT, VEC>(ge + (size_t)row * row_bytes, xrow, hidden, lane);
-        float pu = row_partial_f<WT, VEC>(ue + (size_t)row * row_bytes, xrow, hidden, lane);
-        pg = wave_sum(pg);
-        pu = wave_sum(pu);
-        if (lane == 0) arow[row] = __fmul_rn(det_silu(pg), pu);
+    // four rows of either matrix at a time (rows_per_wave is a multiple of 4): eight loads in flight per
+    // iteration; rows past the bank's end stand in for its last row and are not stored
+    for (int r = 0; r < rows_per_wave; r += 4) {
+        if (row0 + r >= inter) break;
+        const uint8_t *rowp[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int row = row0 + r + j < inter ? row0 + r + j : inter - 1;
+            rowp[j] = ge + (size_t)row * row_bytes;
+            rowp[4 + j] = ue + (size_t)row * row_bytes;
+        }
+        float p[8];
+        rows_partial_f<WT, VEC, 8>(rowp, xrow, hidden, lane, p);
+#pragma unroll
+        for (int j = 0; j < 8; j++) p[j] = wave_sum(p[j]);
+        if (lane < 4 && row0 + r + lane < inter) {
+            const float pg = lane == 0 ? p[0] : (lane == 1 ? p[1] : (lane == 2 ? p[2] : p[3]));
+            const float pu = lane == 0 ? p[4] : (lane == 1 ? p[5] : (lane == 2 ? p[6] : p[7]));
+            arow[row0 + r + lane] = __fmul_rn(det_silu(pg), pu);
+        }
     }
 }
 
@@ -299,12 +311,26 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_f_kernel(const uint8_t *
     const float *arow = act + (size_t)a * (size_t)inter;
     float *yrow = y + (size_t)a * (size_t)hidden;
     const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
-    for (int r = 0; r < rows_per_wave; r++) {
-        const int row = row0 + r;
-        if (row >= hidden) break;
-        float p = row_partial_f<WT, VEC>(de + (size_t)row * row_bytes, arow, inter, lane);
-        p = wave_sum(p);
-        if (lane == 0) yrow[row] = p;
+    // eight rows at a time (rows_per_wave is a multiple of 4; an odd group of four runs half empty)
+    for (int r = 0; r < rows_per_wave; r += 8) {
+        if (row0 + r >= hidden) break;
+        const int live = rows_per_wave - r < 8 ? rows_per_wave - r : 8;
+        const uint8_t *rowp[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int row = (j < live && row0 + r + j < hidden) ? row0 + r + j : (row0 + r < hidden ? row0 + r : hidden - 1);
+            rowp[j] = de + (size_t)row * row_bytes;
+        }
+        float p[8];
+        rows_partial_f<WT, VEC, 8>(rowp, arow, inter, lane, p);
+#pragma unroll
+        for (int j = 0; j < 8; j++) p[j] = wave_sum(p[j]);
+        if (lane < live && row0 + r + lane < hidden) {
+            float v = p[0];
+#pragma unroll
+            for (int j = 1; j < 8; j++) v = lane == j ? p[j] : v;
+            yrow[row0 + r + lane] = v;
+        }
     }
 }
 
@@ -453,7 +479,11 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         const int rpw = pick_rows_per_wave(b.inter, n_assign);
         dim3 block(64 * kGemvWaves), grid(slots, (b.inter + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_assign / slots);
         const bool vec = b.hidden % 4 == 0 && (((uintptr_t)x & 15) == 0);
-        if (vec)
+        constexpr int WIDE = WT == T_F32 ? 4 : 8;  // 16 bytes of a weight row per lane and load
+        if (vec && b.hidden % WIDE == 0 && ((((uintptr_t)b.gate | (uintptr_t)b.up) & 15) == 0))
+            launch_kernel(gate_up_f_kernel<WT, WIDE>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
+                                                           b.n_experts, rpw, act, flags);
+        else if (vec)
             launch_kernel(gate_up_f_kernel<WT, 4>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
                                                            b.n_experts, rpw, act, flags);
         else
@@ -543,7 +573,10 @@ static hipError_t launch_down_t(const ExpertBanks &b, const float *act, QAct act
     } else {
         const int rpw = pick_rows_per_wave(b.hidden, n_assign);
         dim3 grid(slots, (b.hidden + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_assign / slots);
-        if (b.inter % 4 == 0)
+        constexpr int WIDE = WT == T_F32 ? 4 : 8;
+        if (b.inter % WIDE == 0 && (((uintptr_t)b.down & 15) == 0))
+            launch_kernel(down_f_kernel<WT, WIDE>, grid, block, 0, s, b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
+        else if (b.inter % 4 == 0)
             launch_kernel(down_f_kernel<WT, 4>, grid, block, 0, s, b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);
         else
             launch_kernel(down_f_kernel<WT, 1>, grid, block, 0, s, b.down, act, ids, fixed_expert, b.hidden, b.inter, b.n_experts, rpw, y);

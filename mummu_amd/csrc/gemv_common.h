@@ -363,6 +363,61 @@ __device__ inline float row_partial_f(const uint8_t *__restrict__ rowp, const fl
     return acc;
 }
 
+// The same for NR rows at once against one activation row: the loads of all rows of an iteration
+// go out together and every row has its own accumulator chain (a single row at a time leaves a
+// wave waiting on one load and one chain of dependent fmas).  VEC = 8 only for the 16-bit types.
+template <int WT, int VEC, int NR>
+__device__ inline void rows_partial_f(const uint8_t *const (&rowp)[NR], const float *__restrict__ xrow, int in_dim, int lane,
+                                      float (&acc)[NR]) {
+    static_assert(VEC == 1 || VEC == 4 || (VEC == 8 && WT != T_F32), "vector widths: 1, 4, or 8 halfs");
+#pragma unroll
+    for (int r = 0; r < NR; r++) acc[r] = 0.0f;
+    for (int i = lane * VEC; i < in_dim; i += 64 * VEC) {
+        float xv[VEC];
+        if constexpr (VEC == 1) {
+            xv[0] = xrow[i];
+        } else {
+#pragma unroll
+            for (int q = 0; q < VEC / 4; q++) {
+                const float4 v = *(const float4 *)(xrow + i + 4 * q);
+                xv[4 * q] = v.x; xv[4 * q + 1] = v.y; xv[4 * q + 2] = v.z; xv[4 * q + 3] = v.w;
+            }
+        }
+        float w[NR][VEC];
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            if constexpr (WT == T_F32) {
+                if constexpr (VEC == 4) {
+                    const float4 v = *(const float4 *)(rowp[r] + (size_t)i * 4);
+                    w[r][0] = v.x; w[r][1] = v.y; w[r][2] = v.z; w[r][3] = v.w;
+                } else {
+                    w[r][0] = *(const float *)(rowp[r] + (size_t)i * 4);
+                }
+            } else {
+                uint32_t raw[VEC >= 2 ? VEC / 2 : 1];
+                if constexpr (VEC == 8) {
+                    const uint4 v = *(const uint4 *)(rowp[r] + (size_t)i * 2);
+                    raw[0] = v.x; raw[1] = v.y; raw[2] = v.z; raw[3] = v.w;
+                } else if constexpr (VEC == 4) {
+                    const uint2 v = *(const uint2 *)(rowp[r] + (size_t)i * 2);
+                    raw[0] = v.x; raw[1] = v.y;
+                } else {
+                    raw[0] = *(const uint16_t *)(rowp[r] + (size_t)i * 2);
+                }
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    const uint16_t h = (uint16_t)((raw[j / 2] >> (16 * (j & 1))) & 0xFFFFu);
+                    w[r][j] = WT == T_F16 ? half_bits_to_float(h) : bf16_bits_to_float(h);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < NR; r++)
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[r] = __builtin_fmaf(w[r][j], xv[j], acc[r]);
+    }
+}
+
 __host__ __device__ inline size_t type_row_bytes(int type, int in_dim) {
     return (size_t)(in_dim / block_elems(type)) * (size_t)block_bytes(type);
 }
