@@ -700,12 +700,16 @@ int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts) {
 
 template <int WT, bool GATE_UP>
 static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_in, const int32_t *sorted, int k_slots,
-                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
-                                int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
+                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, bool few_rows,
+                                int in_dim, int out_dim, QAct64 act_out, float *y_out, hipStream_t s) {
     dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
-    // two K steps per stage where the launch streams its weights with few rows per expert (small
-    // tiles) and the row length allows
-    const bool ks2 = in_dim % (2 * kBK) == 0;
+    // Two K steps per stage where the row length allows and it measured faster: always for the types
+    // whose one load holds both blocks of a step (Q4_K, Q5_K: no extra registers) and for gate/up;
+    // the down product of the other types only while an expert's rows fit one tile (with several
+    // tiles per expert its second set of raw registers costs more than the barriers saved: Q8_0 at
+    // 4096 tokens 410 -> 462 us); never for Q6_K (slower, and it spills).
+    constexpr bool shared_raw = WT == T_Q4_K || WT == T_Q5_K;
+    const bool ks2 = in_dim % (2 * kBK) == 0 && !gemm_sub16(WT) && (shared_raw || GATE_UP || few_rows);
 #define MUMMU_Q(MT, KS)                                                                                                   \
     launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, MT, KS>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, \
                   in_dim, out_dim, act_out, y_out)
@@ -747,7 +751,7 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     switch (b.gate_type) {
 #define MUMMU_GU(T)                                                                                                          \
     case T:                                                                                                                  \
-        return launch_gemm_q<T, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden, b.inter, \
+        return launch_gemm_q<T, true>(b.gate, b.up, xq, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, true, b.hidden, b.inter, \
                                       actq, nullptr, s)
         MUMMU_GU(T_Q8_0);
         MUMMU_GU(T_Q4_K);
@@ -762,16 +766,17 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     }
 }
 
-hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, const int32_t *tiles,
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, int n_assign, const int32_t *tiles,
                             const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    const bool few_rows = n_assign <= 64 * b.n_experts;  // an expert's rows fit one tile, on average
     if (b.down_type == T_F16)
         return launch_gemm_f16<false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
                                       tile_rows, b.inter, b.hidden, nullptr, y, s);
     switch (b.down_type) {
 #define MUMMU_DN(T)                                                                                                      \
     case T:                                                                                                              \
-        return launch_gemm_q<T, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter, b.hidden, \
+        return launch_gemm_q<T, false>(b.down, nullptr, actq, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, few_rows, b.inter, b.hidden, \
                                        QAct64(), y, s)
         MUMMU_DN(T_Q8_0);
         MUMMU_DN(T_Q4_K);

@@ -113,7 +113,7 @@ hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStr
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
                                QAct64 actq, hipStream_t s);
-hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, const int32_t *tiles,
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, int n_assign, const int32_t *tiles,
                             const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s);
 
 }  // namespace mummu

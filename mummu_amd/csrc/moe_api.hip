@@ -75,8 +75,8 @@ struct mummu_moe {
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
     // batches at least this large take dispatch + grouped GEMM (measured crossovers on the OLMoE shape:
-    // the float decode kernels lose from 4 tokens on, the integer ones from 19)
-    int gemm_min_f16 = 4, gemm_min_quant = 19;
+    // the float decode kernels lose from 6 tokens on, the integer ones from 19)
+    int gemm_min_f16 = 6, gemm_min_quant = 19;
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
@@ -315,7 +315,7 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         LAUNCH(h, K_GEMM_GATE_UP, s,
                launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, actq64, s));
         LAUNCH(h, K_GEMM_DOWN, s,
-               launch_gemm_down(b, h->act16, actq64, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
+               launch_gemm_down(b, h->act16, actq64, na, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
         LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, h->inv, (int)n, k, b.hidden, residual, out, s));
         return MUMMU_OK;
     }
