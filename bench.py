@@ -44,6 +44,7 @@ WORKLOADS = {
     "olmoe_q4k_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q4_K", router="F16"),
     "olmoe_q8_0_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q8_0", router="F16"),
     "olmoe_f16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F16", router="F16"),
+    "olmoe_bf16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="BF16", router="F16"),
     "olmoe_f32_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F32", router="F16"),
     "qwen3_a3b_q4k": dict(hidden=2048, inter=768, experts=128, top_k=8, norm=True, bank="Q4_K", router="F16"),
     # mixed bank types: llama.cpp's Q4_K_M recipe stores part of ffn_down as Q6_K; the shipped qwen4exp file has
@@ -52,7 +53,7 @@ WORKLOADS = {
     "qwen4exp_decode": dict(hidden=2560, inter=640, experts=512, top_k=10, norm=True, bank="Q4_K", down="Q5_1", router="F16",
                             flavour=1),
 }
-BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "F32": 0, "Q6_K": 14, "Q5_1": 7, "Q5_K": 13}
+BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "F32": 0, "Q6_K": 14, "Q5_1": 7, "Q5_K": 13, "BF16": 30}
 
 
 def main() -> int:
@@ -97,10 +98,12 @@ def main() -> int:
 
     def make_bank(in_dim, out_dim, seed, t=None):
         t = bank_t if t is None else t
-        if t not in (M.F16, M.F32):
+        if t not in (M.F16, M.F32, M.BF16):
             return synth.random_bank_fast(t, [in_dim, out_dim, E], seed)
         gg = np.random.Generator(np.random.PCG64(seed))
         w32 = gg.standard_normal(E * out_dim * in_dim, dtype=np.float32) * np.float32(0.02)
+        if t == M.BF16:
+            return (w32.view(np.uint32) >> np.uint32(16)).astype(np.uint16).view(np.uint8)  # (truncated: statistics only)
         return (w32 if t == M.F32 else w32.astype(np.float16)).view(np.uint8)
 
     t_setup = time.time()
@@ -215,10 +218,10 @@ def main() -> int:
     # batched calls: matrix-core rate of the two grouped GEMMs (2*H*I flops per assignment and projection)
     mfma = None
     if per_kernel_us.get("gemm_gate_up") and per_kernel_us.get("gemm_down"):
-        peak = 2500.0 if w["bank"] in ("F16", "F32") else 5000.0  # dense f16 TFLOP/s, int8 TOP/s
+        peak = 2500.0 if w["bank"] in ("F16", "F32", "BF16") else 5000.0  # dense f16 TFLOP/s, int8 TOP/s
         gu_t = n * k * 2 * 2 * H * I / (per_kernel_us["gemm_gate_up"] * 1e-6) / 1e12
         dn_t = n * k * 2 * H * I / (per_kernel_us["gemm_down"] * 1e-6) / 1e12
-        mfma = {"unit": "TFLOP/s" if w["bank"] == "F16" else "TOP/s", "peak": peak, "gemm_gate_up": round(gu_t, 1),
+        mfma = {"unit": "TFLOP/s" if w["bank"] in ("F16", "BF16") else "TOP/s", "peak": peak, "gemm_gate_up": round(gu_t, 1),
                 "gemm_down": round(dn_t, 1), "gemm_gate_up_frac": round(gu_t / peak, 4), "gemm_down_frac": round(dn_t / peak, 4),
                 "hbm_floor_us": round(layer_bytes / (HBM_PEAK_GBS * 1e3), 1)}
 
@@ -233,7 +236,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if w["bank"] in ("F16", "F32") else ("i8*i16->i32" if w["bank"] == "Q8_0" else "u4*i16->i32") +
+        "dtype": "f32" if w["bank"] in ("F16", "F32", "BF16") else ("i8*i16->i32" if w["bank"] == "Q8_0" else "u4*i16->i32") +
                  " (v_dot4_i32_i8), f32 scales",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "

@@ -78,7 +78,9 @@ __device__ inline bool xcd_tile(const int32_t *__restrict__ n_tiles, int slabs, 
 // GATE_UP: A = x (f32, gathered by token through `sorted`), two weight matrices, epilogue
 //          act16[pos, n] = f16(silu(g) * u).
 // else   : A = act16 (f16, rows already in sorted order), one matrix, y[pos, n] = f32 sum.
-template <bool GATE_UP, int MT>
+// BF16: the banks hold bf16; every weight becomes a half on its way into LDS (exact from 2^-14 up:
+// a bf16 has 8 significant bits; smaller weights keep an absolute error below 2^-25).
+template <bool GATE_UP, int MT, bool BF16>
 __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const float *__restrict__ x,
     const _Float16 *__restrict__ act_in, const int32_t *__restrict__ sorted, int k_slots,
@@ -171,7 +173,14 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
 #pragma unroll
         for (int b = 0; b < NB; b++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) *(u32x4 *)&s_b[b][(tid >> 3) + 32 * i][b_chunk * 8] = rb[b][i];
+            for (int i = 0; i < 4; i++) {
+                u32x4 v = rb[b][i];
+                if (BF16) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) v[q] = pack_half2(__uint_as_float(v[q] << 16), __uint_as_float(v[q] & 0xFFFF0000u));
+                }
+                *(u32x4 *)&s_b[b][(tid >> 3) + 32 * i][b_chunk * 8] = v;
+            }
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) {
             if (GATE_UP) {
@@ -680,7 +689,7 @@ bool grouped_gemm_quantized(const ExpertBanks &b) {
 }
 
 bool grouped_gemm_supported(const ExpertBanks &b) {
-    const bool f16 = b.gate_type == T_F16 && b.up_type == T_F16 && b.down_type == T_F16;
+    const bool f16 = (b.gate_type == T_F16 || b.gate_type == T_BF16) && b.up_type == b.gate_type && b.down_type == b.gate_type;
     return (f16 || grouped_gemm_quantized(b)) && b.hidden % kBK == 0 && b.inter % kBK == 0;
 }
 
@@ -721,14 +730,14 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
     return hipGetLastError();
 }
 
-template <bool GATE_UP>
+template <bool GATE_UP, bool BF16>
 static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const float *x, const _Float16 *act_in,
                                   const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
                                   int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
                                   hipStream_t s) {
     dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
 #define MUMMU_F16(MT)                                                                                                    \
-    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, \
+    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT, BF16>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, \
                   in_dim, out_dim, act_out, y_out)
     switch (tile_rows) {
     case 32: MUMMU_F16(1); break;
@@ -746,8 +755,11 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
                                QAct64 actq, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
     if (b.gate_type == T_F16)
-        return launch_gemm_f16<true>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
-                                     b.inter, (_Float16 *)act16, nullptr, s);
+        return launch_gemm_f16<true, false>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+                                            b.inter, (_Float16 *)act16, nullptr, s);
+    if (b.gate_type == T_BF16)
+        return launch_gemm_f16<true, true>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+                                           b.inter, (_Float16 *)act16, nullptr, s);
     switch (b.gate_type) {
 #define MUMMU_GU(T)                                                                                                          \
     case T:                                                                                                                  \
@@ -771,8 +783,11 @@ hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
     const bool few_rows = n_assign <= 64 * b.n_experts;  // an expert's rows fit one tile, on average
     if (b.down_type == T_F16)
-        return launch_gemm_f16<false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
-                                      tile_rows, b.inter, b.hidden, nullptr, y, s);
+        return launch_gemm_f16<false, false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+                                             tile_rows, b.inter, b.hidden, nullptr, y, s);
+    if (b.down_type == T_BF16)
+        return launch_gemm_f16<false, true>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+                                            tile_rows, b.inter, b.hidden, nullptr, y, s);
     switch (b.down_type) {
 #define MUMMU_DN(T)                                                                                                      \
     case T:                                                                                                              \

@@ -102,7 +102,7 @@ hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int 
 
 // gemm.hip ----------------------------------------------------------------------------
 // Grouped GEMMs over the dispatch-sorted assignments on the matrix cores (hidden and inter
-// multiples of 64): F16 banks on the f16 units (act16: f16 [A, inter] in sorted order), every
+// multiples of 64): F16 and BF16 banks on the f16 units (act16: f16 [A, inter] in sorted order), every
 // block-quantized type on the int8 units against 16-bit activations (xq: tokens x hidden, actq:
 // A x inter in sorted order; gate/up and down may differ in type).
 bool grouped_gemm_supported(const ExpertBanks &b);

@@ -19,9 +19,10 @@ def normal(shape, seed, std=1.0):
 
 
 def banks_for(kind, H, I, E, seed):
-    if kind == "F16":
-        mk = lambda i, o, s: synth.encode_float(normal(E * o * i, s, 0.05), synth.F16)
-        return mk(H, I, seed), mk(H, I, seed + 1), mk(I, H, seed + 2), M.F16, orc.F16
+    if kind in ("F16", "BF16"):
+        t, ot = (M.F16, orc.F16) if kind == "F16" else (M.BF16, orc.BF16)
+        mk = lambda i, o, s: synth.encode_float(normal(E * o * i, s, 0.05), t)
+        return mk(H, I, seed), mk(H, I, seed + 1), mk(I, H, seed + 2), t, ot
     t, ot = {"Q8_0": (M.Q8_0, orc.Q8_0), "Q4_K": (M.Q4_K, orc.Q4_K)}[kind]
     mk = lambda i, o, s: synth.random_bank_fast(t, [i, o, E], s)
     return mk(H, I, seed), mk(H, I, seed + 1), mk(I, H, seed + 2), t, ot
@@ -34,6 +35,8 @@ CASES = [
     ("F16", 512, 256, 8, 2, 200),     # 50 per expert -> 96-row tiles
     ("F16", 512, 256, 8, 4, 130),     # 65 per expert -> 96/128-row tiles
     ("F16", 1024, 512, 16, 4, 1027),  # 257 per expert -> several 64-row tiles, 5 dispatch chunks, odd token count
+    ("BF16", 512, 256, 8, 2, 130),    # bf16 weights become halfs on the way into LDS
+    ("BF16", 1024, 512, 16, 4, 515),
     ("Q8_0", 512, 256, 8, 2, 77),
     ("Q8_0", 1024, 512, 16, 4, 515),
     ("Q4_K", 512, 256, 8, 2, 200),

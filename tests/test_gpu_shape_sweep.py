@@ -74,7 +74,9 @@ def test_awkward_shapes_match_the_oracle_on_every_path(gt, dt, H, I, E, k, flavo
         assert np.array_equal(ids, oids[:n].astype(np.int32)), n
         assert np.array_equal(w.view(np.uint32), ow[:n].view(np.uint32)), n
         err = orc.rel_err(outs[n], want[:n], mag[:n]).max()
-        assert err <= tol, f"{n} tokens: max relative error {err:.3e}"
+        # (the batched path rounds the activations of BF16 banks to f16, as it does for F16 banks)
+        tol_n = 2e-3 if n >= batched_from and M.BF16 in (gt, dt) else tol
+        assert err <= tol_n, f"{n} tokens: max relative error {err:.3e}"
         served += np.bincount(oids[:n].reshape(-1), minlength=E)
     assert hits.tolist() == served.tolist()
     # below the batched path a token's result does not depend on its company
