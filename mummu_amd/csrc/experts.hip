@@ -188,16 +188,38 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     MUMMU_PHASE(5);
 }
 
-// gate/up, float banks.
-template <int WT, int VEC>
+// gate/up, float banks.  RJN > 0: the kernel routes by itself (see RouteInline), RJN experts per lane
+// of the routing wave.
+template <int WT, int VEC, int RJN = 0>
 __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_f_kernel(
     const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, const float *__restrict__ x,
     const int32_t *__restrict__ ids, int k, int fixed_expert, int hidden, int inter, int n_experts,
-    int rows_per_wave, float *__restrict__ act, int32_t *__restrict__ flags) {
+    int rows_per_wave, float *__restrict__ act, int32_t *__restrict__ flags, RouteInline route) {
+    constexpr bool ROUTE = RJN > 0;
+    constexpr int JN = ROUTE ? RJN : 1;
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> s_route;
+    __shared__ int s_ids[64];
+    __shared__ float s_w[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.z;  // grid = (slot, row tile, token)
     const int a = t * gridDim.x + blockIdx.x;
-    const int e = fixed_expert >= 0 ? fixed_expert : ids[a];
+    if (ROUTE) {
+        if (wave == 0) {
+            float l[JN];
+#pragma unroll
+            for (int j = 0; j < JN; j++) l[j] = lane + 64 * j < n_experts ? route.logits[(size_t)t * n_experts + lane + 64 * j] : 0.0f;
+            route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
+            wave_lds_sync();
+            if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
+                const int id = s_ids[lane];
+                route.ids[(size_t)t * k + lane] = id;
+                route.weights[(size_t)t * k + lane] = s_w[lane];
+                if (route.hits) atomicAdd(&route.hits[id], 1ULL);
+            }
+        }
+        __syncthreads();
+    }
+    const int e = ROUTE ? s_ids[blockIdx.x] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
     if ((unsigned)e >= (unsigned)n_experts) {
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
@@ -482,13 +504,13 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         constexpr int WIDE = WT == T_F32 ? 4 : 8;  // 16 bytes of a weight row per lane and load
         if (vec && b.hidden % WIDE == 0 && ((((uintptr_t)b.gate | (uintptr_t)b.up) & 15) == 0))
             launch_kernel(gate_up_f_kernel<WT, WIDE>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
-                                                           b.n_experts, rpw, act, flags);
+                                                           b.n_experts, rpw, act, flags, RouteInline());
         else if (vec)
             launch_kernel(gate_up_f_kernel<WT, 4>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
-                                                           b.n_experts, rpw, act, flags);
+                                                           b.n_experts, rpw, act, flags, RouteInline());
         else
             launch_kernel(gate_up_f_kernel<WT, 1>, grid, block, 0, s, b.gate, b.up, x, ids, k, fixed_expert, b.hidden, b.inter,
-                                                           b.n_experts, rpw, act, flags);
+                                                           b.n_experts, rpw, act, flags, RouteInline());
         if (actq_out) {  // float gate/up feeding a quantized down bank: quantize the f32 act rows
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) return e;
@@ -505,6 +527,129 @@ hipError_t launch_gate_up(const ExpertBanks &b, const float *x, QAct xq, const i
     if (n_assign / (fixed_expert >= 0 ? 1 : k) > 65535) return hipErrorInvalidValue;
     return with_bank_type(b.gate_type, [&](auto tag) {
         return launch_gate_up_t<decltype(tag)::value>(b, x, xq, ids, n_assign, k, fixed_expert, act, actq, flags, s);
+    });
+}
+
+// Float banks, few tokens: gate/up with the routing inside (one launch less), then down + combine
+// in one launch.
+bool float_decode_fused(const ExpertBanks &b, int k) {
+    auto fl = [](int t) { return t == T_F32 || t == T_F16 || t == T_BF16; };
+    return fl(b.gate_type) && b.gate_type == b.up_type && fl(b.down_type) && b.n_experts <= 512 && k >= 1 && k <= b.n_experts && k <= 16;
+}
+
+template <int WT>
+static hipError_t launch_gate_up_f_routed_t(const ExpertBanks &b, const float *x, const RouteInline &route, int n_tokens, int k,
+                                            float *act, int32_t *flags, hipStream_t s) {
+    const int rpw = pick_rows_per_wave(b.inter, n_tokens * k);
+    dim3 block(64 * kGemvWaves), grid(k, (b.inter + rpw * kGemvWaves - 1) / (rpw * kGemvWaves), n_tokens);
+    constexpr int WIDE = WT == T_F32 ? 4 : 8;
+    const bool vec = b.hidden % 4 == 0 && (((uintptr_t)x & 15) == 0);
+    const bool wide = vec && b.hidden % WIDE == 0 && ((((uintptr_t)b.gate | (uintptr_t)b.up) & 15) == 0);
+#define MUMMU_GUF(VEC, JN)                                                                                              \
+    launch_kernel(gate_up_f_kernel<WT, VEC, JN>, grid, block, 0, s, b.gate, b.up, x, (const int32_t *)nullptr, k, -1, b.hidden, \
+                  b.inter, b.n_experts, rpw, act, flags, route)
+#define MUMMU_GUF_JN(VEC)                                                                                               \
+    do {                                                                                                                \
+        if (b.n_experts <= 64) MUMMU_GUF(VEC, 1);                                                                       \
+        else if (b.n_experts <= 128) MUMMU_GUF(VEC, 2);                                                                 \
+        else MUMMU_GUF(VEC, 8);                                                                                         \
+    } while (0)
+    if (wide) MUMMU_GUF_JN(WIDE);
+    else if (vec) MUMMU_GUF_JN(4);
+    else MUMMU_GUF_JN(1);
+#undef MUMMU_GUF_JN
+#undef MUMMU_GUF
+    return hipGetLastError();
+}
+
+hipError_t launch_gate_up_f_routed(const ExpertBanks &b, const float *x, const RouteInline &route, int n_tokens, int k, float *act,
+                                   int32_t *flags, hipStream_t s) {
+    if (n_tokens <= 0) return hipSuccess;
+    if (!float_decode_fused(b, k) || n_tokens > 65535) return hipErrorInvalidValue;
+    return with_bank_type(b.gate_type, [&](auto tag) {
+        constexpr int WT = decltype(tag)::value;
+        if constexpr (!is_quant_type(WT)) return launch_gate_up_f_routed_t<WT>(b, x, route, n_tokens, k, act, flags, s);
+        else return hipErrorInvalidValue;
+    });
+}
+
+// down + combine, float down bank, top_k <= 16: blockIdx.x = token, blockIdx.y = tile of 8 output rows.
+// Wave w takes the token's slots w, w + 8; the row sums (the same sums, bit for bit, as down_f_kernel
+// makes) meet in LDS and eight lanes add them as combine_kernel does: ascending expert id, multiply
+// and add rounded separately.
+template <int WT, int VEC>
+__global__ __launch_bounds__(512) void down_combine_f_kernel(const uint8_t *__restrict__ down, const float *__restrict__ act,
+                                                             const int32_t *__restrict__ ids, const float *__restrict__ weights,
+                                                             int k, int hidden, int inter, int n_experts,
+                                                             const float *__restrict__ residual, float *__restrict__ out) {
+    __shared__ float s_y[16][8];
+    __shared__ int s_order[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.x, row0 = blockIdx.y * 8;
+    if (tid < k) {
+        const int id = ids[(size_t)t * k + tid];
+        int rank = 0;
+        for (int j = 0; j < k; j++) {
+            const int o = ids[(size_t)t * k + j];
+            rank += (o < id) || (o == id && j < tid);
+        }
+        s_order[rank] = tid;
+    }
+    const size_t row_bytes = type_row_bytes(WT, inter);
+    for (int sl = wave; sl < k; sl += 8) {
+        const int a = t * k + sl;
+        const int e = ids[a];
+        float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if ((unsigned)e < (unsigned)n_experts) {  // (a bad id was flagged by gate/up)
+            const uint8_t *de = down + (size_t)e * (size_t)hidden * row_bytes;
+            const uint8_t *rowp[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) rowp[j] = de + (size_t)(row0 + j < hidden ? row0 + j : row0) * row_bytes;
+            rows_partial_f<WT, VEC, 8>(rowp, act + (size_t)a * (size_t)inter, inter, lane, p);
+#pragma unroll
+            for (int j = 0; j < 8; j++) p[j] = wave_sum(p[j]);
+        }
+        if (lane < 8) {
+            float v = p[0];
+#pragma unroll
+            for (int j = 1; j < 8; j++) v = lane == j ? p[j] : v;
+            s_y[sl][lane] = v;
+        }
+    }
+    __syncthreads();
+    if (tid < 8 && row0 + tid < hidden) {
+        float sum = 0.0f;
+        for (int r = 0; r < k; r++) {
+            const int sl = s_order[r];
+            sum = __fadd_rn(sum, __fmul_rn(weights[(size_t)t * k + sl], s_y[sl][tid]));
+        }
+        const size_t o = (size_t)t * (size_t)hidden + row0 + tid;
+        out[o] = residual ? __fadd_rn(residual[o], sum) : sum;
+    }
+}
+
+hipError_t launch_down_combine_f(const ExpertBanks &b, const float *act, const int32_t *ids, const float *weights, int n, int k,
+                                 const float *residual, float *out, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (!float_decode_fused(b, k) || n > 65535) return hipErrorInvalidValue;
+    return with_bank_type(b.down_type, [&](auto tag) {
+        constexpr int WT = decltype(tag)::value;
+        if constexpr (!is_quant_type(WT)) {
+            dim3 block(512), grid(n, (b.hidden + 7) / 8);
+            constexpr int WIDE = WT == T_F32 ? 4 : 8;
+            if (b.inter % WIDE == 0 && (((uintptr_t)b.down & 15) == 0))
+                launch_kernel(down_combine_f_kernel<WT, WIDE>, grid, block, 0, s, b.down, act, ids, weights, k, b.hidden, b.inter,
+                              b.n_experts, residual, out);
+            else if (b.inter % 4 == 0)
+                launch_kernel(down_combine_f_kernel<WT, 4>, grid, block, 0, s, b.down, act, ids, weights, k, b.hidden, b.inter,
+                              b.n_experts, residual, out);
+            else
+                launch_kernel(down_combine_f_kernel<WT, 1>, grid, block, 0, s, b.down, act, ids, weights, k, b.hidden, b.inter,
+                              b.n_experts, residual, out);
+            return hipGetLastError();
+        } else {
+            return hipErrorInvalidValue;
+        }
     });
 }
 

@@ -70,6 +70,13 @@ struct RouteInline {
 bool gate_up_routes_inline(const ExpertBanks &b, int k);
 hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInline &route, int n_tokens, int k, QAct actq,
                                  int32_t *flags, hipStream_t s);
+// The same pair for float banks (F32 / F16 / BF16 gate/up and down, at most 512 experts, top_k <= 16):
+// gate/up with the routing inside writes act [n*k, inter] f32, then down + combine in one launch.
+bool float_decode_fused(const ExpertBanks &b, int k);
+hipError_t launch_gate_up_f_routed(const ExpertBanks &b, const float *x, const RouteInline &route, int n_tokens, int k, float *act,
+                                   int32_t *flags, hipStream_t s);
+hipError_t launch_down_combine_f(const ExpertBanks &b, const float *act, const int32_t *ids, const float *weights, int n, int k,
+                                 const float *residual, float *out, hipStream_t s);
 // y[a, c] = <down_e[c,:], act[a,:]>   (actq for a quantized down bank, else act)
 hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign, int k,
                        int fixed_expert, float *y, hipStream_t s);

@@ -75,8 +75,8 @@ struct mummu_moe {
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
     // batches at least this large take dispatch + grouped GEMM (measured crossovers on the OLMoE shape:
-    // the float decode kernels lose from 6 tokens on, the integer ones from 19)
-    int gemm_min_f16 = 6, gemm_min_quant = 19;
+    // the float decode kernels lose from 7 tokens on, the integer ones from 19)
+    int gemm_min_f16 = 7, gemm_min_quant = 19;
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
@@ -375,6 +375,19 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
             route.hits = L.hits;
             LAUNCH(h, K_GATE_UP, s, launch_gate_up_routed(b, h->xq, route, (int)n, k, h->actq, h->flags, s));
             LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, k, residual, out, s));
+            return MUMMU_OK;
+        }
+        if (!batched && float_decode_fused(b, k)) {
+            // float banks: the same two fusions
+            RouteInline route;
+            route.logits = h->logits;
+            route.flavour = h->cfg.router_flavour;
+            route.norm = norm;
+            route.ids = h->ids;
+            route.weights = h->weights;
+            route.hits = L.hits;
+            LAUNCH(h, K_GATE_UP, s, launch_gate_up_f_routed(b, x, route, (int)n, k, h->act, h->flags, s));
+            LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine_f(b, h->act, h->ids, h->weights, (int)n, k, residual, out, s));
             return MUMMU_OK;
         }
         LAUNCH(h, K_ROUTE_TOPK, s,
