@@ -67,6 +67,9 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--stack", action="store_true",
                     help="a step is x <- x + MoE_l(RmsNorm_l(x)) through all --layers layers (reported per layer)")
+    ap.add_argument("--shared-inter", type=int, default=0,
+                    help="also give every layer a shared expert of this intermediate width with a sigmoid gate "
+                         "(Qwen-style block; same bank types); the CPU baseline leg is skipped")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--seed", type=int, default=1234)
@@ -106,6 +109,13 @@ def main() -> int:
             return (w32.view(np.uint32) >> np.uint32(16)).astype(np.uint16).view(np.uint8)  # (truncated: statistics only)
         return (w32 if t == M.F32 else w32.astype(np.float16)).view(np.uint8)
 
+    def make_bank_1(ne, seed, t):
+        gg = np.random.Generator(np.random.PCG64(seed))
+        w32 = gg.standard_normal(ne[0] * ne[1] * ne[2], dtype=np.float32) * np.float32(0.02)
+        if t == M.BF16:
+            return (w32.view(np.uint32) >> np.uint32(16)).astype(np.uint16).view(np.uint8)
+        return (w32 if t == M.F32 else w32.astype(np.float16)).view(np.uint8)
+
     t_setup = time.time()
     moe = M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=max(n, 8), norm_topk_prob=norm,
                       router_flavour=w.get("flavour", 0))
@@ -117,6 +127,13 @@ def main() -> int:
         up = make_bank(H, I, args.seed * 1000 + 3 * l + 1)
         down = make_bank(I, H, args.seed * 1000 + 3 * l + 2, down_t)
         moe.load_layer(l, router, router_t, gate, bank_t, up, bank_t, down, down_t, np.ones(H, np.float32) if args.stack else None)
+        if args.shared_inter:
+            IS = args.shared_inter
+            sh = [synth.random_bank_fast(t_, ne, args.seed * 7000 + 3 * l + j) if t_ not in (M.F16, M.F32, M.BF16) else
+                  make_bank_1(ne, args.seed * 7000 + 3 * l + j, t_)
+                  for j, (t_, ne) in enumerate(((bank_t, [H, IS, 1]), (bank_t, [H, IS, 1]), (down_t, [IS, H, 1])))]
+            gate_vec = (g.standard_normal(H, dtype=np.float32) * np.float32(0.05)).astype(np.float32)
+            moe.load_shared_expert(l, IS, sh[0], bank_t, sh[1], bank_t, sh[2], down_t, gate_vec)
         routers.append(router)
         if l == 0:
             keep_layer0 = (router, gate, up, down)
@@ -241,7 +258,7 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
-                   "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
+                   "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "shared_inter": args.shared_inter, "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
                    "mean_distinct_experts_per_step": round(mean_distinct, 3)},
         "us_per_layer": round(ms_per_step * 1e3, 3),
         "event_ms_per_step": round(ev_ms / args.steps / layers_per_step, 6),
@@ -259,7 +276,7 @@ def main() -> int:
         "setup_s": round(setup_s, 1),
     }
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not args.shared_inter:
         out["cpu_baseline"] = cpu_baseline(keep_layer0, w, bank_t, down_t, xs, n, args.cpu_seconds)
     print(json.dumps(out))
     return 0

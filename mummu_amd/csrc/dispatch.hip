@@ -265,6 +265,27 @@ __global__ __launch_bounds__(kDispatchThreads) void dispatch_fused_kernel(
     }
 }
 
+// The work list of ONE expert that serves every row in order (the shared expert of a Qwen-style
+// block on the batched path): sorted[i] = i, tiles of tile_rows rows of expert 0.
+__global__ __launch_bounds__(256) void identity_tiles_kernel(int n, int tile_rows, int32_t *__restrict__ sorted,
+                                                             int32_t *__restrict__ tiles, int32_t *__restrict__ n_tiles) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) sorted[i] = i;
+    const int nt = (n + tile_rows - 1) / tile_rows;
+    if (i < nt) {
+        tiles[3 * i] = 0;
+        tiles[3 * i + 1] = i * tile_rows;
+        tiles[3 * i + 2] = (n - i * tile_rows) < tile_rows ? (n - i * tile_rows) : tile_rows;
+    }
+    if (i == 0) *n_tiles = nt;
+}
+
+hipError_t launch_identity_tiles(int n, int tile_rows, int32_t *sorted, int32_t *tiles, int32_t *n_tiles, hipStream_t s) {
+    if (n <= 0 || tile_rows < 1) return hipErrorInvalidValue;
+    launch_kernel(identity_tiles_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, tile_rows, sorted, tiles, n_tiles);
+    return hipGetLastError();
+}
+
 size_t dispatch_scratch_ints(int n_assign, int n_experts) {
     const size_t chunks = ((size_t)n_assign + kDispatchThreads - 1) / kDispatchThreads;
     return (size_t)n_assign + chunks * (size_t)n_experts;

@@ -834,27 +834,90 @@ hipError_t launch_combine(const float *y, const int32_t *ids, const float *weigh
 }
 
 // ------------------------------------------------------------------------------------------
-// shared expert: out = [residual +] (out + y * sigmoid(logit)), each operation rounded on its own
-// (models/qwen4exp/model.rs:786-804).  logit null: the shared expert is not gated.
+// shared expert: out = [residual +] (out + y * sigmoid(<gate_vec, x>)), each operation rounded on its
+// own (models/qwen4exp/model.rs:786-804).  gate_vec null: the shared expert is not gated.  Every wave
+// computes the token's gate logit for itself, in the router's order (eight partials per lane over
+// 512-element chunks, the fixed fold, the wave sum): no launch of its own for one dot product.
 // ------------------------------------------------------------------------------------------
+template <int WT, bool VEC>
+__device__ inline float gate_logit(const float *__restrict__ xrow, const void *__restrict__ gv, int hidden, int lane) {
+    float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 4
+    for (int base = lane * 8; base < hidden; base += 512) {
+        if constexpr (VEC) {  // hidden % 8 == 0, both rows 16-byte aligned: the lane's 8 elements are inside the row
+            const float4 p = *(const float4 *)(xrow + base), q = *(const float4 *)(xrow + base + 4);
+            const float xv[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+            float w[8];
+            if constexpr (WT == T_F32) {
+                const float4 u = *(const float4 *)((const float *)gv + base), v = *(const float4 *)((const float *)gv + base + 4);
+                w[0] = u.x; w[1] = u.y; w[2] = u.z; w[3] = u.w; w[4] = v.x; w[5] = v.y; w[6] = v.z; w[7] = v.w;
+            } else {
+                const uint4 u = *(const uint4 *)((const uint16_t *)gv + base);
+                const uint32_t r[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const uint16_t hb = (uint16_t)((r[j / 2] >> (16 * (j & 1))) & 0xFFFFu);
+                    w[j] = WT == T_F16 ? half_bits_to_float(hb) : bf16_bits_to_float(hb);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) a[j] = __builtin_fmaf(xv[j], w[j], a[j]);
+            continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = base + j;
+            float w = 0.0f, xv = 0.0f;  // +0 leaves a partial unchanged
+            if (i < hidden) {
+                xv = xrow[i];
+                if constexpr (WT == T_F32) w = ((const float *)gv)[i];
+                else if constexpr (WT == T_F16) w = half_bits_to_float(((const uint16_t *)gv)[i]);
+                else w = bf16_bits_to_float(((const uint16_t *)gv)[i]);
+            }
+            a[j] = __builtin_fmaf(xv, w, a[j]);
+        }
+    }
+    const float sum = __fadd_rn(__fadd_rn(__fadd_rn(a[0], a[4]), __fadd_rn(a[1], a[5])),
+                                __fadd_rn(__fadd_rn(a[2], a[6]), __fadd_rn(a[3], a[7])));
+    return wave_sum(sum);
+}
+
+template <int WT, bool VEC>
 __global__ __launch_bounds__(256) void shared_add_kernel(float *__restrict__ out, const float *__restrict__ y,
-                                                         const float *__restrict__ logit, const float *__restrict__ residual,
-                                                         int hidden) {
+                                                         const float *__restrict__ x, const void *__restrict__ gate_vec,
+                                                         const float *__restrict__ residual, int hidden) {
     const int t = blockIdx.x;
     float g = 1.0f;
-    if (logit) g = __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-logit[t])));
+    if (gate_vec) {
+        const float logit = gate_logit<WT, VEC>(x + (size_t)t * (size_t)hidden, gate_vec, hidden, threadIdx.x & 63);
+        g = __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-logit)));
+    }
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < hidden; c += gridDim.y * blockDim.x) {
         const size_t o = (size_t)t * (size_t)hidden + c;
-        const float shared = logit ? __fmul_rn(y[o], g) : y[o];
+        const float shared = gate_vec ? __fmul_rn(y[o], g) : y[o];
         const float v = __fadd_rn(out[o], shared);
         out[o] = residual ? __fadd_rn(residual[o], v) : v;
     }
 }
 
-hipError_t launch_shared_add(float *out, const float *y, const float *logit, const float *residual, int n, int hidden, hipStream_t s) {
+hipError_t launch_shared_add(float *out, const float *y, const float *x, const void *gate_vec, int gate_vec_type,
+                             const float *residual, int n, int hidden, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     int ysplit = n >= 64 ? 1 : (hidden + 255) / 256;
-    launch_kernel(shared_add_kernel, dim3(n, ysplit), dim3(256), 0, s, out, y, logit, residual, hidden);
+    dim3 grid(n, ysplit), block(256);
+    const bool vec = hidden % 8 == 0 && ((((uintptr_t)x | (uintptr_t)gate_vec) & 15) == 0);
+#define MUMMU_SA(WT)                                                                                              \
+    do {                                                                                                          \
+        if (vec) launch_kernel(shared_add_kernel<WT, true>, grid, block, 0, s, out, y, x, gate_vec, residual, hidden); \
+        else launch_kernel(shared_add_kernel<WT, false>, grid, block, 0, s, out, y, x, gate_vec, residual, hidden);    \
+    } while (0)
+    switch (gate_vec ? gate_vec_type : T_F32) {
+    case T_F32: MUMMU_SA(T_F32); break;
+    case T_F16: MUMMU_SA(T_F16); break;
+    case T_BF16: MUMMU_SA(T_BF16); break;
+    default: return hipErrorInvalidValue;
+    }
+#undef MUMMU_SA
     return hipGetLastError();
 }
 

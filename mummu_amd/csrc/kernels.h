@@ -91,10 +91,10 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
                                const float *residual, float *out, hipStream_t s);
 
 
-// out[t, :] = [residual[t, :] +] (out[t, :] + y[t, :] * sigmoid(logit[t])), every operation rounded on
-// its own; logit null: no gate.
-hipError_t launch_shared_add(float *out, const float *y, const float *logit, const float *residual, int n, int hidden,
-                             hipStream_t s);
+// out[t, :] = [residual[t, :] +] (out[t, :] + y[t, :] * sigmoid(<gate_vec, x[t, :]>)), every operation
+// rounded on its own, the dot product in the router's order; gate_vec (F32 / F16 / BF16) null: no gate.
+hipError_t launch_shared_add(float *out, const float *y, const float *x, const void *gate_vec, int gate_vec_type,
+                             const float *residual, int n, int hidden, hipStream_t s);
 
 // dispatch.hip ------------------------------------------------------------------------
 // Stable counting sort of the assignments by expert (ranks, histograms and scans in LDS, three
@@ -106,6 +106,10 @@ size_t dispatch_scratch_ints(int n_assign, int n_experts);
 hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int tile_rows, int32_t *offsets,
                            int32_t *sorted, int32_t *inv, int32_t *tiles, int32_t *n_tiles, int32_t *scratch,
                            unsigned long long *hits, int32_t *flags, hipStream_t s);
+
+// One expert serving rows 0..n-1 in order: sorted[i] = i and the tile list of expert 0 (tiles: 3 ints
+// per tile, at least ceil(n / tile_rows) tiles).
+hipError_t launch_identity_tiles(int n, int tile_rows, int32_t *sorted, int32_t *tiles, int32_t *n_tiles, hipStream_t s);
 
 // gemm.hip ----------------------------------------------------------------------------
 // Grouped GEMMs over the dispatch-sorted assignments on the matrix cores (hidden and inter

@@ -82,6 +82,9 @@ struct mummu_moe {
     int64_t sh_ws_tokens = 0;
     float *sh_act = nullptr, *sh_y = nullptr, *sh_logit = nullptr;
     QAct sh_actq;
+    void *sh_act16 = nullptr;                                   // f16 [tokens, shared inter]: batched path, F16 / BF16 banks
+    int32_t *sh_sorted = nullptr, *sh_tiles = nullptr, *sh_ntiles = nullptr;  // its one-expert work list
+    int sh_max_tiles = 0;
 
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing = false;
@@ -122,11 +125,14 @@ void free_ws(mummu_moe *h) {
     h->act16 = nullptr;
     h->ws_tokens = h->ws_assign = 0;
     h->ws_experts = 0;
-    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum};
+    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
+                  h->sh_act16, h->sh_sorted, h->sh_tiles, h->sh_ntiles};
     for (void *p : sh)
         if (p) (void)hipFree(p);
     h->sh_act = h->sh_y = h->sh_logit = nullptr;
     h->sh_actq = QAct();
+    h->sh_act16 = nullptr;
+    h->sh_sorted = h->sh_tiles = h->sh_ntiles = nullptr;
     h->sh_ws_tokens = 0;
 }
 
@@ -134,11 +140,14 @@ void free_ws(mummu_moe *h) {
 int ensure_shared_ws(mummu_moe *h) {
     if (h->sh_inter_max == 0 || h->sh_ws_tokens >= h->ws_tokens) return MUMMU_OK;
     HIPCHK(h, hipDeviceSynchronize());
-    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum};
+    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
+                  h->sh_act16, h->sh_sorted, h->sh_tiles, h->sh_ntiles};
     for (void *p : sh)
         if (p) (void)hipFree(p);
     h->sh_act = h->sh_y = h->sh_logit = nullptr;
     h->sh_actq = QAct();
+    h->sh_act16 = nullptr;
+    h->sh_sorted = h->sh_tiles = h->sh_ntiles = nullptr;
     const size_t nt = (size_t)h->ws_tokens, H = (size_t)h->cfg.hidden_size, I = (size_t)h->sh_inter_max;
     const size_t ae = nt * ((I + 15) / 16 * 16);
     HIPCHK(h, hipMalloc(&h->sh_act, sizeof(float) * nt * I));
@@ -148,6 +157,12 @@ int ensure_shared_ws(mummu_moe *h) {
     HIPCHK(h, hipMalloc(&h->sh_actq.lo, ae));
     HIPCHK(h, hipMalloc(&h->sh_actq.scale, sizeof(float) * (ae / 16)));
     HIPCHK(h, hipMalloc(&h->sh_actq.sum, sizeof(int32_t) * (ae / 16)));
+    HIPCHK(h, hipMalloc(&h->sh_act16, 2 * nt * I));
+
+    h->sh_max_tiles = (int)((nt + 31) / 32) + 1;
+    HIPCHK(h, hipMalloc(&h->sh_sorted, sizeof(int32_t) * nt));
+    HIPCHK(h, hipMalloc(&h->sh_tiles, sizeof(int32_t) * 3 * (size_t)h->sh_max_tiles));
+    HIPCHK(h, hipMalloc(&h->sh_ntiles, sizeof(int32_t)));
     h->sh_ws_tokens = h->ws_tokens;
     return MUMMU_OK;
 }
@@ -405,8 +420,6 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     const Layer &L = h->layers[layer];
     if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s, norm_gamma);
     if (norm_gamma) return fail(h, MUMMU_ERR_ARG, "fused RmsNorm with a shared expert");
-    int rc = routed_impl(h, layer, x, n, k, norm, nullptr, out, s);
-    if (rc) return rc;
     if (n > h->sh_ws_tokens) return fail(h, MUMMU_ERR_TOKENS, "shared-expert workspace is smaller than the call");
     const int H = h->cfg.hidden_size;
     ExpertBanks b;
@@ -419,13 +432,33 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     b.hidden = H;
     b.inter = L.sh_inter;
     b.n_experts = 1;
-    // the routed path may have left the 16-bit activations in the batched layout (or not made them)
-    if (is_quant_type(b.gate_type)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x, (int)n, H, h->xq, s));
-    LAUNCH(h, K_SHARED, s, launch_gate_up(b, x, h->xq, nullptr, (int)n, 1, 0, h->sh_act, h->sh_actq, h->flags, s));
-    LAUNCH(h, K_SHARED, s, launch_down(b, h->sh_act, h->sh_actq, nullptr, (int)n, 1, 0, h->sh_y, s));
-    if (L.sh_gatevec)
-        LAUNCH(h, K_SHARED, s, launch_router_logits(x, L.sh_gatevec, L.sh_gatevec_type, h->sh_logit, (int)n, H, 1, QAct(), s));
-    LAUNCH(h, K_SHARED, s, launch_shared_add(out, h->sh_y, L.sh_gatevec ? h->sh_logit : nullptr, residual, (int)n, H, s));
+    const int sh_from = !grouped_gemm_supported(b) ? 0x7fffffff : (grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16);
+    // (one expert makes few workgroups: tiles x 128-row slabs.  Measured at H 2048, shared inter 2048, Q4_K: the
+    // per-token kernels cost 68 us at 64 tokens and 396 us at 512, the GEMM pair about 145 us at either)
+    int rc = routed_impl(h, layer, x, n, k, norm, nullptr, out, s);
+    if (rc) return rc;
+    if (n >= sh_from && n >= 192) {
+        // many tokens: the shared expert is one more grouped GEMM pair, every row in order on expert 0
+        const int tile_rows = grouped_gemm_tile_rows(b, (int)n, 1);
+        const QAct64 xq64{h->xq.hi, h->xq.lo, h->xq.scale, (float *)h->xq.sum};
+        const QAct64 actq64{h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, (float *)h->sh_actq.sum};
+        LAUNCH(h, K_SHARED, s, launch_identity_tiles((int)n, tile_rows, h->sh_sorted, h->sh_tiles, h->sh_ntiles, s));
+        // (the routed path may have left the 16-bit activations in the decode layout, or not made them)
+        if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, H, xq64, s));
+        LAUNCH(h, K_SHARED, s,
+               launch_gemm_gate_up(b, x, xq64, h->sh_sorted, 1, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_act16,
+                                   actq64, s));
+        LAUNCH(h, K_SHARED, s,
+               launch_gemm_down(b, h->sh_act16, actq64, (int)n, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_y, s));
+    } else {
+        // the routed decode kernels leave x in the 16-bit decode layout when their own banks are quantized;
+        // otherwise (float routed banks, or the batched path's layout) it is made here
+        const bool have_xq = is_quant_type(L.gate_type) && H % 64 == 0 && n < batched_from(h, L);
+        if (is_quant_type(b.gate_type) && !have_xq) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x, (int)n, H, h->xq, s));
+        LAUNCH(h, K_SHARED, s, launch_gate_up(b, x, h->xq, nullptr, (int)n, 1, 0, h->sh_act, h->sh_actq, h->flags, s));
+        LAUNCH(h, K_SHARED, s, launch_down(b, h->sh_act, h->sh_actq, nullptr, (int)n, 1, 0, h->sh_y, s));
+    }
+    LAUNCH(h, K_SHARED, s, launch_shared_add(out, h->sh_y, x, L.sh_gatevec, L.sh_gatevec_type, residual, (int)n, H, s));
     return MUMMU_OK;
 }
 
