@@ -80,7 +80,7 @@ struct mummu_moe {
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
-    float *sh_act = nullptr, *sh_y = nullptr, *sh_logit = nullptr;
+    float *sh_act = nullptr, *sh_y = nullptr;
     QAct sh_actq;
     void *sh_act16 = nullptr;                                   // f16 [tokens, shared inter]: batched path, F16 / BF16 banks
     int32_t *sh_sorted = nullptr, *sh_tiles = nullptr, *sh_ntiles = nullptr;  // its one-expert work list
@@ -125,11 +125,11 @@ void free_ws(mummu_moe *h) {
     h->act16 = nullptr;
     h->ws_tokens = h->ws_assign = 0;
     h->ws_experts = 0;
-    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
+    void *sh[] = {h->sh_act, h->sh_y, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
                   h->sh_act16, h->sh_sorted, h->sh_tiles, h->sh_ntiles};
     for (void *p : sh)
         if (p) (void)hipFree(p);
-    h->sh_act = h->sh_y = h->sh_logit = nullptr;
+    h->sh_act = h->sh_y = nullptr;
     h->sh_actq = QAct();
     h->sh_act16 = nullptr;
     h->sh_sorted = h->sh_tiles = h->sh_ntiles = nullptr;
@@ -140,11 +140,11 @@ void free_ws(mummu_moe *h) {
 int ensure_shared_ws(mummu_moe *h) {
     if (h->sh_inter_max == 0 || h->sh_ws_tokens >= h->ws_tokens) return MUMMU_OK;
     HIPCHK(h, hipDeviceSynchronize());
-    void *sh[] = {h->sh_act, h->sh_y, h->sh_logit, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
+    void *sh[] = {h->sh_act, h->sh_y, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
                   h->sh_act16, h->sh_sorted, h->sh_tiles, h->sh_ntiles};
     for (void *p : sh)
         if (p) (void)hipFree(p);
-    h->sh_act = h->sh_y = h->sh_logit = nullptr;
+    h->sh_act = h->sh_y = nullptr;
     h->sh_actq = QAct();
     h->sh_act16 = nullptr;
     h->sh_sorted = h->sh_tiles = h->sh_ntiles = nullptr;
@@ -152,7 +152,6 @@ int ensure_shared_ws(mummu_moe *h) {
     const size_t ae = nt * ((I + 15) / 16 * 16);
     HIPCHK(h, hipMalloc(&h->sh_act, sizeof(float) * nt * I));
     HIPCHK(h, hipMalloc(&h->sh_y, sizeof(float) * nt * H));
-    HIPCHK(h, hipMalloc(&h->sh_logit, sizeof(float) * nt));
     HIPCHK(h, hipMalloc(&h->sh_actq.hi, ae));
     HIPCHK(h, hipMalloc(&h->sh_actq.lo, ae));
     HIPCHK(h, hipMalloc(&h->sh_actq.scale, sizeof(float) * (ae / 16)));
