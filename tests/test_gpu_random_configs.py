@@ -83,5 +83,7 @@ def test_a_random_configuration_matches_the_oracle(seed):
     want, mag = orc.moe_ref_f64(banks, oids, ow, x)
     exact_float = gt in (M.F32, M.BF16) and dt in (M.F32, M.BF16) and n < batched_from
     tol = 1e-5 if exact_float else 2e-3
-    err = orc.rel_err(got, want, mag).max()
+    # (outputs 100 times smaller than the batch's typical magnitude - a token whose hidden row is all but zero - are
+    # held to the tolerance against that floor, not against their own magnitude)
+    err = orc.rel_err(got, want, np.maximum(mag, 1e-2 * np.median(mag))).max()
     assert err <= tol, f"{what}: max relative error {err:.3e} > {tol}"

@@ -27,7 +27,9 @@ def bank(t, ne, seed, std=0.05):
 
 
 def reference(banks, shared, router, rt, gate_vec, x, k, norm, flavour):
-    """(routed, full): routed from the oracle's block, full = routed + shared * sigmoid (f64 for the tolerance)."""
+    """(ids, weights, routed, full, magnitude): routed from the oracle's block, full = routed + shared * sigmoid
+    (f64 for the tolerance).  Each part is held to the tolerance against its own magnitude, so their sum is held
+    against the sum of the two."""
     _, ids, w, _ = orc.moe_forward(banks, router, rt, x, k, norm, flavour)
     routed, mag = orc.moe_ref_f64(banks, ids, w, x)
     n = x.shape[0]
@@ -37,7 +39,7 @@ def reference(banks, shared, router, rt, gate_vec, x, k, norm, flavour):
     else:
         z = orc.router_logits(x, gate_vec, orc.F32, 1).astype(np.float64).reshape(n, 1)
         g = 1.0 / (1.0 + np.exp(-z))
-    return ids, w, routed, routed + sh * g, np.maximum(mag, smag * g)
+    return ids, w, routed, routed + sh * g, mag + smag * g
 
 
 CASES = [
@@ -159,3 +161,55 @@ def test_shared_expert_arguments_are_checked():
         with pytest.raises(M.MoeError, match="share one type"):
             m.load_shared_expert(0, 64, z(64 * H // 32 * 34, np.uint8), M.Q8_0, z(64 * H, np.float32), M.F32,
                                  z(H * 64, np.float32), M.F32)
+
+
+def draw_shared(seed):
+    g = np.random.Generator(np.random.PCG64(500 + seed))
+    quant = [M.Q4_0, M.Q4_1, M.Q5_0, M.Q5_1, M.Q8_0, M.Q4_K, M.Q5_K, M.Q6_K]
+    pool = quant + [M.F32]
+    kq = (M.Q4_K, M.Q5_K, M.Q6_K)
+    gt, dt, sgt, sdt = (pool[g.integers(0, len(pool))] for _ in range(4))
+    if g.integers(0, 2):  # the usual file: routed and shared banks of the same types
+        sgt, sdt = gt, dt
+    unit_h = 256 if (gt in kq or sgt in kq) else 64
+    H = int(unit_h * g.integers(1, 1 + 768 // unit_h))
+    I = int((256 if dt in kq else 64) * g.integers(1, 3))
+    IS = int((256 if sdt in kq else 64) * g.integers(1, 5))
+    E = int(g.choice([4, 8, 20, 64]))
+    k = int(g.integers(1, min(E, 8) + 1))
+    n = int(g.choice([1, 2, 7, 8, 9, 20, 40, 191, 192, 260]))   # 192: the shared expert moves to the grouped GEMM
+    flavour = int(g.integers(0, 2))
+    return gt, dt, sgt, sdt, H, I, IS, E, k, n, flavour, bool(g.integers(0, 4))
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_a_random_block_with_a_shared_expert_matches_the_composition(seed):
+    gt, dt, sgt, sdt, H, I, IS, E, k, n, flavour, gated = draw_shared(seed)
+    gate, up, down = bank(gt, [H, I, E], 11 * seed + 1), bank(gt, [H, I, E], 11 * seed + 2), bank(dt, [I, H, E], 11 * seed + 3)
+    sgate, sup, sdown = bank(sgt, [H, IS, 1], 11 * seed + 4), bank(sgt, [H, IS, 1], 11 * seed + 5), bank(sdt, [IS, H, 1], 11 * seed + 6)
+    router = normal((E, H), 11 * seed + 7, 0.05)
+    gate_vec = normal((H,), 11 * seed + 8, 0.2) if gated else None
+    x = normal((n, H), 11 * seed + 9)
+    norm = flavour == M.ROUTER_QWEN4EXP or bool(seed & 1)
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=n, router_flavour=flavour) as m:
+        m.load_layer(0, router, M.F32, gate, gt, up, gt, down, dt)
+        m.load_shared_expert(0, IS, sgate, sgt, sup, sgt, sdown, sdt, gate_vec)
+        got = m.forward(x, k, norm)
+        gids, gw = m.last_routing(n, k)
+        again = m.forward(x, k, norm)
+    banks = orc.LayerBanks(H, I, E, gate, up, down, gt, gt, dt)
+    shared = orc.LayerBanks(H, IS, 1, sgate, sup, sdown, sgt, sgt, sdt)
+    ids, w, _, full, mag = reference(banks, shared, router, orc.F32, gate_vec, x, k, norm, flavour)
+    what = f"seed {seed}: routed {gt}/{dt}, shared {sgt}/{sdt}, H {H}, I {I}, IS {IS}, E {E}, k {k}, n {n}, flavour {flavour}, gated {gated}"
+    assert np.array_equal(gids, ids.astype(np.int32)), what
+    assert np.array_equal(gw.view(np.uint32), w.view(np.uint32)), what
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), what
+    tol = 1e-5 if all(t == M.F32 for t in (gt, dt, sgt, sdt)) else 2e-3
+    # A token whose gate pre-activations are all far below zero has a hidden row of near-zeros with one element
+    # standing out by many orders of magnitude, and outputs 1e5 times smaller than the batch's: the 16-bit
+    # block-scaled activations keep few bits of the small elements beside the large one, so such outputs are held
+    # to the tolerance against a floor of 1e-2 of the batch's typical magnitude instead of their own (seed 7 has
+    # one such token).
+    floor = 1e-2 * np.median(mag)
+    err = orc.rel_err(got, full, np.maximum(mag, floor)).max()
+    assert err <= tol, f"{what}: max relative error {err:.3e} > {tol}"
