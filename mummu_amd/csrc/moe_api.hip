@@ -60,6 +60,9 @@ struct mummu_moe {
     mummu_moe_config cfg{};
     std::vector<Layer> layers;
     hipStream_t stream = nullptr;
+    // pinned host staging for the host-pointer entry points: [input | output | flags]; small calls go through
+    // it with asynchronous copies and one synchronisation
+    uint8_t *pin = nullptr;
     std::mutex mu;
     mutable std::string err;
 
@@ -221,11 +224,17 @@ int reset_flags(mummu_moe *h) {
     return MUMMU_OK;
 }
 
+int flags_to_status(mummu_moe *h, const int32_t *f);
+
 // Synchronise and translate the device error flags.
 int check_flags(mummu_moe *h, hipStream_t s) {
     HIPCHK(h, hipStreamSynchronize(s));
     int32_t f[4];
     HIPCHK(h, hipMemcpy(f, h->flags, sizeof(f), hipMemcpyDeviceToHost));
+    return flags_to_status(h, f);
+}
+
+int flags_to_status(mummu_moe *h, const int32_t *f) {
     if (f[FLAG_NONFINITE] == 0 && f[FLAG_BAD_ID] == 0) return MUMMU_OK;
     int rc = reset_flags(h);
     if (rc != MUMMU_OK) return rc;
@@ -237,6 +246,45 @@ int check_flags(mummu_moe *h, hipStream_t s) {
         return fail(h, MUMMU_ERR_NONFINITE, buf);
     }
     return fail(h, MUMMU_ERR_RANGE, "a routed expert id is out of range");
+}
+
+// Host-pointer calls of up to kPinIO bytes each way: the input is staged through pinned memory (the
+// copy is then truly asynchronous), and the output and the error flags come back with one
+// synchronisation instead of one per copy.  Larger calls copy straight from / to the caller's memory.
+constexpr size_t kPinIO = 256 * 1024;
+
+int upload_rows(mummu_moe *h, float *dev, const float *host, size_t bytes, hipStream_t s) {
+    if (h->pin && bytes <= kPinIO) {
+        memcpy(h->pin, host, bytes);
+        HIPCHK(h, hipMemcpyAsync(dev, h->pin, bytes, hipMemcpyHostToDevice, s));
+    } else {
+        HIPCHK(h, hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, s));
+    }
+    return MUMMU_OK;
+}
+
+// Wait for the stream, report what the device flagged, hand the result rows to the caller.
+int download_rows(mummu_moe *h, float *host, const float *dev, size_t bytes, hipStream_t s, bool with_flags) {
+    if (h->pin && bytes <= kPinIO) {
+        int32_t *pf = (int32_t *)(h->pin + 2 * kPinIO);
+        if (with_flags) HIPCHK(h, hipMemcpyAsync(pf, h->flags, sizeof(int32_t) * kFlagWords, hipMemcpyDeviceToHost, s));
+        HIPCHK(h, hipMemcpyAsync(h->pin + kPinIO, dev, bytes, hipMemcpyDeviceToHost, s));
+        HIPCHK(h, hipStreamSynchronize(s));
+        if (with_flags) {
+            const int rc = flags_to_status(h, pf);
+            if (rc) return rc;
+        }
+        memcpy(host, h->pin + kPinIO, bytes);
+        return MUMMU_OK;
+    }
+    if (with_flags) {
+        const int rc = check_flags(h, s);
+        if (rc) return rc;
+    } else {
+        HIPCHK(h, hipStreamSynchronize(s));
+    }
+    HIPCHK(h, hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
 }
 
 // Per-kernel timing: binds a pair of pooled events to the one kernel the enclosed launcher
@@ -545,6 +593,10 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     };
     if (hipSetDevice(0) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipSetDevice(0) failed"));
     if (hipStreamCreate(&h->stream) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipStreamCreate failed"));
+    if (hipHostMalloc((void **)&h->pin, 2 * kPinIO + 64, hipHostMallocDefault) != hipSuccess) {
+        h->pin = nullptr;  // not fatal: the calls then copy straight from the caller's memory
+        (void)hipGetLastError();
+    }
     if (hipEventCreate(&h->t0) != hipSuccess || hipEventCreate(&h->t1) != hipSuccess)
         return bail(fail(h, MUMMU_ERR_DEVICE, "hipEventCreate failed"));
     if (hipMalloc(&h->flags, sizeof(int32_t) * kFlagWords) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(flags) failed"));
@@ -573,6 +625,7 @@ void mummu_moe_destroy(mummu_moe *h) {
     for (auto e : h->event_pool) (void)hipEventDestroy(e);
     if (h->t0) (void)hipEventDestroy(h->t0);
     if (h->t1) (void)hipEventDestroy(h->t1);
+    if (h->pin) (void)hipHostFree(h->pin);
     if (h->stream) (void)hipStreamDestroy(h->stream);
     delete h;
 }
@@ -711,11 +764,9 @@ int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n, int to
     if (!x || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
     if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
     const size_t bytes = sizeof(float) * (size_t)n * (size_t)h->cfg.hidden_size;
-    HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, h->stream));
+    if ((rc = upload_rows(h, h->xin, x, bytes, h->stream))) return rc;
     if ((rc = forward_impl(h, layer, h->xin, n, top_k, norm, nullptr, h->xout, h->stream))) return rc;
-    if ((rc = check_flags(h, h->stream))) return rc;
-    HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
-    return MUMMU_OK;
+    return download_rows(h, out, h->xout, bytes, h->stream, true);
 }
 
 int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_k, int norm, int32_t *ids, float *weights,
@@ -806,9 +857,7 @@ int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const f
         HIPCHK(h, hipMemcpy(L.hits, cur.data(), sizeof(unsigned long long) * cur.size(), hipMemcpyHostToDevice));
     }
     if ((rc = run_experts(h, L, h->xin, false, n, top_k, nullptr, h->xout, s))) return rc;
-    if ((rc = check_flags(h, s))) return rc;
-    HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
-    return MUMMU_OK;
+    return download_rows(h, out, h->xout, bytes, s, true);
 }
 
 int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const float *xs, int64_t n, int top_k, float *out) {
@@ -841,14 +890,12 @@ int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_
     if ((rc = ensure_ws(h, rows, rows, 0))) return rc;
     hipStream_t s = h->stream;
     const size_t bytes = sizeof(float) * (size_t)rows * (size_t)hidden;
-    HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, s));
+    if ((rc = upload_rows(h, h->xin, x, bytes, s))) return rc;
     ExpertBanks b = banks_of(h, h->layers[layer]);
     if (is_quant_type(b.gate_type)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(h->xin, (int)rows, hidden, h->xq, s));
     LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, h->xin, h->xq, nullptr, (int)rows, 1, expert, h->act, h->actq, h->flags, s));
     LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->actq, nullptr, (int)rows, 1, expert, h->y, s));
-    HIPCHK(h, hipStreamSynchronize(s));
-    HIPCHK(h, hipMemcpy(out, h->y, bytes, hipMemcpyDeviceToHost));
-    return MUMMU_OK;
+    return download_rows(h, out, h->y, bytes, s, false);
 }
 
 int mummu_moe_take_hits(mummu_moe *h, int layer, uint64_t *hits) {
@@ -874,11 +921,9 @@ int mummu_moe_stack_forward(mummu_moe *h, const float *x, int64_t n, int top_k, 
     if (!x || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
     if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
     const size_t bytes = sizeof(float) * (size_t)n * (size_t)h->cfg.hidden_size;
-    HIPCHK(h, hipMemcpyAsync(h->xin, x, bytes, hipMemcpyHostToDevice, h->stream));
+    if ((rc = upload_rows(h, h->xin, x, bytes, h->stream))) return rc;
     if ((rc = stack_impl(h, h->xin, n, top_k, norm, h->xout, h->stream, ids))) return rc;
-    if ((rc = check_flags(h, h->stream))) return rc;
-    HIPCHK(h, hipMemcpy(out, h->xout, bytes, hipMemcpyDeviceToHost));
-    return MUMMU_OK;
+    return download_rows(h, out, h->xout, bytes, h->stream, true);
 }
 
 int mummu_dequantize(int type, const void *bytes, size_t nbytes, float *out) {
