@@ -253,10 +253,11 @@ int flags_to_status(mummu_moe *h, const int32_t *f) {
 // synchronisation instead of one per copy.  Larger calls copy straight from / to the caller's memory.
 constexpr size_t kPinIO = 256 * 1024;
 
-int upload_rows(mummu_moe *h, float *dev, const float *host, size_t bytes, hipStream_t s) {
-    if (h->pin && bytes <= kPinIO) {
-        memcpy(h->pin, host, bytes);
-        HIPCHK(h, hipMemcpyAsync(dev, h->pin, bytes, hipMemcpyHostToDevice, s));
+// (pin_offset: where in the input half this upload is staged - a call with two inputs gives each its own place)
+int upload_rows(mummu_moe *h, float *dev, const float *host, size_t bytes, hipStream_t s, size_t pin_offset = 0) {
+    if (h->pin && pin_offset + bytes <= kPinIO) {
+        memcpy(h->pin + pin_offset, host, bytes);
+        HIPCHK(h, hipMemcpyAsync(dev, h->pin + pin_offset, bytes, hipMemcpyHostToDevice, s));
     } else {
         HIPCHK(h, hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, s));
     }
@@ -862,17 +863,25 @@ int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const f
 
 int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const float *xs, int64_t n, int top_k, float *out) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    int rc;
-    {
-        std::lock_guard<std::mutex> lock(h->mu);
-        if ((rc = check_layer(h, layer))) return rc;
-    }
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
     if (n <= 0) return n < 0 ? fail(h, MUMMU_ERR_SHAPE, "negative token count") : MUMMU_OK;
-    if (top_k < 1 || top_k > h->cfg.num_experts) return check_topk(h, top_k, h->cfg.num_experts);
-    std::vector<int32_t> ids((size_t)(n * top_k));
-    std::vector<float> w((size_t)(n * top_k));
-    if ((rc = mummu_route_logits(h, router_logits, n, h->cfg.num_experts, top_k, MUMMU_ROUTER_QWEN4EXP, 1, ids.data(), w.data()))) return rc;
-    return mummu_moe_apply_routing(h, layer, ids.data(), w.data(), xs, n, top_k, out);
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if (!router_logits || !xs || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
+    // route on the device from the caller's logits (experts.rs:502-582), then the experts: one
+    // upload of each input, one synchronisation at the end
+    const Layer &L = h->layers[layer];
+    const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
+    hipStream_t s = h->stream;
+    const size_t lbytes = sizeof(float) * (size_t)n * (size_t)E, xbytes = sizeof(float) * (size_t)n * (size_t)H;
+    if ((rc = upload_rows(h, h->logits, router_logits, lbytes, s, 0))) return rc;
+    if ((rc = upload_rows(h, h->xin, xs, xbytes, s, lbytes <= kPinIO ? (lbytes + 63) / 64 * 64 : kPinIO))) return rc;
+    LAUNCH(h, K_ROUTE_TOPK, s,
+           launch_route_topk(h->logits, (int)n, E, top_k, MUMMU_ROUTER_QWEN4EXP, 1, h->ids, h->weights, L.hits, h->flags, s));
+    if ((rc = run_experts(h, L, h->xin, false, n, top_k, nullptr, h->xout, s))) return rc;
+    return download_rows(h, out, h->xout, xbytes, s, true);
 }
 
 int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden, float *out) {
