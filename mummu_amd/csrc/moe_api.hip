@@ -878,6 +878,22 @@ int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const 
     const size_t lbytes = sizeof(float) * (size_t)n * (size_t)E, xbytes = sizeof(float) * (size_t)n * (size_t)H;
     if ((rc = upload_rows(h, h->logits, router_logits, lbytes, s, 0))) return rc;
     if ((rc = upload_rows(h, h->xin, xs, xbytes, s, lbytes <= kPinIO ? (lbytes + 63) / 64 * 64 : kPinIO))) return rc;
+    const ExpertBanks b = banks_of(h, L);
+    if (n <= 8 && n < batched_from(h, L) && is_quant_type(L.gate_type) && H % 64 == 0 && gate_up_routes_inline(b, top_k) &&
+        down_combine_supported(b, top_k)) {
+        // few tokens: the decode pair, gate/up routing by itself from the uploaded logits
+        RouteInline route;
+        route.logits = h->logits;
+        route.flavour = MUMMU_ROUTER_QWEN4EXP;
+        route.norm = 1;
+        route.ids = h->ids;
+        route.weights = h->weights;
+        route.hits = L.hits;
+        LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(h->xin, (int)n, H, h->xq, s));
+        LAUNCH(h, K_GATE_UP, s, launch_gate_up_routed(b, h->xq, route, (int)n, top_k, h->actq, h->flags, s));
+        LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, top_k, nullptr, h->xout, s));
+        return download_rows(h, out, h->xout, xbytes, s, true);
+    }
     LAUNCH(h, K_ROUTE_TOPK, s,
            launch_route_topk(h->logits, (int)n, E, top_k, MUMMU_ROUTER_QWEN4EXP, 1, h->ids, h->weights, L.hits, h->flags, s));
     if ((rc = run_experts(h, L, h->xin, false, n, top_k, nullptr, h->xout, s))) return rc;
