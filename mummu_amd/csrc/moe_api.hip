@@ -253,6 +253,10 @@ int flags_to_status(mummu_moe *h, const int32_t *f) {
 // synchronisation instead of one per copy.  Larger calls copy straight from / to the caller's memory.
 constexpr size_t kPinIO = 256 * 1024;
 
+// The routing of n*k pairs back to the caller (ids, weights; logits too when asked for) under one
+// synchronisation, with the error flags.
+int download_routing(mummu_moe *h, int32_t *ids, float *weights, size_t pairs, float *logits, size_t n_logits, hipStream_t s);
+
 // (pin_offset: where in the input half this upload is staged - a call with two inputs gives each its own place)
 int upload_rows(mummu_moe *h, float *dev, const float *host, size_t bytes, hipStream_t s, size_t pin_offset = 0) {
     if (h->pin && pin_offset + bytes <= kPinIO) {
@@ -285,6 +289,31 @@ int download_rows(mummu_moe *h, float *host, const float *dev, size_t bytes, hip
         HIPCHK(h, hipStreamSynchronize(s));
     }
     HIPCHK(h, hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost));
+    return MUMMU_OK;
+}
+
+int download_routing(mummu_moe *h, int32_t *ids, float *weights, size_t pairs, float *logits, size_t n_logits, hipStream_t s) {
+    const size_t ib = sizeof(int32_t) * pairs, wb = sizeof(float) * pairs, lb = logits ? sizeof(float) * n_logits : 0;
+    if (h->pin && ib + wb + lb <= kPinIO) {
+        uint8_t *p = h->pin + kPinIO;
+        int32_t *pf = (int32_t *)(h->pin + 2 * kPinIO);
+        HIPCHK(h, hipMemcpyAsync(pf, h->flags, sizeof(int32_t) * kFlagWords, hipMemcpyDeviceToHost, s));
+        HIPCHK(h, hipMemcpyAsync(p, h->ids, ib, hipMemcpyDeviceToHost, s));
+        HIPCHK(h, hipMemcpyAsync(p + ib, h->weights, wb, hipMemcpyDeviceToHost, s));
+        if (lb) HIPCHK(h, hipMemcpyAsync(p + ib + wb, h->logits, lb, hipMemcpyDeviceToHost, s));
+        HIPCHK(h, hipStreamSynchronize(s));
+        const int rc = flags_to_status(h, pf);
+        if (rc) return rc;
+        memcpy(ids, p, ib);
+        memcpy(weights, p + ib, wb);
+        if (lb) memcpy(logits, p + ib + wb, lb);
+        return MUMMU_OK;
+    }
+    const int rc = check_flags(h, s);
+    if (rc) return rc;
+    HIPCHK(h, hipMemcpy(ids, h->ids, ib, hipMemcpyDeviceToHost));
+    HIPCHK(h, hipMemcpy(weights, h->weights, wb, hipMemcpyDeviceToHost));
+    if (lb) HIPCHK(h, hipMemcpy(logits, h->logits, lb, hipMemcpyDeviceToHost));
     return MUMMU_OK;
 }
 
@@ -788,11 +817,7 @@ int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_
     LAUNCH(h, K_ROUTER_LOGITS, s, launch_router_logits(h->xin, L.router, L.router_type, h->logits, (int)n, H, E, QAct(), s));
     LAUNCH(h, K_ROUTE_TOPK, s,
            launch_route_topk(h->logits, (int)n, E, top_k, h->cfg.router_flavour, norm, h->ids, h->weights, nullptr, h->flags, s));
-    if (logits) HIPCHK(h, hipMemcpyAsync(logits, h->logits, sizeof(float) * (size_t)n * E, hipMemcpyDeviceToHost, s));
-    if ((rc = check_flags(h, s))) return rc;
-    HIPCHK(h, hipMemcpy(ids, h->ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
-    HIPCHK(h, hipMemcpy(weights, h->weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
-    return MUMMU_OK;
+    return download_routing(h, ids, weights, (size_t)(n * top_k), logits, (size_t)n * (size_t)E, s);
 }
 
 int mummu_route_logits(mummu_moe *h, const float *logits, int64_t n, int n_experts, int top_k, int flavour, int norm,
