@@ -21,11 +21,12 @@ hipError_t launch_dequantize(int type, const uint8_t *bytes, size_t nblocks, flo
 // logits[t, e] = <x[t, :], W[e, :]> in the fixed 512-partial order.  W row-major [E, H].
 // xq.hi != nullptr: also the 16-bit quantization of x for the integer expert products.
 // norm_gamma != nullptr (only where router_logits_can_norm says so): x is the raw residual stream and
-// both outputs are computed from RmsNorm(x) = (x * r) * gamma, bit for bit what launch_rmsnorm writes.
+// both outputs are computed from RmsNorm(x) = (x * r) * gamma, bit for bit what launch_rmsnorm writes;
+// xnorm_out (nullable, only with norm_gamma) also receives those normalised rows.
 bool router_logits_can_norm(const float *x, const void *w, const float *gamma, int n, int hidden);
 hipError_t launch_router_logits(const float *x, const void *w, int wtype, float *logits, int n, int hidden,
                                 int n_experts, QAct xq, hipStream_t s, const float *norm_gamma = nullptr,
-                                float norm_eps = 0.0f);
+                                float norm_eps = 0.0f, float *xnorm_out = nullptr);
 // softmax -> top-k -> (re)normalise per token; one wave per token.
 //   ids/weights [n, k] in slot order; hits (nullable) [E] += rows routed; flags see above.
 hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, int flavour, int norm,

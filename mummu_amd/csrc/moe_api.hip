@@ -436,7 +436,7 @@ bool decode_three_launches(const mummu_moe *h, const Layer &L, int64_t n, int k)
 // norm_gamma != nullptr (only where decode_three_launches holds): x is the raw residual stream and the
 // first launch applies the layer's RmsNorm itself.
 int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
-                hipStream_t s, const float *norm_gamma = nullptr) {
+                hipStream_t s, const float *norm_gamma = nullptr, float *xnorm_out = nullptr) {
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
     // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
@@ -454,7 +454,7 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
     } else {
         // few tokens: the router rows are spread over as many CUs as there are experts
         LAUNCH(h, K_ROUTER_LOGITS, s,
-               launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s, norm_gamma, h->cfg.rms_norm_eps));
+               launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s, norm_gamma, h->cfg.rms_norm_eps, xnorm_out));
         const ExpertBanks b = banks_of(h, L);
         if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
             // ... and the gate/up kernel routes by itself: one launch less on the decode path
@@ -496,7 +496,9 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
                  hipStream_t s, const float *norm_gamma = nullptr) {
     const Layer &L = h->layers[layer];
     if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s, norm_gamma);
-    if (norm_gamma) return fail(h, MUMMU_ERR_ARG, "fused RmsNorm with a shared expert");
+    // with the RmsNorm inside the router launch the shared expert reads the normalised rows that launch leaves in h2
+    const float *x_raw = x;
+    if (norm_gamma) x = h->h2;
     if (n > h->sh_ws_tokens) return fail(h, MUMMU_ERR_TOKENS, "shared-expert workspace is smaller than the call");
     const int H = h->cfg.hidden_size;
     ExpertBanks b;
@@ -512,7 +514,8 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     const int sh_from = !grouped_gemm_supported(b) ? 0x7fffffff : (grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16);
     // (one expert makes few workgroups: tiles x 128-row slabs.  Measured at H 2048, shared inter 2048, Q4_K: the
     // per-token kernels cost 68 us at 64 tokens and 396 us at 512, the GEMM pair about 145 us at either)
-    int rc = routed_impl(h, layer, x, n, k, norm, nullptr, out, s);
+    int rc = norm_gamma ? routed_impl(h, layer, x_raw, n, k, norm, nullptr, out, s, norm_gamma, h->h2)
+                        : routed_impl(h, layer, x, n, k, norm, nullptr, out, s);
     if (rc) return rc;
     if (n >= sh_from && n >= 192) {
         // many tokens: the shared expert is one more grouped GEMM pair, every row in order on expert 0
@@ -562,7 +565,7 @@ int stack_impl(mummu_moe *h, const float *x, int64_t n, int k, int norm, float *
         float *dst = l == nl - 1 ? out : h->resid[l & 1];
         const Layer &L = h->layers[l];
         int rc;
-        if (!L.sh_loaded && decode_three_launches(h, L, n, k) && router_logits_can_norm(src, L.router, L.gamma, (int)n, H)) {
+        if (decode_three_launches(h, L, n, k) && router_logits_can_norm(src, L.router, L.gamma, (int)n, H)) {
             // decode: the router launch normalises the row it already holds; no launch of its own
             rc = forward_impl(h, l, src, n, k, norm, src, dst, s, L.gamma);
         } else {

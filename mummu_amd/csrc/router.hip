@@ -32,7 +32,8 @@ template <int WT, bool VEC, bool NORM = false>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x, const void *__restrict__ w,
                                                             float *__restrict__ logits, int n, int hidden,
                                                             int n_experts, QAct xq, int tokens_per_block,
-                                                            const float *__restrict__ gamma, float eps) {
+                                                            const float *__restrict__ gamma, float eps,
+                                                            float *__restrict__ xnorm_out) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int e = blockIdx.y * (blockDim.x >> 6) + wave;
@@ -112,6 +113,17 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
                 xb[c].w = __fmul_rn(__fmul_rn(xb[c].w, r), gb[c].w);
             }
         }
+        if (NORM && xnorm_out != nullptr && blockIdx.y == 0 && wave == 0) {
+            // the normalised row itself, for whoever reads float activations after this launch
+            float *xo = xnorm_out + (size_t)t0 * (size_t)hidden;
+#pragma unroll
+            for (int c = 0; c < kRouterChunks; c++) {
+                const int base = lane * 8 + 512 * c;
+                if (base >= hidden) continue;
+                ((float4 *)(xo + base))[0] = xa[c];
+                ((float4 *)(xo + base))[1] = xb[c];
+            }
+        }
         quantize_share(r);  // its loads join the ones above; its stores do not hold them back
 #pragma unroll
         for (int c = 0; c < kRouterChunks; c++) {
@@ -165,10 +177,12 @@ bool router_logits_can_norm(const float *x, const void *w, const float *gamma, i
 }
 
 hipError_t launch_router_logits(const float *x, const void *w, int wtype, float *logits, int n, int hidden,
-                                int n_experts, QAct xq, hipStream_t s, const float *norm_gamma, float norm_eps) {
+                                int n_experts, QAct xq, hipStream_t s, const float *norm_gamma, float norm_eps,
+                                float *xnorm_out) {
     if (n <= 0) return hipSuccess;
     if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
     if (norm_gamma && !router_logits_can_norm(x, w, norm_gamma, n, hidden)) return hipErrorInvalidValue;
+    if (xnorm_out && (!norm_gamma || ((uintptr_t)xnorm_out & 15))) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
     // few tokens: one wave per workgroup so the expert rows spread over as many CUs as possible
     const int waves = n <= 8 ? 1 : 4;
@@ -180,13 +194,13 @@ hipError_t launch_router_logits(const float *x, const void *w, int wtype, float 
     do {                                                                                                              \
         if (norm_gamma)                                                                                               \
             launch_kernel(router_logits_kernel<WT, true, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb, \
-                          norm_gamma, norm_eps);                                                                      \
+                          norm_gamma, norm_eps, xnorm_out);                                                           \
         else if (vec)                                                                                                 \
             launch_kernel(router_logits_kernel<WT, true>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb, \
-                          (const float *)nullptr, 0.0f);                                                              \
+                          (const float *)nullptr, 0.0f, (float *)nullptr);                                                              \
         else                                                                                                          \
             launch_kernel(router_logits_kernel<WT, false>, grid, block, 0, s, x, w, logits, n, hidden, n_experts, xq, tpb, \
-                          (const float *)nullptr, 0.0f);                                                              \
+                          (const float *)nullptr, 0.0f, (float *)nullptr);                                                              \
     } while (0)
     switch (wtype) {
     case T_F32: MUMMU_LAUNCH_ROUTER(T_F32); break;

@@ -213,3 +213,24 @@ def test_a_random_block_with_a_shared_expert_matches_the_composition(seed):
     floor = 1e-2 * np.median(mag)
     err = orc.rel_err(got, full, np.maximum(mag, floor)).max()
     assert err <= tol, f"{what}: max relative error {err:.3e} > {tol}"
+
+
+@pytest.mark.parametrize("sgt", [M.Q8_0, M.F32], ids=["quantized-shared", "float-shared"])
+def test_decode_stack_with_a_shared_expert_and_the_norm_inside_the_router_launch(sgt):
+    # up to 8 tokens the stack normalises inside the router launch and hands the normalised rows to the shared
+    # expert; from 9 tokens on RmsNorm is a launch of its own.  A token must get the same bits either way.
+    H, I, IS, E, k, L = 512, 128, 192, 8, 2, 3
+    g = np.random.Generator(np.random.PCG64(5))
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=12, rms_norm_eps=1e-6) as m:
+        for l in range(L):
+            gamma = (1.0 + 0.2 * g.standard_normal(H)).astype(np.float32)
+            m.load_layer(l, normal((E, H), 10 + l, 0.05), M.F32, bank(M.Q4_K, [H, I, E], 20 + l), M.Q4_K,
+                         bank(M.Q4_K, [H, I, E], 30 + l), M.Q4_K, bank(M.Q8_0, [I, H, E], 40 + l), M.Q8_0, gamma)
+            m.load_shared_expert(l, IS, bank(sgt, [H, IS, 1], 50 + l), sgt, bank(sgt, [H, IS, 1], 60 + l), sgt,
+                                 bank(sgt, [IS, H, 1], 70 + l), sgt, normal((H,), 80 + l, 0.2))
+        x = normal((12, H), 91, 2.0)
+        many, many_ids = m.stack_forward(x, k, True, return_ids=True)
+        for n in (1, 4, 8):
+            few, few_ids = m.stack_forward(x[:n], k, True, return_ids=True)
+            assert np.array_equal(few_ids, many_ids[:, :n])
+            assert np.array_equal(few.view(np.uint32), many[:n].view(np.uint32)), f"{n} tokens"
