@@ -407,6 +407,116 @@ __device__ inline void expand_q(const RawQ<WT> &r, int k0, int half, uint32_t (&
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// F32 banks: v_mfma_f32_32x32x2_f32, everything stays f32 (tolerance class 1e-5)
+// ---------------------------------------------------------------------------------------
+constexpr int kFK = 32;          // K step (floats): a row's step is 128 B = 8 lanes x 16 B, as for the halfs
+constexpr int kLdsF = kFK + 4;   // LDS row (floats)
+
+// Same tiles and work list as the f16 kernel.  One MFMA multiplies two K values: lane half g supplies
+// k = 16 g + j of the step for j = 0..15, so a lane's operands for four consecutive instructions are
+// one 16-byte LDS read.
+// GATE_UP: A = x (gathered by token through `sorted`), two weight matrices, act_out[pos, n] = silu(g) * u.
+// else   : A = the f32 activation rows in sorted order, one matrix, y[pos, n] = the sum.
+template <bool GATE_UP, int MT>
+__global__ __launch_bounds__(256) void grouped_gemm_f32_kernel(
+    const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const float *__restrict__ a_in,
+    const int32_t *__restrict__ sorted, int k_slots, const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles,
+    int in_dim, int out_dim, float *__restrict__ act_out, float *__restrict__ y_out) {
+    constexpr int NB = GATE_UP ? 2 : 1;
+    constexpr int BM = 32 * MT;
+    __shared__ __attribute__((aligned(16))) float s_a[BM][kLdsF];
+    __shared__ __attribute__((aligned(16))) float s_b[NB][kBN][kLdsF];
+
+    int tile, slab;
+    if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
+    const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int n0 = slab * kBN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t row_bytes = (size_t)in_dim * 4;
+
+    // weight tile: thread -> 16-byte chunk tid%8 of rows tid/8 + 32*i; activation tile alike, MT passes
+    const int chunk = tid & 7;
+    const uint8_t *b_ptr[NB][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = (tid >> 3) + 32 * i;
+        const int b_out = n0 + r < out_dim ? n0 + r : out_dim - 1;  // clamped; never stored
+        b_ptr[0][i] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)chunk * 16;
+        if (GATE_UP) b_ptr[NB - 1][i] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)chunk * 16;
+    }
+    const float *a_src[MT];
+#pragma unroll
+    for (int p = 0; p < MT; p++) {
+        // rows past the tile's end read the tile's last row: their products are never stored
+        const int r = 32 * p + (tid >> 3) < rows ? 32 * p + (tid >> 3) : rows - 1;
+        const int src = GATE_UP ? sorted[p0 + r] / k_slots : p0 + r;
+        a_src[p] = a_in + (size_t)src * (size_t)in_dim + chunk * 4;
+    }
+
+    float16v acc[NB][MT];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
+
+    f32x4 rb[NB][4], ra[MT];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) rb[b][i] = *(const f32x4 *)(b_ptr[b][i] + (size_t)k0 * 4);
+#pragma unroll
+        for (int p = 0; p < MT; p++) ra[p] = *(const f32x4 *)(a_src[p] + k0);
+    };
+    fetch(0);
+    const int col = 32 * wave + (lane & 31), g = lane >> 5;
+    for (int k0 = 0; k0 < in_dim; k0 += kFK) {
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) *(f32x4 *)&s_b[b][(tid >> 3) + 32 * i][chunk * 4] = rb[b][i];
+#pragma unroll
+        for (int p = 0; p < MT; p++) *(f32x4 *)&s_a[32 * p + (tid >> 3)][chunk * 4] = ra[p];
+        __syncthreads();
+        if (k0 + kFK < in_dim) fetch(k0 + kFK);
+#pragma unroll
+        for (int jq = 0; jq < 4; jq++) {
+            f32x4 bv[NB];
+#pragma unroll
+            for (int b = 0; b < NB; b++) bv[b] = *(const f32x4 *)&s_b[b][col][16 * g + 4 * jq];
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const f32x4 av = *(const f32x4 *)&s_a[32 * m + (lane & 31)][16 * g + 4 * jq];
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int b = 0; b < NB; b++) acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q], bv[b][q], acc[b][m], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    const int n = n0 + col;
+    if (n < out_dim) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = 32 * m + acc_row(r, lane);
+                if (row < rows) {
+                    const size_t o = (size_t)(p0 + row) * (size_t)out_dim + (size_t)n;
+                    if (GATE_UP) act_out[o] = __fmul_rn(det_silu(acc[0][m][r]), acc[NB - 1][m][r]);
+                    else y_out[o] = acc[0][m][r];
+                }
+            }
+        }
+    }
+}
+
 template <bool GATE_UP, int MT, int KS>
 struct QTileLds {
     static constexpr int NB = GATE_UP ? 2 : 1;
@@ -689,7 +799,8 @@ bool grouped_gemm_quantized(const ExpertBanks &b) {
 }
 
 bool grouped_gemm_supported(const ExpertBanks &b) {
-    const bool f16 = (b.gate_type == T_F16 || b.gate_type == T_BF16) && b.up_type == b.gate_type && b.down_type == b.gate_type;
+    const bool f16 = (b.gate_type == T_F16 || b.gate_type == T_BF16 || b.gate_type == T_F32) && b.up_type == b.gate_type &&
+                     b.down_type == b.gate_type;
     return (f16 || grouped_gemm_quantized(b)) && b.hidden % kBK == 0 && b.inter % kBK == 0;
 }
 
@@ -698,7 +809,7 @@ bool grouped_gemm_supported(const ExpertBanks &b) {
 // plus its spread (binomial: about +-sqrt(avg) per expert, 3.5 sigma here) when that fits; the f16
 // kernel goes up to 128 rows, the int8 kernel (more registers per row) to 64.
 int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts) {
-    const int max_rows = grouped_gemm_quantized(b) ? 64 : 128;
+    const int max_rows = (grouped_gemm_quantized(b) || b.gate_type == T_F32) ? 64 : 128;
     const double avg = (double)n_assign / (double)n_experts;
     const int want = (int)(avg + 3.5 * __builtin_sqrt(avg) + 1.0);
     if (want > max_rows) return 64;  // several full tiles per expert whatever the size: 64 rows measured best
@@ -730,6 +841,22 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
     return hipGetLastError();
 }
 
+template <bool GATE_UP>
+static hipError_t launch_gemm_f32(const uint8_t *w0, const uint8_t *w1, const float *a_in, const int32_t *sorted, int k_slots,
+                                  const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
+                                  int out_dim, float *act_out, float *y_out, hipStream_t s) {
+    dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
+    if (tile_rows == 64)
+        launch_kernel(grouped_gemm_f32_kernel<GATE_UP, 2>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
+                      out_dim, act_out, y_out);
+    else if (tile_rows == 32)
+        launch_kernel(grouped_gemm_f32_kernel<GATE_UP, 1>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, in_dim,
+                      out_dim, act_out, y_out);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 template <bool GATE_UP, bool BF16>
 static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const float *x, const _Float16 *act_in,
                                   const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
@@ -752,8 +879,11 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const fl
 
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
-                               QAct64 actq, hipStream_t s) {
+                               float *act32, QAct64 actq, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (b.gate_type == T_F32)
+        return launch_gemm_f32<true>(b.gate, b.up, x, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden, b.inter, act32,
+                                     nullptr, s);
     if (b.gate_type == T_F16)
         return launch_gemm_f16<true, false>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
                                             b.inter, (_Float16 *)act16, nullptr, s);
@@ -778,9 +908,12 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     }
 }
 
-hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, int n_assign, const int32_t *tiles,
-                            const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s) {
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, int n_assign,
+                            const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (b.down_type == T_F32)
+        return launch_gemm_f32<false>(b.down, nullptr, act32, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter, b.hidden,
+                                      nullptr, y, s);
     const bool few_rows = n_assign <= 64 * b.n_experts;  // an expert's rows fit one tile, on average
     if (b.down_type == T_F16)
         return launch_gemm_f16<false, false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,

@@ -114,7 +114,8 @@ hipError_t launch_identity_tiles(int n, int tile_rows, int32_t *sorted, int32_t 
 
 // gemm.hip ----------------------------------------------------------------------------
 // Grouped GEMMs over the dispatch-sorted assignments on the matrix cores (hidden and inter
-// multiples of 64): F16 and BF16 banks on the f16 units (act16: f16 [A, inter] in sorted order), every
+// multiples of 64): F16 and BF16 banks on the f16 units (act16: f16 [A, inter] in sorted order), F32 banks on
+// the f32 units (act32: f32 [A, inter]), every
 // block-quantized type on the int8 units against 16-bit activations (xq: tokens x hidden, actq:
 // A x inter in sorted order; gate/up and down may differ in type).
 bool grouped_gemm_supported(const ExpertBanks &b);
@@ -124,8 +125,8 @@ int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts);
 hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s);
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
-                               QAct64 actq, hipStream_t s);
-hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, QAct64 actq, int n_assign, const int32_t *tiles,
-                            const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s);
+                               float *act32, QAct64 actq, hipStream_t s);
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, int n_assign,
+                            const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s);
 
 }  // namespace mummu

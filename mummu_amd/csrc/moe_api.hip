@@ -78,8 +78,8 @@ struct mummu_moe {
     void *act16 = nullptr;       // f16 [pairs, inter]
     int max_tiles = 0;
     // batches at least this large take dispatch + grouped GEMM (measured crossovers on the OLMoE shape:
-    // the float decode kernels lose from 7 tokens on, the integer ones from 19)
-    int gemm_min_f16 = 7, gemm_min_quant = 19;
+    // the 16-bit float decode kernels lose from 7 tokens on, the f32 ones from 10, the integer ones from 19)
+    int gemm_min_f16 = 7, gemm_min_quant = 19, gemm_min_f32 = 10;
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
@@ -387,6 +387,7 @@ int check_topk(mummu_moe *h, int top_k, int n_experts) {
 int batched_from(const mummu_moe *h, const Layer &L) {
     const ExpertBanks b = banks_of(h, L);
     if (!grouped_gemm_supported(b)) return 0x7fffffff;
+    if (b.gate_type == T_F32) return h->gemm_min_f32;
     return grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16;
 }
 
@@ -405,9 +406,9 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
                launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch,
                                count_hits ? L.hits : nullptr, h->flags, s));
         LAUNCH(h, K_GEMM_GATE_UP, s,
-               launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, actq64, s));
+               launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, h->act, actq64, s));
         LAUNCH(h, K_GEMM_DOWN, s,
-               launch_gemm_down(b, h->act16, actq64, na, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
+               launch_gemm_down(b, h->act16, h->act, actq64, na, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
         LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, h->inv, (int)n, k, b.hidden, residual, out, s));
         return MUMMU_OK;
     }
@@ -511,7 +512,8 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
     b.hidden = H;
     b.inter = L.sh_inter;
     b.n_experts = 1;
-    const int sh_from = !grouped_gemm_supported(b) ? 0x7fffffff : (grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16);
+    const int sh_from = !grouped_gemm_supported(b) ? 0x7fffffff
+                        : (b.gate_type == T_F32 ? h->gemm_min_f32 : (grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16));
     // (one expert makes few workgroups: tiles x 128-row slabs.  Measured at H 2048, shared inter 2048, Q4_K: the
     // per-token kernels cost 68 us at 64 tokens and 396 us at 512, the GEMM pair about 145 us at either)
     int rc = norm_gamma ? routed_impl(h, layer, x_raw, n, k, norm, nullptr, out, s, norm_gamma, h->h2)
@@ -527,9 +529,9 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
         if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, H, xq64, s));
         LAUNCH(h, K_SHARED, s,
                launch_gemm_gate_up(b, x, xq64, h->sh_sorted, 1, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_act16,
-                                   actq64, s));
+                                   h->sh_act, actq64, s));
         LAUNCH(h, K_SHARED, s,
-               launch_gemm_down(b, h->sh_act16, actq64, (int)n, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_y, s));
+               launch_gemm_down(b, h->sh_act16, h->sh_act, actq64, (int)n, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_y, s));
     } else {
         // the routed decode kernels leave x in the 16-bit decode layout when their own banks are quantized;
         // otherwise (float routed banks, or the batched path's layout) it is made here
@@ -616,7 +618,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
     if (const char *e = getenv("MUMMU_GEMM_MIN_TOKENS")) {
         const int v = atoi(e);
-        if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = v;
+        if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = h->gemm_min_f32 = v;
     }
     h->layers.resize((size_t)cfg->num_layers);
     auto bail = [&](int rc) {

@@ -19,8 +19,8 @@ def normal(shape, seed, std=1.0):
 
 
 def banks_for(kind, H, I, E, seed):
-    if kind in ("F16", "BF16"):
-        t, ot = (M.F16, orc.F16) if kind == "F16" else (M.BF16, orc.BF16)
+    if kind in ("F16", "BF16", "F32"):
+        t, ot = {"F16": (M.F16, orc.F16), "BF16": (M.BF16, orc.BF16), "F32": (M.F32, orc.F32)}[kind]
         mk = lambda i, o, s: synth.encode_float(normal(E * o * i, s, 0.05), t)
         return mk(H, I, seed), mk(H, I, seed + 1), mk(I, H, seed + 2), t, ot
     t, ot = {"Q8_0": (M.Q8_0, orc.Q8_0), "Q4_K": (M.Q4_K, orc.Q4_K)}[kind]
@@ -37,6 +37,8 @@ CASES = [
     ("F16", 1024, 512, 16, 4, 1027),  # 257 per expert -> several 64-row tiles, 5 dispatch chunks, odd token count
     ("BF16", 512, 256, 8, 2, 130),    # bf16 weights become halfs on the way into LDS
     ("BF16", 1024, 512, 16, 4, 515),
+    ("F32", 512, 256, 8, 2, 77),      # f32 matrix cores, everything f32: held to 1e-5
+    ("F32", 1024, 512, 16, 4, 515),
     ("Q8_0", 512, 256, 8, 2, 77),
     ("Q8_0", 1024, 512, 16, 4, 515),
     ("Q4_K", 512, 256, 8, 2, 200),
@@ -64,9 +66,10 @@ def test_prefill_matches_the_oracle(kind, H, I, E, k, n):
     assert hits.tolist() == np.bincount(oids.reshape(-1), minlength=E).tolist()
     assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), "the batched path is not deterministic"
     want, mag = orc.moe_ref_f64(banks, oids, ow, x)
+    tol = 1e-5 if kind == "F32" else 2e-3
     err = orc.rel_err(got, want, mag)
-    assert err.max() <= 2e-3, f"max relative error {err.max():.3e}"
-    assert orc.rel_err(one, want[:1], mag[:1]).max() <= 2e-3
+    assert err.max() <= tol, f"max relative error {err.max():.3e}"
+    assert orc.rel_err(one, want[:1], mag[:1]).max() <= tol
 
 
 def test_prefill_with_experts_nobody_picks_and_two_everybody_picks():
