@@ -506,7 +506,7 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
     // enough tokens to fill the chip with independent waves: activations in registers, weight
     // rows streamed (on this path the caller quantizes x separately)
-    if (n > 64 && vec && xq.hi == nullptr && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks) {
+    if (n > 8 && vec && xq.hi == nullptr && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks) {
         // two tokens per wave once there are enough waves to keep every SIMD busy, else one; below a
         // wave per SIMD a token gets a whole workgroup
         const int tt = n > 2048 ? 2 : 1;
