@@ -350,6 +350,18 @@ __device__ inline void k4_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j
     }
 }
 
+// The same for sub-blocks 2c and 2c+1 at once, each pair packed as two bytes (sub-block 2c in byte 0),
+// without a branch.
+__device__ inline void k4_scale_min_both(uint32_t y, uint32_t z, uint32_t w, int c, uint32_t &sc, uint32_t &mn) {
+    const int sh = 16 * (c & 1);
+    const uint32_t a = y >> sh, b = z >> sh, p = w >> sh;
+    const uint32_t lo_sc = a & 0x3F3Fu, lo_mn = b & 0x3F3Fu;
+    const uint32_t hi_sc = (p & 0x0F0Fu) | ((a >> 2) & 0x3030u);
+    const uint32_t hi_mn = ((p >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);
+    sc = c < 2 ? lo_sc : hi_sc;
+    mn = c < 2 ? lo_mn : hi_mn;
+}
+
 // The block's 32 integers as bytes in element order, with weight = scale * byte + offset.
 // Types with one scale per 16 elements return the second half's scale in scale1 (else scale1 =
 // scale).  Bytes are codes 0..31 (unsigned) or, for Q8_0 / Q6_K, signed values.
@@ -601,6 +613,9 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
 
+    // raw registers of the next stage: refilled right after a stage has been expanded into LDS, so the loads fly
+    // under the products.  (A second set, two stages ahead, was measured and bought nothing: with few rows per
+    // expert the launch already moves 3.5 TB/s of 72-byte row pieces.)
     RawQ<WT> rb[NB][NRAW];
     uint4 ra[A_PASSES];
     float ras = 0.0f, ram = 0.0f;
@@ -619,15 +634,48 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
         ras = as_ptr ? as_ptr[k0 >> 6] : 0.0f;
         if (OFFSET) ram = am_ptr ? am_ptr[k0 >> 5] : 0.0f;
     };
-    fetch(0);
 
     const int col = 32 * wave + (lane & 31), g = lane >> 5;
     MUMMU_TIMER_DECL;
-    for (int k0 = 0; k0 < in_dim; k0 += KS * kBK) {
-        MUMMU_TIMER_MARK(0);
-        // registers -> LDS
+    // registers of set S -> LDS
+    auto stage = [&](int k0) {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
+            if constexpr (KS == 2 && SHARED) {
+                // both blocks of this thread's step come out of one 32-byte chunk: header, scale pair and nibble
+                // split are done once (same values, bit for bit, as two expand_q calls)
+                const RawQ<WT> &r = rb[b][0];
+                const int c = ((k0 + kBK * b_half) & 255) >> 6;
+                const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFFu));
+                const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
+                uint32_t scp, mnp;
+                k4_scale_min_both(r.hdr.y, r.hdr.z, r.hdr.w, c, scp, mnp);
+                const uint32_t qw[8] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w, r.q[1].x, r.q[1].y, r.q[1].z, r.q[1].w};
+                uint32_t lo[8], hi[8];
+#pragma unroll
+                for (int w = 0; w < 8; w++) {
+                    lo[w] = qw[w] & 0x0F0F0F0Fu;
+                    hi[w] = (qw[w] >> 4) & 0x0F0F0F0Fu;
+                }
+                if constexpr (WT == T_Q5_K) {
+                    const uint32_t hw[8] = {r.qh[0].x, r.qh[0].y, r.qh[0].z, r.qh[0].w, r.qh[1].x, r.qh[1].y, r.qh[1].z, r.qh[1].w};
+#pragma unroll
+                    for (int w = 0; w < 8; w++) {
+                        lo[w] |= ((hw[w] >> (2 * c)) & 0x01010101u) << 4;
+                        hi[w] |= ((hw[w] >> (2 * c + 1)) & 0x01010101u) << 4;
+                    }
+                }
+                uint4 *dst = (uint4 *)(s_b(b, b_row) + 2 * b_half * 32);
+                dst[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                dst[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+                dst[2] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                dst[3] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+                s_bd[b][b_row][2 * b_half] = __fmul_rn(d, (float)(scp & 0xFFu));
+                s_bd[b][b_row][2 * b_half + 1] = __fmul_rn(d, (float)((scp >> 8) & 0xFFu));
+                s_bm[b][b_row][2 * b_half] = -__fmul_rn(dmin, (float)(mnp & 0xFFu));
+                s_bm[b][b_row][2 * b_half + 1] = -__fmul_rn(dmin, (float)((mnp >> 8) & 0xFFu));
+                continue;
+            }
 #pragma unroll
             for (int hh = 0; hh < NBLK; hh++) {
                 // the block this pass stages: block `blk` (0 .. 2 KS - 1) of the stage
@@ -651,12 +699,8 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
         for (int p = 0; p < A_PASSES; p++) *(uint4 *)(s_a(a_plane, a_row[p]) + a_chunk * 16) = ra[p];
         if (tid < KS * BM) s_as[tid / BM][tid % BM] = ras;
         if (OFFSET && tid < 2 * KS * BM) s_am[tid / (2 * KS)][tid & (2 * KS - 1)] = ram;
-        MUMMU_TIMER_MARK(1);
-        __syncthreads();
-        MUMMU_TIMER_MARK(2);
-        if (k0 + KS * kBK < in_dim) fetch(k0 + KS * kBK);
-        MUMMU_TIMER_MARK(3);
-
+    };
+    auto multiply = [&]() {
         // multiply: wave owns columns 32*wave .. +31
 #pragma unroll
         for (int sub = 0; sub < KS; sub++) {
@@ -737,6 +781,18 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
             }
         }
         }
+    };
+    constexpr int STEP = KS * kBK;
+    fetch(0);
+    for (int k0 = 0; k0 < in_dim; k0 += STEP) {
+        MUMMU_TIMER_MARK(0);
+        stage(k0);
+        MUMMU_TIMER_MARK(1);
+        __syncthreads();
+        MUMMU_TIMER_MARK(2);
+        if (k0 + STEP < in_dim) fetch(k0 + STEP);
+        MUMMU_TIMER_MARK(3);
+        multiply();
         MUMMU_TIMER_MARK(4);
         __syncthreads();
         MUMMU_TIMER_MARK(5);
@@ -830,9 +886,10 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
     // 4096 tokens 410 -> 462 us); never for Q6_K (slower, and it spills).
     constexpr bool shared_raw = WT == T_Q4_K || WT == T_Q5_K;
     const bool ks2 = in_dim % (2 * kBK) == 0 && !gemm_sub16(WT) && (shared_raw || GATE_UP || few_rows);
-#define MUMMU_Q(MT, KS)                                                                                                   \
-    launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, MT, KS>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles, n_tiles, \
-                  in_dim, out_dim, act_out, y_out)
+#define MUMMU_Q(MT, KS)                                                                                             \
+    launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, MT, KS>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles,   \
+                  n_tiles, in_dim, out_dim, act_out, y_out)
+    // small tiles (few rows per expert: the launch is a stream of weights) also keep two stages of loads in flight
     if (tile_rows == 64 && ks2) MUMMU_Q(2, 2);
     else if (tile_rows == 64) MUMMU_Q(2, 1);
     else if (ks2) MUMMU_Q(1, 2);
