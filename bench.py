@@ -77,7 +77,7 @@ def main() -> int:
 
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
-              "(expert-parallel sharding over several GPUs is described in DESIGN.md, not built).", file=sys.stderr)
+              "(sharding the experts over several GPUs is a design note of this library, not built).", file=sys.stderr)
         return 2
 
     from mummu_amd import _lib, moe as M, synth
