@@ -93,6 +93,10 @@ MUMMU_API const char *mummu_moe_last_error(const mummu_moe *h);
  * exactly as the reference asserts, then allocates the workspace on HIP device 0. */
 MUMMU_API int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out);
 MUMMU_API void mummu_moe_destroy(mummu_moe *h);
+/* The configuration the handle was created with (the fields of SparseMoeConfig, nn/moe.rs:42-59, plus
+ * this library's own).  The file loaders below use it to refuse a model file whose geometry is not the
+ * handle's before any payload is read. */
+MUMMU_API int mummu_moe_get_config(const mummu_moe *h, mummu_moe_config *out);
 
 /* The checked load of one block's tensors: `mlp.gate.weight` and
  * `mlp.experts.{gate,up,down}` <- GGUF `ffn_gate_inp`, `ffn_{gate,up,down}_exps`

@@ -348,6 +348,12 @@ class SparseMoe {
     }
 
     uint64_t resident_bytes() const { return mummu_moe_resident_bytes(h_.get()); }
+    /// The configuration the handle was created with.
+    mummu_moe_config config() const {
+        mummu_moe_config c{};
+        mummu_moe_get_config(h_.get(), &c);
+        return c;
+    }
     /// Smallest token count that takes dispatch + grouped GEMM on this layer (INT32_MAX: never).
     int batched_from(int layer = 0) const { return mummu_moe_batched_from(h_.get(), layer); }
 

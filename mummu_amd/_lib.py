@@ -64,6 +64,7 @@ SIGNATURES = {
     "mummu_moe_destroy": (None, [_P]),
     "mummu_moe_load_layer": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P]),
     "mummu_moe_load_shared_expert": (_I, [_P, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I]),
+    "mummu_moe_get_config": (_I, [_P, _P]),
     "mummu_moe_resident_bytes": (C.c_uint64, [_P]),
     "mummu_moe_batched_from": (C.c_int, [_P, C.c_int]),
     "mummu_moe_forward": (_I, [_P, _I, _P, _I64, _I, _I, _P]),

@@ -560,6 +560,21 @@ int mummu_gguf_locate_moe_layer(const mummu_gguf *g, int layer, mummu_gguf_moe_l
 int mummu_moe_load_gguf(mummu_moe *h, mummu_gguf *g, int first_layer, int n_layers) {
     if (!h || !g) return fail(MUMMU_ERR_ARG, "null argument");
     if (first_layer < 0 || n_layers < 1) return fail(MUMMU_ERR_RANGE, "first_layer must be >= 0 and n_layers >= 1");
+    {
+        // the handle reads its banks by its own geometry: a file of another geometry would be read past its tensors
+        mummu_moe_config have, file;
+        int rc = mummu_moe_get_config(h, &have);
+        if (rc) return fail(rc, "the handle's configuration could not be read");
+        if ((rc = mummu_gguf_moe_config(g, &file))) return rc;
+        if (have.hidden_size != file.hidden_size || have.expert_intermediate_size != file.expert_intermediate_size ||
+            have.num_experts != file.num_experts)
+            return fail(MUMMU_ERR_SHAPE, "the handle was created for hidden " + std::to_string(have.hidden_size) + ", intermediate " +
+                                             std::to_string(have.expert_intermediate_size) + ", " + std::to_string(have.num_experts) +
+                                             " experts; the file holds hidden " + std::to_string(file.hidden_size) + ", intermediate " +
+                                             std::to_string(file.expert_intermediate_size) + ", " + std::to_string(file.num_experts) + " experts");
+        if (n_layers > have.num_layers)
+            return fail(MUMMU_ERR_RANGE, std::to_string(n_layers) + " layers do not fit the handle's " + std::to_string(have.num_layers));
+    }
     for (int l = 0; l < n_layers; l++) {
         mummu_gguf_moe_layer at;
         int rc = mummu_gguf_locate_moe_layer(g, first_layer + l, &at);

@@ -781,6 +781,12 @@ int mummu_moe_batched_from(const mummu_moe *h, int layer) {
     return batched_from(h, h->layers[layer]);
 }
 
+int mummu_moe_get_config(const mummu_moe *h, mummu_moe_config *out) {
+    if (!h || !out) return fail(nullptr, MUMMU_ERR_ARG, "null argument");
+    *out = h->cfg;
+    return MUMMU_OK;
+}
+
 uint64_t mummu_moe_resident_bytes(const mummu_moe *h) {
     if (!h) return 0;
     uint64_t total = 0;

@@ -668,6 +668,19 @@ int mummu_moe_load_safetensors(mummu_moe *h, mummu_st *st, int first_layer, int 
     if (!st->have_cfg) return fail(st->cfg_status, st->cfg_error);
     if (first_layer < 0 || n_layers < 1) return fail(MUMMU_ERR_RANGE, "first_layer must be >= 0 and n_layers >= 1");
     const mummu_moe_config &c = st->cfg;
+    {
+        // the handle reads its banks by its own geometry: a checkpoint of another geometry would be read past its buffers
+        mummu_moe_config have;
+        const int rc = mummu_moe_get_config(h, &have);
+        if (rc) return fail(rc, "the handle's configuration could not be read");
+        if (have.hidden_size != c.hidden_size || have.expert_intermediate_size != c.expert_intermediate_size || have.num_experts != c.num_experts)
+            return fail(MUMMU_ERR_SHAPE, "the handle was created for hidden " + std::to_string(have.hidden_size) + ", intermediate " +
+                                             std::to_string(have.expert_intermediate_size) + ", " + std::to_string(have.num_experts) +
+                                             " experts; the checkpoint holds hidden " + std::to_string(c.hidden_size) + ", intermediate " +
+                                             std::to_string(c.expert_intermediate_size) + ", " + std::to_string(c.num_experts) + " experts");
+        if (n_layers > have.num_layers)
+            return fail(MUMMU_ERR_RANGE, std::to_string(n_layers) + " layers do not fit the handle's " + std::to_string(have.num_layers));
+    }
     std::vector<uint8_t> router, banks[3];
     std::vector<float> gamma;
     for (int l = 0; l < n_layers; l++) {

@@ -141,6 +141,11 @@ class GgufFile:
         return {k: (self.tensor_at(getattr(at, k)) if getattr(at, k) >= 0 else None)
                 for k in ("router", "gate", "up", "down", "norm")}
 
+    def load_into(self, moe: SparseMoe, first_layer: int = 0, n_layers: int = 1) -> None:
+        """Layers [first_layer, first_layer + n_layers) of the file into layers 0.. of an existing handle; refused when
+        the handle was created for another geometry than the file's."""
+        self._check(self._lib.mummu_moe_load_gguf(moe._h, self._h, first_layer, n_layers))
+
     def load_moe(self, first_layer: int = 0, n_layers: Optional[int] = None, *, max_tokens: int = 64,
                  router_flavour: int = _lib.ROUTER_SPARSE_MOE) -> SparseMoe:
         """A SparseMoe holding the MoE blocks of layers [first_layer, first_layer + n_layers)."""

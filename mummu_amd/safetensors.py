@@ -100,6 +100,11 @@ class Checkpoint:
         """The fuse's planning pass for one layer: names, completeness, dtypes and shapes."""
         self._check(self._lib.mummu_st_check_moe_layer(self._h, layer))
 
+    def load_into(self, moe: SparseMoe, first_layer: int = 0, n_layers: int = 1) -> None:
+        """Layers [first_layer, first_layer + n_layers) of the checkpoint into layers 0.. of an existing handle; refused
+        when the handle was created for another geometry than the checkpoint's."""
+        self._check(self._lib.mummu_moe_load_safetensors(moe._h, self._h, first_layer, n_layers))
+
     def load_moe(self, first_layer: int = 0, n_layers: Optional[int] = None, *, max_tokens: int = 64) -> SparseMoe:
         cfg = self.moe_config()
         n_layers = cfg.num_layers - first_layer if n_layers is None else n_layers

@@ -96,3 +96,20 @@ def test_a_bank_type_without_a_kernel_is_refused_with_the_tensor_named(tmp_path)
         with pytest.raises(GgufError, match="blk.0") as e:
             f.load_moe(max_tokens=8)
         assert e.value.code == M._lib.ERR_TYPE
+
+
+def test_a_file_of_another_geometry_is_refused_by_an_existing_handle(tmp_path):
+    lw = weights(CASE, 1, 11)
+    path = W.moe_gguf(CASE, lw).write(tmp_path / "m.gguf")
+    with GgufFile.open(path) as f:
+        for H, I, E in [(1024, 256, 8), (512, 512, 8), (512, 256, 16)]:
+            with M.SparseMoe(M.SparseMoeConfig(H, I, E, 2), max_tokens=4) as m:
+                with pytest.raises(GgufError, match="the handle was created for"):
+                    f.load_into(m)
+        with M.SparseMoe(M.SparseMoeConfig(512, 256, 8, 2), max_tokens=4) as m:
+            with pytest.raises(GgufError, match="do not fit the handle"):
+                f.load_into(m, 0, 2)
+            f.load_into(m)
+            x = np.random.Generator(np.random.PCG64(1)).standard_normal((3, 512), dtype=np.float32)
+            with direct(CASE, lw, 4) as ref:
+                assert np.array_equal(m.forward(x, 2, True).view(np.uint32), ref.forward(x, 2, True).view(np.uint32))

@@ -62,3 +62,16 @@ def test_a_short_group_is_refused_before_anything_is_loaded(tmp_path):
             ck.load_moe(max_tokens=8)
         with ck.load_moe(0, 1, max_tokens=8) as m:  # layer 0 alone is whole
             assert m.resident_bytes() > 0
+
+
+def test_a_checkpoint_of_another_geometry_is_refused_by_an_existing_handle(tmp_path):
+    d = SW.write_checkpoint(tmp_path / "ck", SW.olmoe_config(H, I, E, K, L), make_layers(4), "BF16")
+    with Checkpoint.open(d) as ck:
+        for h, i, e in [(2 * H, I, E), (H, 2 * I, E), (H, I, 2 * E)]:
+            with M.SparseMoe(M.SparseMoeConfig(h, i, e, K), num_layers=L, max_tokens=4) as m:
+                with pytest.raises(SafetensorsError, match="the handle was created for"):
+                    ck.load_into(m, 0, L)
+        with M.SparseMoe(M.SparseMoeConfig(H, I, E, K), num_layers=1, max_tokens=4) as m:
+            with pytest.raises(SafetensorsError, match="do not fit the handle"):
+                ck.load_into(m, 0, 2)
+            ck.load_into(m, 1, 1)
