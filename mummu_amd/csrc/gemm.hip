@@ -740,7 +740,24 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                         acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_am[arow][2 * sub + g], s_bm[b][col][2 * sub + g], acc[b][m], 0, 0, 0);
                 }
             }
-        } else {
+        }
+        }
+    };
+    constexpr int STEP = KS * kBK;
+    fetch(0);
+    for (int k0 = 0; k0 < in_dim; k0 += STEP) {
+        MUMMU_TIMER_MARK(0);
+        stage(k0);
+        MUMMU_TIMER_MARK(1);
+        __syncthreads();
+        MUMMU_TIMER_MARK(2);
+        if (k0 + STEP < in_dim) fetch(k0 + STEP);
+        MUMMU_TIMER_MARK(3);
+        if constexpr (SUB16) {
+            // (written out here, not in a lambda like the products of the other types: in a lambda this form
+            // compiles to half as many more registers, spills for gate/up, and measures 10 % slower)
+#pragma unroll
+            for (int sub = 0; sub < KS; sub++) {
             // one weight scale per 16 elements: the K step is four 16-deep integer products
 #pragma unroll
             for (int b = 0; b < NB; b++) {
@@ -779,20 +796,10 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
                     }
                 }
             }
+            }
+        } else {
+            multiply();
         }
-        }
-    };
-    constexpr int STEP = KS * kBK;
-    fetch(0);
-    for (int k0 = 0; k0 < in_dim; k0 += STEP) {
-        MUMMU_TIMER_MARK(0);
-        stage(k0);
-        MUMMU_TIMER_MARK(1);
-        __syncthreads();
-        MUMMU_TIMER_MARK(2);
-        if (k0 + STEP < in_dim) fetch(k0 + STEP);
-        MUMMU_TIMER_MARK(3);
-        multiply();
         MUMMU_TIMER_MARK(4);
         __syncthreads();
         MUMMU_TIMER_MARK(5);
