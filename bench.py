@@ -43,6 +43,7 @@ WORKLOADS = {
     # name: (hidden, inter, experts, top_k, norm, bank type, router type)
     "olmoe_q4k_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q4_K", router="F16"),
     "olmoe_q8_0_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q8_0", router="F16"),
+    "olmoe_q6k_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="Q6_K", router="F16"),
     "olmoe_f16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F16", router="F16"),
     "olmoe_bf16_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="BF16", router="F16"),
     "olmoe_f32_decode": dict(hidden=2048, inter=1024, experts=64, top_k=8, norm=False, bank="F32", router="F16"),

@@ -890,9 +890,10 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
     // whose one load holds both blocks of a step (Q4_K, Q5_K: no extra registers) and for gate/up;
     // the down product of the other types only while an expert's rows fit one tile (with several
     // tiles per expert its second set of raw registers costs more than the barriers saved: Q8_0 at
-    // 4096 tokens 410 -> 462 us); never for Q6_K (slower, and it spills).
+    // 4096 tokens 410 -> 462 us), and for Q6_K only with 32-row tiles (32 tokens 84 -> 72 us, but 512
+    // tokens 138 -> 142 us).
     constexpr bool shared_raw = WT == T_Q4_K || WT == T_Q5_K;
-    const bool ks2 = in_dim % (2 * kBK) == 0 && !gemm_sub16(WT) && (shared_raw || GATE_UP || few_rows);
+    const bool ks2 = in_dim % (2 * kBK) == 0 && (shared_raw || GATE_UP || few_rows) && !(gemm_sub16(WT) && !GATE_UP && tile_rows == 64);
 #define MUMMU_Q(MT, KS)                                                                                             \
     launch_kernel(grouped_gemm_q_kernel<WT, GATE_UP, MT, KS>, grid, block, 0, s, w0, w1, a_in, sorted, k_slots, tiles,   \
                   n_tiles, in_dim, out_dim, act_out, y_out)
