@@ -158,6 +158,11 @@ MUMMU_API int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *id
  * SwiGLU of one expert on rows x hidden f32, row-major in and out. */
 MUMMU_API int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden,
                                float *out);
+/* ExpertExec::gate_energy (nn/moe.rs:411-418, DeviceExpert's at :508-521): per row of x, the sum over the
+ * intermediate width of silu(x . gate_i)^2 - the gate product only, on the stored gate rows dequantized to
+ * f32; the reference's skip mode compares it against a row's total (nn/moe.rs:1494-1522).  energy [rows]. */
+MUMMU_API int mummu_expert_gate_energy(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden,
+                                       float *energy);
 
 /* ExpertPool::take_hits (nn/moe.rs:1562-1564, 857-874): rows served per expert since the
  * last take; hits is uint64[num_experts] and the counters reset. */

@@ -34,6 +34,7 @@
 #pragma once
 
 #include <cstdint>
+#include <limits>
 #include <memory>
 #include <optional>
 #include <stdexcept>
@@ -348,8 +349,8 @@ class SparseMoe {
     }
 
     uint64_t resident_bytes() const { return mummu_moe_resident_bytes(h_.get()); }
-    /// The configuration the handle was created with.
-    mummu_moe_config config() const {
+    /// The configuration as the handle holds it (mummu_moe_get_config).
+    mummu_moe_config handle_config() const {
         mummu_moe_config c{};
         mummu_moe_get_config(h_.get(), &c);
         return c;
@@ -427,18 +428,36 @@ class SparseMoe {
 using SparseMoePerExpert = SparseMoe;
 
 // ExpertExec (nn/moe.rs:348-419), the host-slice seam: SwiGLU of one expert on rows x hidden f32.
+// Tier (tier.rs:66-71): the device an expert is placed on and the stored level it is loaded at (here: the GGML
+// type of its gate bank).
+struct Tier {
+    int device = 0;
+    int precision = MUMMU_F32;
+};
+
 class ExpertExec {
   public:
     virtual ~ExpertExec() = default;
+    virtual Tier tier() const = 0;
     virtual std::vector<float> run(const float *x, size_t rows, size_t hidden) const = 0;
     virtual uint64_t resident_bytes() const = 0;
-    virtual bool is_staged() const { return true; }  // pinned executors are always resident
+    // An executor pinned to its device is always resident there: staging and evicting it are no-ops, as the
+    // trait's defaults are (nn/moe.rs:383-397); there is no second multiply path to fall back to either.
+    virtual void stage(int /*device*/) const {}
+    virtual void evict() const {}
+    virtual bool is_staged() const { return true; }
+    virtual void disable_native() const {}
+    // Per-row energy of the gate activations; the default never skips (nn/moe.rs:411-418).
+    virtual std::vector<float> gate_energy(const float * /*x*/, size_t rows, size_t /*hidden*/) const {
+        return std::vector<float>(rows, std::numeric_limits<float>::infinity());
+    }
 };
 
 // One expert of one layer of a SparseMoe, as an ExpertExec.
 class HipExpert final : public ExpertExec {
   public:
-    HipExpert(SparseMoe moe, int layer, int expert) : moe_(std::move(moe)), layer_(layer), expert_(expert) {}
+    HipExpert(SparseMoe moe, int layer, int expert, int gate_type = MUMMU_F32)
+        : moe_(std::move(moe)), layer_(layer), expert_(expert), gate_type_(gate_type) {}
     std::vector<float> run(const float *x, size_t rows, size_t hidden) const override {
         std::vector<float> out(rows * hidden);
         moe_.check(mummu_expert_run(moe_.handle(), layer_, expert_, x, (int64_t)rows, (int)hidden, out.data()));
@@ -448,10 +467,16 @@ class HipExpert final : public ExpertExec {
         const int e = moe_.config().num_experts * moe_.config().num_layers;
         return e > 0 ? moe_.resident_bytes() / (uint64_t)e : 0;
     }
+    Tier tier() const override { return Tier{0, gate_type_}; }
+    std::vector<float> gate_energy(const float *x, size_t rows, size_t hidden) const override {
+        std::vector<float> out(rows);
+        moe_.check(mummu_expert_gate_energy(moe_.handle(), layer_, expert_, x, (int64_t)rows, (int)hidden, out.data()));
+        return out;
+    }
 
   private:
     SparseMoe moe_;
-    int layer_, expert_;
+    int layer_, expert_, gate_type_;
 };
 
 // RoutedExperts (models/qwen4exp/experts.rs:1066-1150): caller-supplied router logits, qwen4exp

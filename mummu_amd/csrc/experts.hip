@@ -921,4 +921,87 @@ hipError_t launch_shared_add(float *out, const float *y, const float *x, const v
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------
+// gate energy (nn/moe.rs:508-521): energy[t] = sum over the intermediate width of
+// silu(<gate_i, x_t>)^2, the gate product only.  w holds the expert's gate rows as f32 (the
+// dequantizer's output or an F32 bank).  A workgroup takes kEnergyRows token rows (in LDS) and
+// kEnergyGate gate rows (four per wave, a wave-wide dot each); the squares of a tile are added in
+// a fixed order (per wave by row, then the four waves pairwise), the tiles by the second kernel in
+// ascending order.  Not a hot path: the reference calls it only to pick rows in its skip mode.
+// ------------------------------------------------------------------------------------------
+constexpr int kEnergyRows = 4, kEnergyGate = 16;
+
+__global__ __launch_bounds__(256) void gate_energy_partial_kernel(const float *__restrict__ w, const float *__restrict__ x,
+                                                                  int rows, int hidden, int inter,
+                                                                  float *__restrict__ partial) {
+    extern __shared__ float s_x[];  // kEnergyRows * hidden
+    __shared__ float s_e[4][kEnergyRows];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r0 = blockIdx.x * kEnergyRows, tile = blockIdx.y;
+    for (int idx = tid; idx < kEnergyRows * hidden; idx += 256) {
+        const int r = idx / hidden, c = idx - r * hidden;
+        s_x[idx] = r0 + r < rows ? x[(size_t)(r0 + r) * (size_t)hidden + c] : 0.0f;
+    }
+    __syncthreads();
+    float e[kEnergyRows];
+#pragma unroll
+    for (int r = 0; r < kEnergyRows; r++) e[r] = 0.0f;
+    for (int j = 0; j < kEnergyGate / 4; j++) {
+        const int i = tile * kEnergyGate + 4 * j + wave;  // uniform over the wave
+        if (i >= inter) break;
+        const float *wr = w + (size_t)i * (size_t)hidden;
+        float acc[kEnergyRows];
+#pragma unroll
+        for (int r = 0; r < kEnergyRows; r++) acc[r] = 0.0f;
+        for (int c = lane; c < hidden; c += 64) {
+            const float wv = wr[c];
+#pragma unroll
+            for (int r = 0; r < kEnergyRows; r++) acc[r] = fmaf(wv, s_x[r * hidden + c], acc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < kEnergyRows; r++) {
+            const float sl = det_silu(wave_sum(acc[r]));
+            e[r] = __fadd_rn(e[r], __fmul_rn(sl, sl));
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < kEnergyRows; r++) s_e[wave][r] = e[r];
+    }
+    __syncthreads();
+    if (tid < kEnergyRows && r0 + tid < rows)
+        partial[(size_t)tile * (size_t)rows + (size_t)(r0 + tid)] =
+            __fadd_rn(__fadd_rn(s_e[0][tid], s_e[1][tid]), __fadd_rn(s_e[2][tid], s_e[3][tid]));
+}
+
+__global__ __launch_bounds__(256) void gate_energy_sum_kernel(const float *__restrict__ partial, int tiles, int rows,
+                                                              float *__restrict__ energy) {
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    float e = 0.0f;
+    for (int t = 0; t < tiles; t++) e = __fadd_rn(e, partial[(size_t)t * (size_t)rows + r]);
+    energy[r] = e;
+}
+
+int gate_energy_tiles(int inter) { return (inter + kEnergyGate - 1) / kEnergyGate; }
+
+hipError_t launch_gate_energy(const float *w, const float *x, int rows, int hidden, int inter, float *partial, float *energy,
+                              hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    const size_t lds = sizeof(float) * (size_t)kEnergyRows * (size_t)hidden;
+    if (lds > 128 * 1024 || hidden < 1 || inter < 1) return hipErrorInvalidValue;
+    const int tiles = gate_energy_tiles(inter);
+    if (tiles > 65535) return hipErrorInvalidValue;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)gate_energy_partial_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    launch_kernel(gate_energy_partial_kernel, dim3((rows + kEnergyRows - 1) / kEnergyRows, tiles), dim3(256), lds, s, w, x, rows,
+                  hidden, inter, partial);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    launch_kernel(gate_energy_sum_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, (const float *)partial, tiles, rows, energy);
+    return hipGetLastError();
+}
+
 }  // namespace mummu

@@ -97,6 +97,12 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
 hipError_t launch_shared_add(float *out, const float *y, const float *x, const void *gate_vec, int gate_vec_type,
                              const float *residual, int n, int hidden, hipStream_t s);
 
+// energy[t] = sum_i silu(<w_i, x_t>)^2 over the inter rows of w (f32 [inter][hidden], device); partial holds
+// gate_energy_tiles(inter) * rows floats of scratch.  hidden <= 8192.
+int gate_energy_tiles(int inter);
+hipError_t launch_gate_energy(const float *w, const float *x, int rows, int hidden, int inter, float *partial, float *energy,
+                              hipStream_t s);
+
 // dispatch.hip ------------------------------------------------------------------------
 // Stable counting sort of the assignments by expert (ranks, histograms and scans in LDS, three
 // small launches): offsets[E+1], sorted[A] (position -> assignment), inv[A] (assignment ->

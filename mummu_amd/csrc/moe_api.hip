@@ -959,6 +959,41 @@ int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_
     return download_rows(h, out, h->y, bytes, s, false);
 }
 
+int mummu_expert_gate_energy(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden, float *energy) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if (expert < 0 || expert >= h->cfg.num_experts)
+        return fail(h, MUMMU_ERR_RANGE, "expert " + std::to_string(expert) + " out of range (" + std::to_string(h->cfg.num_experts) + ")");
+    if (hidden != h->cfg.hidden_size)
+        return fail(h, MUMMU_ERR_SHAPE, "input hidden " + std::to_string(hidden) + " does not match expert hidden " + std::to_string(h->cfg.hidden_size));
+    if (rows < 0) return fail(h, MUMMU_ERR_SHAPE, "negative row count");
+    if (rows == 0) return MUMMU_OK;
+    if (!x || !energy) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if (hidden > 8192) return fail(h, MUMMU_ERR_SHAPE, "gate_energy: hidden above 8192 is not supported");
+    if ((rc = ensure_ws(h, rows, rows, 0))) return rc;
+    hipStream_t s = h->stream;
+    if ((rc = upload_rows(h, h->xin, x, sizeof(float) * (size_t)rows * (size_t)hidden, s))) return rc;
+    const Layer &L = h->layers[layer];
+    const int I = h->cfg.expert_intermediate_size;
+    const size_t n = (size_t)I * (size_t)hidden;
+    const uint8_t *bank = L.gate + (size_t)expert * (size_t)I * row_bytes_of(L.gate_type, hidden);
+    // scratch of this call: the gate rows as f32 (unless the bank is F32 already), the tile partials, the result
+    const size_t w_floats = L.gate_type == T_F32 ? 0 : n, p_floats = (size_t)gate_energy_tiles(I) * (size_t)rows;
+    float *scratch = nullptr;
+    HIPCHK(h, hipMalloc(&scratch, sizeof(float) * (w_floats + p_floats + (size_t)rows)));
+    float *w = w_floats ? scratch : nullptr, *partial = scratch + w_floats, *e_dev = partial + p_floats;
+    hipError_t e = hipSuccess;
+    if (w) e = launch_dequantize(L.gate_type, bank, n / (size_t)block_elems(L.gate_type), w, s);
+    if (e == hipSuccess) e = launch_gate_energy(w ? w : (const float *)bank, h->xin, (int)rows, hidden, I, partial, e_dev, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e == hipSuccess) e = hipMemcpy(energy, e_dev, sizeof(float) * (size_t)rows, hipMemcpyDeviceToHost);
+    (void)hipFree(scratch);
+    if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("gate_energy: ") + hipGetErrorString(e));
+    return MUMMU_OK;
+}
+
 int mummu_moe_take_hits(mummu_moe *h, int layer, uint64_t *hits) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     std::lock_guard<std::mutex> lock(h->mu);

@@ -233,6 +233,15 @@ class SparseMoe:
         self._check(self._lib.mummu_expert_run(self._h, layer, expert, _ptr(x), rows, hidden, _ptr(out)))
         return out
 
+    def gate_energy(self, layer: int, expert: int, x) -> np.ndarray:
+        """ExpertExec::gate_energy (nn/moe.rs:411-418, 508-521): per row, sum_i silu(x . gate_i)^2."""
+        x = _f32(x)
+        hidden = x.shape[-1]
+        rows = x.size // max(hidden, 1)
+        out = np.empty(rows, dtype=np.float32)
+        self._check(self._lib.mummu_expert_gate_energy(self._h, layer, expert, _ptr(x), rows, hidden, _ptr(out)))
+        return out
+
     def take_hits(self, layer: int = 0) -> np.ndarray:
         hits = np.zeros(self.config.num_experts, dtype=np.uint64)
         self._check(self._lib.mummu_moe_take_hits(self._h, layer, _ptr(hits)))

@@ -65,6 +65,7 @@ def lib():
         L.orc_router_logits.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]
         L.orc_matvec.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]
         L.orc_expert_ffn.argtypes = [C.POINTER(Banks), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.orc_gate_energy.argtypes = [C.POINTER(Banks), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
         L.orc_apply_routing.argtypes = [C.POINTER(Banks), C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_moe_forward.argtypes = [C.POINTER(Banks), C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                       C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -234,6 +235,16 @@ def expert_ffn(banks: LayerBanks, expert: int, xs) -> np.ndarray:
     rc = lib().orc_expert_ffn(C.byref(banks.c), expert, _p(xs), xs.shape[0], _p(out))
     if rc:
         raise OracleError(rc, "expert_ffn")
+    return out
+
+
+def gate_energy(banks: LayerBanks, expert: int, xs) -> np.ndarray:
+    """nn/moe.rs:508-521: per row, sum over the intermediate width of silu(x . gate_i)^2."""
+    xs = _f32(xs).reshape(-1, banks.hidden)
+    out = np.empty(xs.shape[0], dtype=np.float32)
+    rc = lib().orc_gate_energy(C.byref(banks.c), expert, _p(xs), xs.shape[0], _p(out))
+    if rc:
+        raise OracleError(rc, "gate_energy")
     return out
 
 

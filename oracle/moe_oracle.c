@@ -28,6 +28,10 @@
  *   orc_rmsnorm        - x * rsqrt(mean(x^2) + eps) * gamma, sum of squares in the router's
  *                        512-partial order.
  *                        PARITY UNPINNED (burn RmsNorm is third-party).
+ *   orc_gate_energy    - sum over the intermediate width of silu(x . gate_i)^2, squares added in row
+ *                        order in f32.  PARITY UNPINNED at ulp level (the reference takes matmul,
+ *                        silu, powf and sum_dim from burn, nn/moe.rs:508-521); pinned by the tests
+ *                        against an f64 evaluation on the dequantized gate rows.
  *
  * Everything else (GGUF dequantizers, f16 conversion, the 8-lane dot, silu, the
  * qwen4exp router, expert FFN, ascending-expert two-rounding combine) is fully specified
@@ -632,6 +636,33 @@ ORC_API int orc_expert_ffn(const orc_banks *b, int expert, const float *xs, size
     }
     free(hid);
     free(upv);
+    return rc;
+}
+
+/* nn/moe.rs:508-521 (DeviceExpert::gate_energy): per row, the sum over the intermediate width of
+ * silu(x . gate_i)^2 - the gate product only, on the dequantized gate rows; the squares are added in
+ * row order i = 0, 1, ... in f32.  xs [n x H] -> out [n]. */
+ORC_API int orc_gate_energy(const orc_banks *b, int expert, const float *xs, size_t n, float *out) {
+    int rc = banks_check(b);
+    if (rc != ORC_OK) return rc;
+    if (expert < 0 || expert >= b->n_experts) return ORC_ERR_RANGE;
+    if (n == 0) return ORC_OK;
+    size_t H = (size_t)b->hidden, I = (size_t)b->inter;
+    const uint8_t *g = b->gate + (size_t)expert * I * bank_row_bytes(b->gate_type, H);
+    float *hid = (float *)malloc(sizeof(float) * n * I);
+    rc = orc_matvec(b->gate_type, g, H, I, xs, n, hid);
+    if (rc == ORC_OK) {
+        for (size_t t = 0; t < n; t++) {
+            float e = 0.0f;
+            for (size_t i = 0; i < I; i++) {
+                float s = orc_silu(hid[t * I + i]);
+                float sq = s * s;
+                e = e + sq;
+            }
+            out[t] = e;
+        }
+    }
+    free(hid);
     return rc;
 }
 

@@ -353,6 +353,15 @@ int main(int argc, char **argv) {
         mummu::RoutedExperts re(moe);
         const std::vector<float> y2 = re.apply_routing(0, {2, 2, 2}, {1.0f, 1.0f, 1.0f}, x, 3, 1);
         EXPECT(std::memcmp(y.data(), y2.data(), y.size() * 4) == 0, "ExpertExec::run == apply_routing(top-1, weight 1)");
+        // the rest of the trait: pinned to device 0, always staged, gate energy = sum_i silu(x . gate_i)^2 >= 0
+        const std::vector<float> en = ex.gate_energy(x.data(), 3, H);
+        EXPECT(en.size() == 3 && std::isfinite(en[0]) && en[0] > 0.0f && en[1] > 0.0f && en[2] > 0.0f, "gate_energy finite and positive");
+        const std::vector<float> en1 = ex.gate_energy(x.data() + H, 1, H);
+        EXPECT(std::memcmp(&en1[0], &en[1], 4) == 0, "gate_energy of a row does not depend on the rows beside it");
+        ex.stage(0);
+        ex.evict();
+        ex.disable_native();
+        EXPECT(ex.tier().device == 0 && ex.is_staged(), "tier / is_staged");
         EXPECT(throws([&] { re.apply_routing(0, {2, 9, 2}, {1.0f, 1.0f, 1.0f}, x, 3, 1); }, MUMMU_ERR_RANGE, "expert"), "bad expert id");
     }
     // route known answers (experts.rs:1365-1388)

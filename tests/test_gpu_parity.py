@@ -304,3 +304,37 @@ def test_unsupported_bank_types_and_ragged_rows_are_refused():
         with pytest.raises(M.MoeError, match="whole blocks"):
             m.load_layer(0, np.zeros((2, 640), np.float32), M.F32, np.zeros(10, np.uint8), M.Q4_K, np.zeros(10, np.uint8),
                          M.Q4_K, np.zeros(2 * 640 * 34, np.uint8), M.Q8_0)
+
+
+# ---------------------------------------------------------------------------------------------
+# ExpertExec::gate_energy (nn/moe.rs:411-418, 508-521)
+# ---------------------------------------------------------------------------------------------
+
+def test_gate_energy_matches_the_oracle_and_the_f64_sum(toy_q):
+    m, raw, banks, _ = toy_q
+    H, F, E = TOY_D["hidden"], TOY_D["ffn"], TOY_D["experts"]
+    xs = synth.SplitMix64(31).uniform_vec(9 * H).reshape(9, H)
+    gate = orc.dequantize(raw["gate_type"], raw["gate"]).reshape(E, F, H).astype(np.float64)
+    for e in (0, 3, E - 1):
+        got = m.gate_energy(0, e, xs)
+        pre = xs.astype(np.float64) @ gate[e].T
+        want = ((pre / (1.0 + np.exp(-pre))) ** 2).sum(axis=1)
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(want, 1e-30)), e
+        assert np.allclose(got, orc.gate_energy(banks, e, xs), rtol=1e-5, atol=0)
+    # a row's energy does not depend on the rows beside it; zero rows have none; bad arguments are refused
+    assert np.array_equal(bits(m.gate_energy(0, 2, xs[4:5])), bits(m.gate_energy(0, 2, xs)[4:5]))
+    assert m.gate_energy(0, 2, np.zeros((3, H), np.float32)).tolist() == [0.0, 0.0, 0.0]
+    with pytest.raises(M.MoeError, match="out of range"):
+        m.gate_energy(0, E, xs)
+    with pytest.raises(M.MoeError, match="hidden"):
+        m.gate_energy(0, 0, np.zeros((2, H + 32), np.float32))
+
+
+def test_gate_energy_on_float_banks_and_many_rows(toy):
+    m, router, gate, up, down, banks = toy
+    x = np.tile(toy_a_input(4, 0.25), (5, 1))[:8]  # max_tokens of the fixture is 8
+    g = np.asarray(gate, np.float64).reshape(TOY_A["experts"], TOY_A["inter"], TOY_A["hidden"])
+    for e in range(TOY_A["experts"]):
+        pre = x.astype(np.float64) @ g[e].T
+        want = ((pre / (1.0 + np.exp(-pre))) ** 2).sum(axis=1)
+        assert np.allclose(m.gate_energy(0, e, x), want, rtol=1e-5, atol=1e-12)

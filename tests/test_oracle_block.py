@@ -237,3 +237,46 @@ def test_rmsnorm_and_layer_stack():
         assert np.array_equal(i_l, ids[l])
         cur = (cur + moe).astype(np.float32)
     assert np.array_equal(out.view(np.uint32), cur.view(np.uint32))
+
+
+# --- gate energy (nn/moe.rs:508-521) --------------------------------------------------------
+
+def energy_f64(gate_f32, xs):
+    """sum_i silu(x . g_i)^2 in f64 on the dequantized gate rows [I, H]."""
+    pre = xs.astype(np.float64) @ gate_f32.astype(np.float64).T
+    s = pre / (1.0 + np.exp(-pre))
+    return (s * s).sum(axis=1)
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_gate_energy_is_the_sum_of_squared_silu_gate_activations(which):
+    raw = toy_d_layers(11)[which]
+    H, F, E = TOY_D["hidden"], TOY_D["ffn"], TOY_D["experts"]
+    banks = orc.LayerBanks(H, F, E, raw["gate"], raw["up"], raw["down"], raw["gate_type"], raw["up_type"], raw["down_type"])
+    xs = synth.SplitMix64(21).uniform_vec(6 * H).reshape(6, H)
+    gate = orc.dequantize(raw["gate_type"], raw["gate"]).reshape(E, F, H)
+    for e in (0, E - 1):
+        got = orc.gate_energy(banks, e, xs)
+        want = energy_f64(gate[e], xs)
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(want, 1e-30))
+    # an expert's energy does not depend on which rows share the call, and zero rows have none
+    assert np.array_equal(orc.gate_energy(banks, 2, xs[3:4]), orc.gate_energy(banks, 2, xs)[3:4])
+    assert orc.gate_energy(banks, 2, np.zeros((2, H), np.float32)).tolist() == [0.0, 0.0]
+    with pytest.raises(orc.OracleError):
+        orc.gate_energy(banks, E, xs)
+
+
+def test_gate_energy_on_the_closed_form_toy_block():
+    # the f32 toy layer of nn/moe.rs:1617-1651: the same sum written out in plain Python
+    _, gate, _, _, banks = toy_a_banks()
+    x = toy_a_input(3, 0.5)
+    g = np.asarray(gate, np.float32).reshape(TOY_A["experts"], TOY_A["inter"], TOY_A["hidden"])
+    for e in range(TOY_A["experts"]):
+        want = []
+        for t in range(3):
+            tot = 0.0
+            for i in range(TOY_A["inter"]):
+                pre = sum(float(g[e, i, c]) * float(x[t, c]) for c in range(TOY_A["hidden"]))
+                tot += (pre / (1.0 + np.exp(-pre))) ** 2
+            want.append(tot)
+        assert np.allclose(orc.gate_energy(banks, e, x), want, rtol=1e-5, atol=1e-12)
