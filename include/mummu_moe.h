@@ -189,6 +189,10 @@ MUMMU_API int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, in
  * reported synchronously here; mummu_moe_check() reads the flag back. */
 MUMMU_API int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_t n_tokens, int top_k,
                                        int norm_topk_prob, float *out_dev, void *stream);
+/* ExpertExec::run_tensor_resident (nn/moe.rs:360-371, DeviceExpert's at :470-501): the SwiGLU of one expert on rows
+ * that are already on this device, the result left there; only enqueues on `stream`.  rows <= max_tokens. */
+MUMMU_API int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_dev, int64_t rows, int hidden,
+                                      float *out_dev, void *stream);
 MUMMU_API int mummu_moe_stack_forward_device(mummu_moe *h, const float *x_dev, int64_t n_tokens, int top_k,
                                              int norm_topk_prob, float *out_dev, void *stream);
 /* Synchronises the stream and returns MUMMU_ERR_NONFINITE if any call since the last check

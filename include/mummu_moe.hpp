@@ -468,6 +468,12 @@ class HipExpert final : public ExpertExec {
         return e > 0 ? moe_.resident_bytes() / (uint64_t)e : 0;
     }
     Tier tier() const override { return Tier{0, gate_type_}; }
+    // run_tensor_resident (nn/moe.rs:360-371): rows already on this device, the result left there; only enqueues
+    // on the handle's stream.
+    void run_resident(const float *x_dev, size_t rows, size_t hidden, float *out_dev) const {
+        moe_.check(mummu_expert_run_device(moe_.handle(), layer_, expert_, x_dev, (int64_t)rows, (int)hidden, out_dev,
+                                           mummu_moe_stream(moe_.handle())));
+    }
     std::vector<float> gate_energy(const float *x, size_t rows, size_t hidden) const override {
         std::vector<float> out(rows);
         moe_.check(mummu_expert_gate_energy(moe_.handle(), layer_, expert_, x, (int64_t)rows, (int)hidden, out.data()));

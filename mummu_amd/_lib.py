@@ -73,6 +73,7 @@ SIGNATURES = {
     "mummu_moe_routed": (_I, [_P, _I, _P, _P, _I64, _I, _P]),
     "mummu_moe_apply_routing": (_I, [_P, _I, _P, _P, _P, _I64, _I, _P]),
     "mummu_expert_run": (_I, [_P, _I, _I, _P, _I64, _I, _P]),
+    "mummu_expert_run_device": (_I, [_P, _I, _I, _P, _I64, _I, _P, _P]),
     "mummu_expert_gate_energy": (_I, [_P, _I, _I, _P, _I64, _I, _P]),
     "mummu_moe_take_hits": (_I, [_P, _I, _P]),
     "mummu_moe_stack_forward": (_I, [_P, _P, _I64, _I, _I, _P, _P]),

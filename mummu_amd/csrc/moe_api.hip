@@ -1083,6 +1083,25 @@ int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_
     return forward_impl(h, layer, x_dev, n, top_k, norm, nullptr, out_dev, (hipStream_t)stream);
 }
 
+int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_dev, int64_t rows, int hidden, float *out_dev,
+                            void *stream) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if (expert < 0 || expert >= h->cfg.num_experts)
+        return fail(h, MUMMU_ERR_RANGE, "expert " + std::to_string(expert) + " out of range (" + std::to_string(h->cfg.num_experts) + ")");
+    if (hidden != h->cfg.hidden_size)
+        return fail(h, MUMMU_ERR_SHAPE, "input hidden " + std::to_string(hidden) + " does not match expert hidden " + std::to_string(h->cfg.hidden_size));
+    if ((rc = check_device_call(h, rows, 1, x_dev, out_dev))) return rc;
+    if (rows == 0) return MUMMU_OK;
+    hipStream_t s = (hipStream_t)stream;
+    ExpertBanks b = banks_of(h, h->layers[layer]);
+    if (is_quant_type(b.gate_type)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x_dev, (int)rows, hidden, h->xq, s));
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x_dev, h->xq, nullptr, (int)rows, 1, expert, h->act, h->actq, h->flags, s));
+    LAUNCH(h, K_DOWN, s, launch_down(b, h->act, h->actq, nullptr, (int)rows, 1, expert, out_dev, s));
+    return MUMMU_OK;
+}
+
 int mummu_moe_stack_forward_device(mummu_moe *h, const float *x_dev, int64_t n, int top_k, int norm, float *out_dev, void *stream) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     int rc = check_topk(h, top_k, h->cfg.num_experts);

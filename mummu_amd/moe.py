@@ -271,6 +271,11 @@ class SparseMoe:
         self._check(self._lib.mummu_moe_forward_device(self._h, layer, x_dev.ptr, n, top_k, int(norm_topk_prob),
                                                        out_dev.ptr, self.stream))
 
+    def expert_run_device(self, layer: int, expert: int, x_dev: "DeviceBuffer", rows: int, out_dev: "DeviceBuffer"):
+        """ExpertExec::run_tensor_resident (nn/moe.rs:360-371): rows already on the device, result left there."""
+        self._check(self._lib.mummu_expert_run_device(self._h, layer, expert, x_dev.ptr, rows, self.config.hidden_size,
+                                                      out_dev.ptr, self.stream))
+
     def stack_forward_device(self, x_dev: "DeviceBuffer", n: int, top_k: int, norm_topk_prob: bool, out_dev: "DeviceBuffer"):
         self._check(self._lib.mummu_moe_stack_forward_device(self._h, x_dev.ptr, n, top_k, int(norm_topk_prob),
                                                              out_dev.ptr, self.stream))

@@ -338,3 +338,19 @@ def test_gate_energy_on_float_banks_and_many_rows(toy):
         pre = x.astype(np.float64) @ g[e].T
         want = ((pre / (1.0 + np.exp(-pre))) ** 2).sum(axis=1)
         assert np.allclose(m.gate_energy(0, e, x), want, rtol=1e-5, atol=1e-12)
+
+
+def test_expert_run_device_leaves_the_same_bits_on_the_device(toy_q):
+    # ExpertExec::run_tensor_resident (nn/moe.rs:360-371): rows already on the device, the result left there
+    m = toy_q[0]
+    H = TOY_D["hidden"]
+    xs = synth.SplitMix64(41).uniform_vec(7 * H).reshape(7, H)
+    xd, od = M.DeviceBuffer.from_array(xs), M.DeviceBuffer(xs.nbytes)
+    for e in (1, 5):
+        m.expert_run_device(0, e, xd, 7, od)
+        m.check()
+        assert np.array_equal(bits(od.download(np.float32, (7, H))), bits(m.expert_run(0, e, xs)))
+    with pytest.raises(M.MoeError, match="out of range"):
+        m.expert_run_device(0, 99, xd, 7, od)
+    with pytest.raises(M.MoeError, match="exceeds the workspace"):
+        m.expert_run_device(0, 1, xd, 17, od)
