@@ -312,6 +312,30 @@ MUMMU_API int mummu_st_check_moe_layer(const mummu_st *st, int layer);
  * (BF16 / F16 / F32 kept as stored) and loaded into the handle's layers 0..n_layers. */
 MUMMU_API int mummu_moe_load_safetensors(mummu_moe *h, mummu_st *st, int first_layer, int n_layers);
 
+/* ---- the packed-GEMV custom op over burn's block-32 layout ---------------------------------
+ * Q4GemvOps::q4s_gemv (nn/packed_gemv.rs:248-260; routed by try_q4s_gemv, :98-152; CubeCL kernel
+ * packed_gemv_kernel, :370-451): y = x . w for a weight [K, N] stored as burn stores a quantized tensor on
+ * a device (pack.rs:940-985): values two's complement in 4 bits (Q4S) or 8 bits (Q8S), element j of a u32
+ * word at bits j*bits, words running along N, then one f32 scale per (k, 32 consecutive n):
+ *     y[n] = sum_k float(q(k, n)) * (x[k] * scale(k, n / 32))        (two roundings per term, f32 sum).
+ * A weight is uploaded once and stays in HBM; a call takes 1 row (decode) up to 64 (the reference runs a
+ * short prefill row by row through the same op, :138-150).  The K split is fixed per weight shape, so a
+ * call's bits do not depend on the batch or on timing. */
+typedef struct mummu_packed_weight mummu_packed_weight;
+/* Message of the last failed mummu_packed_* / mummu_q4s_* call on this thread. */
+MUMMU_API const char *mummu_packed_last_error(void);
+/* words: K * N * value_bits / 32 u32; scales: K * N / 32 f32; value_bits 4 or 8; N a multiple of 32. */
+MUMMU_API int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k, int n, int value_bits,
+                                         mummu_packed_weight **out);
+MUMMU_API void mummu_packed_weight_destroy(mummu_packed_weight *w);
+/* Bytes the weight holds in HBM (values + scales: 5 bits per weight at Q4S). */
+MUMMU_API uint64_t mummu_packed_weight_bytes(const mummu_packed_weight *w);
+/* x [m, K] f32 -> y [m, N] f32, host pointers; m <= 64. */
+MUMMU_API int mummu_q4s_gemv(mummu_packed_weight *w, const float *x, int64_t m, int k, float *y);
+/* The same on device pointers; only enqueues on `stream`.  Calls on one weight must not overlap (they share
+ * the partial sums of the K split). */
+MUMMU_API int mummu_q4s_gemv_device(mummu_packed_weight *w, const float *x_dev, int64_t m, int k, float *y_dev, void *stream);
+
 /* ---- plumbing for harnesses that do not link HIP themselves -----------------------------*/
 MUMMU_API void *mummu_device_alloc(size_t bytes);
 MUMMU_API void mummu_device_free(void *p);

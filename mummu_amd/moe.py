@@ -357,6 +357,59 @@ def probe_copy(dst: "DeviceBuffer", src: "DeviceBuffer", nbytes: int, stream=Non
         raise MoeError(rc, lib.mummu_moe_last_error(None).decode())
 
 
+class PackedWeight:
+    """A weight in burn's packed block-32 layout, resident in HBM, behind Q4GemvOps::q4s_gemv
+    (nn/packed_gemv.rs:248-260): `words` [K, N*bits/32] u32 (element j of a word at bits j*bits), `scales`
+    [K, N/32] f32 (pack.rs:940-985)."""
+
+    def __init__(self, words, scales, k: int, n: int, value_bits: int = 4):
+        self._lib = _lib.load()
+        self._h = None
+        words = np.ascontiguousarray(words, dtype=np.uint32)
+        scales = _f32(scales)
+        if words.size != k * n * value_bits // 32 or scales.size != k * (n // 32):
+            raise MoeError(_lib.ERR_SHAPE, f"packed weight: {words.size} words / {scales.size} scales do not make [{k}, {n}] "
+                                           f"at {value_bits} bits")
+        h = C.c_void_p()
+        rc = self._lib.mummu_packed_weight_create(_ptr(words), _ptr(scales), k, n, value_bits, C.byref(h))
+        if rc:
+            raise MoeError(rc, self._lib.mummu_packed_last_error().decode())
+        self._h, self.k, self.n, self.value_bits = h, k, n, value_bits
+
+    def _check(self, rc: int):
+        if rc:
+            raise MoeError(rc, self._lib.mummu_packed_last_error().decode())
+
+    def resident_bytes(self) -> int:
+        return int(self._lib.mummu_packed_weight_bytes(self._h))
+
+    def gemv(self, x) -> np.ndarray:
+        """try_q4s_gemv (nn/packed_gemv.rs:98-152): x [m, K] -> [m, N], m <= 64."""
+        x = _f32(x)
+        k = x.shape[-1] if x.ndim else 0
+        m = x.size // max(k, 1)
+        y = np.empty((m, self.n), dtype=np.float32)
+        self._check(self._lib.mummu_q4s_gemv(self._h, _ptr(x), m, k, _ptr(y)))
+        return y
+
+    def gemv_device(self, x_dev: "DeviceBuffer", m: int, y_dev: "DeviceBuffer", stream=None):
+        self._check(self._lib.mummu_q4s_gemv_device(self._h, x_dev.ptr, m, self.k, y_dev.ptr, stream))
+
+    def close(self):
+        if self._h:
+            self._lib.mummu_packed_weight_destroy(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        self.close()
+
+
 class DeviceBuffer:
     """A plain HIP allocation (hipMalloc) addressed through the library."""
 

@@ -65,6 +65,7 @@ def lib():
         L.orc_router_logits.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]
         L.orc_matvec.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]
         L.orc_expert_ffn.argtypes = [C.POINTER(Banks), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.orc_q4s_gemv.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
         L.orc_gate_energy.argtypes = [C.POINTER(Banks), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
         L.orc_apply_routing.argtypes = [C.POINTER(Banks), C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_moe_forward.argtypes = [C.POINTER(Banks), C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
@@ -235,6 +236,18 @@ def expert_ffn(banks: LayerBanks, expert: int, xs) -> np.ndarray:
     rc = lib().orc_expert_ffn(C.byref(banks.c), expert, _p(xs), xs.shape[0], _p(out))
     if rc:
         raise OracleError(rc, "expert_ffn")
+    return out
+
+
+def q4s_gemv(words, scales, k: int, n: int, bits: int, xs) -> np.ndarray:
+    """nn/packed_gemv.rs:370-451 at split 1: x . w over burn's packed block-32 layout, sequential in k."""
+    words = np.ascontiguousarray(words, dtype=np.uint32)
+    scales = _f32(scales)
+    xs = _f32(xs).reshape(-1, k)
+    out = np.empty((xs.shape[0], n), dtype=np.float32)
+    rc = lib().orc_q4s_gemv(_p(words), _p(scales), k, n, bits, _p(xs), xs.shape[0], _p(out))
+    if rc:
+        raise OracleError(rc, "q4s_gemv")
     return out
 
 

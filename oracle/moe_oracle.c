@@ -639,6 +639,35 @@ ORC_API int orc_expert_ffn(const orc_banks *b, int expert, const float *xs, size
     return rc;
 }
 
+/* nn/packed_gemv.rs:370-451 (packed_gemv_kernel at split 1) == the dequantize-then-matmul form it is
+ * tested against (:1593-1624): y[r][n] = sum over k, in order, of float(q(k, n)) * (x[r][k] * scale(k, n/32)),
+ * the inner product rounded, the outer product rounded, then added.  Layout pack.rs:940-985: values two's
+ * complement in `bits` (4 or 8) bits, element j of a u32 word at bits j*bits, words along N; one f32 scale
+ * per (k, 32 consecutive n).  xs [m x K] -> out [m x N]. */
+ORC_API int orc_q4s_gemv(const uint32_t *words, const float *scales, int k_len, int n, int bits, const float *xs,
+                         size_t m, float *out) {
+    if (bits != 4 && bits != 8) return ORC_ERR_TYPE;
+    if (k_len < 1 || n < 1 || n % 32 != 0) return ORC_ERR_BLOCKS;
+    int per = 32 / bits;
+    size_t n_words = (size_t)n / (size_t)per, n_blocks = (size_t)n / 32;
+    for (size_t r = 0; r < m; r++) {
+        for (int c = 0; c < n; c++) {
+            float acc = 0.0f;
+            for (int k = 0; k < k_len; k++) {
+                uint32_t word = words[(size_t)k * n_words + (size_t)(c / per)];
+                uint32_t raw = (word >> ((uint32_t)(c % per) * (uint32_t)bits)) & ((1u << bits) - 1u);
+                int q = (int)raw;
+                if (raw >= (1u << (bits - 1))) q -= (1 << bits);
+                float x_scaled = xs[r * (size_t)k_len + (size_t)k] * scales[(size_t)k * n_blocks + (size_t)(c / 32)];
+                float prod = (float)q * x_scaled;
+                acc = acc + prod;
+            }
+            out[r * (size_t)n + (size_t)c] = acc;
+        }
+    }
+    return ORC_OK;
+}
+
 /* nn/moe.rs:508-521 (DeviceExpert::gate_energy): per row, the sum over the intermediate width of
  * silu(x . gate_i)^2 - the gate product only, on the dequantized gate rows; the squares are added in
  * row order i = 0, 1, ... in f32.  xs [n x H] -> out [n]. */
