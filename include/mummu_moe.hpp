@@ -485,6 +485,36 @@ class HipExpert final : public ExpertExec {
     int layer_, expert_, gate_type_;
 };
 
+// A weight in burn's packed block-32 layout behind Q4GemvOps::q4s_gemv (nn/packed_gemv.rs:248-260): words
+// [K, N*bits/32] u32, scales [K, N/32] f32 (pack.rs:940-985), uploaded once.
+class PackedWeight {
+  public:
+    PackedWeight(const std::vector<uint32_t> &words, const std::vector<float> &scales, int k, int n, int value_bits = 4)
+        : k_(k), n_(n) {
+        if (words.size() != (size_t)k * (size_t)n * (size_t)value_bits / 32 || scales.size() != (size_t)k * (size_t)(n / 32))
+            throw MoeError(MUMMU_ERR_SHAPE, "packed weight: words / scales do not make [K, N] at this width");
+        mummu_packed_weight *h = nullptr;
+        const int rc = mummu_packed_weight_create(words.data(), scales.data(), k, n, value_bits, &h);
+        if (rc != MUMMU_OK) throw MoeError(rc, mummu_packed_last_error());
+        h_.reset(h, mummu_packed_weight_destroy);
+    }
+    // try_q4s_gemv (nn/packed_gemv.rs:98-152): x [m, K] -> [m, N], m <= 64.
+    std::vector<float> gemv(const std::vector<float> &x) const {
+        if (k_ <= 0 || x.size() % (size_t)k_ != 0) throw MoeError(MUMMU_ERR_SHAPE, "input length is not a whole number of K-wide rows");
+        const size_t m = x.size() / (size_t)k_;
+        std::vector<float> y(m * (size_t)n_);
+        const int rc = mummu_q4s_gemv(h_.get(), x.data(), (int64_t)m, k_, y.data());
+        if (rc != MUMMU_OK) throw MoeError(rc, mummu_packed_last_error());
+        return y;
+    }
+    uint64_t resident_bytes() const { return mummu_packed_weight_bytes(h_.get()); }
+    mummu_packed_weight *handle() const { return h_.get(); }
+
+  private:
+    int k_, n_;
+    std::shared_ptr<mummu_packed_weight> h_;
+};
+
 // RoutedExperts (models/qwen4exp/experts.rs:1066-1150): caller-supplied router logits, qwen4exp
 // routing rules (f64 normaliser, 2^-14 floor, non-finite logits refused).
 class RoutedExperts {

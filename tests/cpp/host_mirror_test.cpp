@@ -364,6 +364,19 @@ int main(int argc, char **argv) {
         EXPECT(ex.tier().device == 0 && ex.is_staged(), "tier / is_staged");
         EXPECT(throws([&] { re.apply_routing(0, {2, 9, 2}, {1.0f, 1.0f, 1.0f}, x, 3, 1); }, MUMMU_ERR_RANGE, "expert"), "bad expert id");
     }
+    // the packed GEMV op: a weight whose every code is -8 with unit scales against a row of ones gives -8 K
+    {
+        const int PK = 64, PN = 64;
+        std::vector<uint32_t> words((size_t)PK * PN / 8, 0x88888888u);
+        std::vector<float> scales((size_t)PK * PN / 32, 1.0f);
+        mummu::PackedWeight pw(words, scales, PK, PN);
+        const std::vector<float> y = pw.gemv(std::vector<float>(PK, 1.0f));
+        bool all = y.size() == (size_t)PN;
+        for (float v : y) all = all && v == -8.0f * PK;
+        EXPECT(all, "q4s_gemv decodes two's complement nibbles");
+        EXPECT(pw.resident_bytes() == (uint64_t)PK * PN / 2 + (uint64_t)PK * PN / 8, "packed weight bytes");
+        EXPECT(throws([&] { pw.gemv(std::vector<float>(PK + 1, 0.0f)); }, MUMMU_ERR_SHAPE, "rows"), "ragged packed input");
+    }
     // route known answers (experts.rs:1365-1388)
     {
         const std::vector<float> logits = {0.0f, 3.0f, 1.0f, 2.5f, -2.0f, 2.0f, 0.5f, 2.9f};
