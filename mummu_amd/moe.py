@@ -53,6 +53,22 @@ class SparseMoeConfig:
     num_experts: int
     num_experts_per_tok: int
 
+    def init(self, seed: int = 0, **handle_args) -> "SparseMoe":
+        """SparseMoeConfig::init (nn/moe.rs:61-99): a block with Linear-style uniform weights, every projection
+        bounded by 1/sqrt(its fan-in) (router and gate/up: hidden, down: intermediate), as f32 banks.  The
+        reference draws from burn's generator; here the draws are SplitMix64 of `seed`.  The same checks refuse
+        fewer than two experts, a top-k outside 1..=num_experts and zero widths."""
+        from . import synth
+        moe = SparseMoe(self, **handle_args)
+        h, i, e = self.hidden_size, self.expert_intermediate_size, self.num_experts
+        rng = synth.SplitMix64(seed)
+        bh, bi = 1.0 / np.sqrt(float(h)), 1.0 / np.sqrt(float(i))
+        router = rng.uniform(-bh, bh, e * h)
+        gate, up = rng.uniform(-bh, bh, e * i * h), rng.uniform(-bh, bh, e * i * h)
+        down = rng.uniform(-bi, bi, e * h * i)
+        moe.load_layer(0, router, F32, gate, F32, up, F32, down, F32)
+        return moe
+
 
 @dataclass
 class Routing:

@@ -354,3 +354,20 @@ def test_expert_run_device_leaves_the_same_bits_on_the_device(toy_q):
         m.expert_run_device(0, 99, xd, 7, od)
     with pytest.raises(M.MoeError, match="exceeds the workspace"):
         m.expert_run_device(0, 1, xd, 17, od)
+
+
+def test_config_init_draws_fan_in_bounded_uniform_weights_and_checks_like_the_reference():
+    # nn/moe.rs:61-99
+    cfg = M.SparseMoeConfig(64, 32, 4, 2)
+    with cfg.init(seed=3, max_tokens=4) as m:
+        g, d = m.dequantize_expert(0, "gate", 1), m.dequantize_expert(0, "down", 3)
+        assert g.shape == (32, 64) and d.shape == (64, 32)
+        assert np.abs(g).max() <= 1 / 8 and np.abs(g).max() > 0.9 / 8          # 1/sqrt(64)
+        assert np.abs(d).max() <= 1 / np.sqrt(32) and np.abs(d).max() > 0.9 / np.sqrt(32)
+        x = synth.SplitMix64(1).uniform_vec(3 * 64).reshape(3, 64)
+        assert np.all(np.isfinite(m.forward(x, 2, False))) and np.any(m.forward(x, 2, False) != 0)
+    with cfg.init(seed=3, max_tokens=4) as a, cfg.init(seed=4, max_tokens=4) as b:
+        assert not np.array_equal(a.dequantize_expert(0, "up", 0), b.dequantize_expert(0, "up", 0))
+    for bad in (M.SparseMoeConfig(64, 32, 1, 1), M.SparseMoeConfig(64, 32, 4, 5), M.SparseMoeConfig(0, 32, 4, 2)):
+        with pytest.raises(M.MoeError):
+            bad.init()
