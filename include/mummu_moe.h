@@ -133,6 +133,12 @@ MUMMU_API uint64_t mummu_moe_resident_bytes(const mummu_moe *h);
  * x [n_tokens, hidden] f32 -> out [n_tokens, hidden] f32. */
 MUMMU_API int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n_tokens, int top_k,
                                 int norm_topk_prob, float *out);
+/* The same with the activations in the caller's ambient dtype, as the reference's forward takes and returns
+ * them (nn/moe.rs:116-135: the block works in f32 and the result goes back to the input's dtype): x_type
+ * MUMMU_F32, MUMMU_F16 or MUMMU_BF16; x and out hold n_tokens * hidden values of that type.  16-bit rows are
+ * widened exactly on the device, the f32 result is rounded to nearest even. */
+MUMMU_API int mummu_moe_forward_typed(mummu_moe *h, int layer, const void *x, int x_type, int64_t n_tokens, int top_k,
+                                      int norm_topk_prob, void *out);
 
 /* SparseMoePerExpert::route (nn/moe.rs:247-290): ids/weights [n_tokens, top_k] in slot
  * (descending probability) order; logits [n_tokens, E] optional (may be NULL). */

@@ -67,6 +67,7 @@ SIGNATURES = {
     "mummu_moe_get_config": (_I, [_P, _P]),
     "mummu_moe_resident_bytes": (C.c_uint64, [_P]),
     "mummu_moe_batched_from": (C.c_int, [_P, C.c_int]),
+    "mummu_moe_forward_typed": (_I, [_P, _I, _P, _I, _I64, _I, _I, _P]),
     "mummu_moe_forward": (_I, [_P, _I, _P, _I64, _I, _I, _P]),
     "mummu_moe_route": (_I, [_P, _I, _P, _I64, _I, _I, _P, _P, _P]),
     "mummu_route_logits": (_I, [_P, _P, _I64, _I, _I, _I, _I, _P, _P]),

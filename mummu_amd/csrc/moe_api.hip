@@ -585,6 +585,31 @@ int stack_impl(mummu_moe *h, const float *x, int64_t n, int k, int norm, float *
 
 }  // namespace
 
+namespace mummu {
+
+// 16-bit rows <-> f32 rows for the entry point that takes the caller's ambient dtype.  Widening is exact;
+// narrowing rounds to nearest even (NaN stays NaN).
+template <int T>
+__global__ __launch_bounds__(256) void widen_rows_kernel(const uint16_t *__restrict__ src, size_t n, float *__restrict__ dst) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = T == T_F16 ? half_bits_to_float(src[i]) : bf16_bits_to_float(src[i]);
+}
+
+template <int T>
+__global__ __launch_bounds__(256) void narrow_rows_kernel(const float *__restrict__ src, size_t n, uint16_t *__restrict__ dst) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = src[i];
+    if (T == T_F16) {
+        dst[i] = __builtin_bit_cast(uint16_t, (_Float16)v);  // round to nearest even
+    } else {
+        const uint32_t b = __float_as_uint(v);
+        dst[i] = v != v ? (uint16_t)((b >> 16) | 0x0040u) : (uint16_t)((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
+    }
+}
+
+}  // namespace mummu
+
 extern "C" {
 
 int mummu_device_count(void) {
@@ -808,6 +833,35 @@ int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n, int to
     if ((rc = upload_rows(h, h->xin, x, bytes, h->stream))) return rc;
     if ((rc = forward_impl(h, layer, h->xin, n, top_k, norm, nullptr, h->xout, h->stream))) return rc;
     return download_rows(h, out, h->xout, bytes, h->stream, true);
+}
+
+int mummu_moe_forward_typed(mummu_moe *h, int layer, const void *x, int x_type, int64_t n, int top_k, int norm, void *out) {
+    if (x_type == MUMMU_F32) return mummu_moe_forward(h, layer, (const float *)x, n, top_k, norm, (float *)out);
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    if (x_type != MUMMU_F16 && x_type != MUMMU_BF16)
+        return fail(h, MUMMU_ERR_TYPE, "forward: activations are F32, F16 or BF16 (got type " + std::to_string(x_type) + ")");
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (!x || !out) return fail(h, MUMMU_ERR_ARG, "null buffer");
+    if ((rc = ensure_ws(h, n, n * top_k, 0))) return rc;
+    hipStream_t s = h->stream;
+    const size_t count = (size_t)n * (size_t)h->cfg.hidden_size, bytes16 = count * 2;
+    const dim3 grid((unsigned)((count + 255) / 256)), block(256);
+    // the 16-bit rows land in the output buffer (not yet needed), are widened into the input buffer, and after the
+    // block has run the f32 result is narrowed into the input buffer (no longer needed) and read back from there
+    if ((rc = upload_rows(h, h->xout, (const float *)x, bytes16, s))) return rc;
+    if (x_type == MUMMU_F16) launch_kernel(widen_rows_kernel<T_F16>, grid, block, 0, s, (const uint16_t *)h->xout, count, h->xin);
+    else launch_kernel(widen_rows_kernel<T_BF16>, grid, block, 0, s, (const uint16_t *)h->xout, count, h->xin);
+    HIPCHK(h, hipGetLastError());
+    if ((rc = forward_impl(h, layer, h->xin, n, top_k, norm, nullptr, h->xout, s))) return rc;
+    if (x_type == MUMMU_F16) launch_kernel(narrow_rows_kernel<T_F16>, grid, block, 0, s, (const float *)h->xout, count, (uint16_t *)h->xin);
+    else launch_kernel(narrow_rows_kernel<T_BF16>, grid, block, 0, s, (const float *)h->xout, count, (uint16_t *)h->xin);
+    HIPCHK(h, hipGetLastError());
+    return download_rows(h, (float *)out, h->xin, bytes16, s, true);
 }
 
 int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_k, int norm, int32_t *ids, float *weights,

@@ -199,6 +199,16 @@ class SparseMoe:
         self._check(self._lib.mummu_moe_forward(self._h, layer, _ptr(xt), xt.shape[0], top_k, int(norm_topk_prob), _ptr(out)))
         return out.reshape(shape)
 
+    def forward_typed(self, x_bits, dtype: int, top_k: int, norm_topk_prob: bool, layer: int = 0) -> np.ndarray:
+        """forward on activations in their ambient dtype (nn/moe.rs:116-135): `x_bits` holds [tokens, hidden] values
+        as float32 (F32) or as the uint16 bit patterns of F16 / BF16; the result comes back in the same form."""
+        want = np.float32 if dtype == F32 else np.uint16
+        xb = np.ascontiguousarray(x_bits, dtype=want).reshape(-1, self.config.hidden_size)
+        out = np.empty_like(xb)
+        self._check(self._lib.mummu_moe_forward_typed(self._h, layer, _ptr(xb), dtype, xb.shape[0], top_k, int(norm_topk_prob),
+                                                      _ptr(out)))
+        return out
+
     def route(self, xt, top_k: int, norm_topk_prob: bool, layer: int = 0, return_logits: bool = False):
         """nn/moe.rs:247-290."""
         xt, _ = self._rows(xt)

@@ -371,3 +371,20 @@ def test_config_init_draws_fan_in_bounded_uniform_weights_and_checks_like_the_re
     for bad in (M.SparseMoeConfig(64, 32, 1, 1), M.SparseMoeConfig(64, 32, 4, 5), M.SparseMoeConfig(0, 32, 4, 2)):
         with pytest.raises(M.MoeError):
             bad.init()
+
+
+@pytest.mark.parametrize("dtype", [M.F16, M.BF16])
+def test_forward_in_the_ambient_dtype_is_the_f32_block_between_exact_widening_and_nearest_even_narrowing(toy_q, dtype):
+    # nn/moe.rs:116-135: the block works in f32 and hands the result back in the input's dtype
+    m = toy_q[0]
+    H = TOY_D["hidden"]
+    x32 = synth.SplitMix64(51).uniform_vec(6 * H).reshape(6, H)
+    bits16 = synth.encode_float(x32, dtype).view(np.uint16).reshape(6, H)
+    widened = (bits16.astype(np.uint32) << 16).view(np.float32) if dtype == M.BF16 else bits16.view(np.float16).astype(np.float32)
+    want = synth.encode_float(m.forward(widened, 2, True), dtype).view(np.uint16).reshape(6, H)
+    got = m.forward_typed(bits16, dtype, 2, True)
+    assert got.dtype == np.uint16 and np.array_equal(got, want)
+    # F32 through the same entry point is the plain forward
+    assert np.array_equal(bits(m.forward_typed(x32, M.F32, 2, True)), bits(m.forward(x32, 2, True)))
+    with pytest.raises(M.MoeError, match="F32, F16 or BF16"):
+        m._check(m._lib.mummu_moe_forward_typed(m._h, 0, bits16.ctypes.data, M.Q8_0, 6, 2, 1, got.ctypes.data))
