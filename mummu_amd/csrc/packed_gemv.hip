@@ -119,8 +119,15 @@ __global__ __launch_bounds__(256) void packed_gemv_sum_kernel(const float *__res
                                                               float *__restrict__ y) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
+    // ascending slices, eight loads out before the first add (a missing slice adds +0.0, which changes nothing)
     float total = 0.0f;
-    for (int s = 0; s < slices; s++) total = __fadd_rn(total, partial[(size_t)s * n + i]);
+    for (int s0 = 0; s0 < slices; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = s0 + u < slices ? partial[(size_t)(s0 + u) * n + i] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) total = __fadd_rn(total, v[u]);
+    }
     y[i] = total;
 }
 
