@@ -333,6 +333,10 @@ MUMMU_API const char *mummu_packed_last_error(void);
 /* words: K * N * value_bits / 32 u32; scales: K * N / 32 f32; value_bits 4 or 8; N a multiple of 32. */
 MUMMU_API int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k, int n, int value_bits,
                                          mummu_packed_weight **out);
+/* The same for a weight that is already in HBM (a backend's own quantized tensor): the two device buffers are
+ * borrowed, not copied and not freed, and must outlive the handle. */
+MUMMU_API int mummu_packed_weight_wrap_device(const uint32_t *words_dev, const float *scales_dev, int k, int n, int value_bits,
+                                              mummu_packed_weight **out);
 MUMMU_API void mummu_packed_weight_destroy(mummu_packed_weight *w);
 /* Bytes the weight holds in HBM (values + scales: 5 bits per weight at Q4S). */
 MUMMU_API uint64_t mummu_packed_weight_bytes(const mummu_packed_weight *w);

@@ -78,6 +78,7 @@ SIGNATURES = {
     "mummu_expert_gate_energy": (_I, [_P, _I, _I, _P, _I64, _I, _P]),
     "mummu_packed_last_error": (C.c_char_p, []),
     "mummu_packed_weight_create": (_I, [_P, _P, _I, _I, _I, _P]),
+    "mummu_packed_weight_wrap_device": (_I, [_P, _P, _I, _I, _I, _P]),
     "mummu_packed_weight_destroy": (None, [_P]),
     "mummu_packed_weight_bytes": (C.c_uint64, [_P]),
     "mummu_q4s_gemv": (_I, [_P, _P, _I64, _I, _P]),

@@ -140,6 +140,7 @@ struct mummu_packed_weight {
     float *scales = nullptr;    // device [K][N/32]
     float *x = nullptr, *y = nullptr, *partial = nullptr;  // staging for the host-pointer call and the K partials
     int k = 0, n = 0, bits = 4, grid_k = 1, k_chunk = 0;
+    bool owns_weight = true;  // false: words and scales are the caller's device buffers
     hipStream_t stream = nullptr;
     std::mutex mu;
     std::string error;
@@ -191,8 +192,8 @@ extern "C" {
 
 const char *mummu_packed_last_error(void) { return g_packed_error.c_str(); }
 
-int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k, int n, int value_bits,
-                               mummu_packed_weight **out) {
+static int packed_create(const uint32_t *words, const float *scales, int k, int n, int value_bits, bool on_device,
+                         mummu_packed_weight **out) {
     if (!out) return pfail(nullptr, MUMMU_ERR_ARG, "null argument");
     *out = nullptr;
     if (!words || !scales) return pfail(nullptr, MUMMU_ERR_ARG, "null weight buffer");
@@ -210,6 +211,7 @@ int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k
     w->k = k;
     w->n = n;
     w->bits = value_bits;
+    w->owns_weight = !on_device;
     const int per = 32 / value_bits, n_words = n / per;
     // K split over the grid: two workgroups per CU at one row (more slices only add partial sums to write and
     // read again), slices a whole number of unrolled steps and at least 64 steps long
@@ -223,14 +225,20 @@ int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k
     w->k_chunk = ((k + slices - 1) / slices + kPgUnroll - 1) / kPgUnroll * kPgUnroll;
     w->grid_k = (k + w->k_chunk * kPgWaves - 1) / (w->k_chunk * kPgWaves);  // (rounding the slices up may empty the last workgroups)
     const size_t wb = sizeof(uint32_t) * (size_t)k * (size_t)n_words, sb = sizeof(float) * (size_t)k * (size_t)(n / 32);
-    hipError_t e = hipMalloc(&w->words, wb);
-    if (e == hipSuccess) e = hipMalloc(&w->scales, sb);
+    hipError_t e = hipSuccess;
+    if (on_device) {
+        w->words = const_cast<uint32_t *>(words);
+        w->scales = const_cast<float *>(scales);
+    } else {
+        e = hipMalloc(&w->words, wb);
+        if (e == hipSuccess) e = hipMalloc(&w->scales, sb);
+    }
     if (e == hipSuccess) e = hipMalloc(&w->x, sizeof(float) * (size_t)kMaxRows * (size_t)k);
     if (e == hipSuccess) e = hipMalloc(&w->y, sizeof(float) * (size_t)kMaxRows * (size_t)n);
     if (e == hipSuccess) e = hipMalloc(&w->partial, sizeof(float) * (size_t)grid_k * (size_t)kMaxRows * (size_t)n);
     if (e == hipSuccess) e = hipStreamCreate(&w->stream);
-    if (e == hipSuccess) e = hipMemcpy(w->words, words, wb, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemcpy(w->scales, scales, sb, hipMemcpyHostToDevice);
+    if (e == hipSuccess && !on_device) e = hipMemcpy(w->words, words, wb, hipMemcpyHostToDevice);
+    if (e == hipSuccess && !on_device) e = hipMemcpy(w->scales, scales, sb, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         const std::string msg = std::string("packed weight: ") + hipGetErrorString(e);
         mummu_packed_weight_destroy(w);
@@ -240,14 +248,26 @@ int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k
     return MUMMU_OK;
 }
 
+int mummu_packed_weight_create(const uint32_t *words, const float *scales, int k, int n, int value_bits,
+                               mummu_packed_weight **out) {
+    return packed_create(words, scales, k, n, value_bits, false, out);
+}
+
+int mummu_packed_weight_wrap_device(const uint32_t *words_dev, const float *scales_dev, int k, int n, int value_bits,
+                                    mummu_packed_weight **out) {
+    return packed_create(words_dev, scales_dev, k, n, value_bits, true, out);
+}
+
 void mummu_packed_weight_destroy(mummu_packed_weight *w) {
     if (!w) return;
     if (w->stream) {
         (void)hipStreamSynchronize(w->stream);
         (void)hipStreamDestroy(w->stream);
     }
-    (void)hipFree(w->words);
-    (void)hipFree(w->scales);
+    if (w->owns_weight) {
+        (void)hipFree(w->words);
+        (void)hipFree(w->scales);
+    }
     (void)hipFree(w->x);
     (void)hipFree(w->y);
     (void)hipFree(w->partial);

@@ -402,6 +402,20 @@ class PackedWeight:
             raise MoeError(rc, self._lib.mummu_packed_last_error().decode())
         self._h, self.k, self.n, self.value_bits = h, k, n, value_bits
 
+    @classmethod
+    def wrap_device(cls, words_dev: "DeviceBuffer", scales_dev: "DeviceBuffer", k: int, n: int, value_bits: int = 4):
+        """A weight whose words and scales already lie in device memory (borrowed; keep the buffers alive)."""
+        self = cls.__new__(cls)
+        self._lib = _lib.load()
+        h = C.c_void_p()
+        rc = self._lib.mummu_packed_weight_wrap_device(words_dev.ptr, scales_dev.ptr, k, n, value_bits, C.byref(h))
+        if rc:
+            self._h = None
+            raise MoeError(rc, self._lib.mummu_packed_last_error().decode())
+        self._h, self.k, self.n, self.value_bits = h, k, n, value_bits
+        self._keep = (words_dev, scales_dev)
+        return self
+
     def _check(self, rc: int):
         if rc:
             raise MoeError(rc, self._lib.mummu_packed_last_error().decode())

@@ -112,3 +112,15 @@ def test_gpu_packed_gemv_decodes_every_code_and_checks_its_arguments():
         M.PackedWeight(np.zeros(k * n // 16, np.uint32), np.ones((k, 2), np.float32), k, n, 2)
     with pytest.raises(M.MoeError):
         M.PackedWeight(np.zeros(k * 6, np.uint32), np.ones((k, 1), np.float32), k, 48, 4)
+
+
+@pytest.mark.gpu
+def test_gpu_packed_gemv_on_a_weight_that_is_already_in_device_memory():
+    from mummu_amd import moe as M
+    k, n = 1024, 2048
+    codes, scales, words, x = case(k, n, 4, 3, 77)
+    wd, sd = M.DeviceBuffer.from_array(words), M.DeviceBuffer.from_array(scales)
+    with M.PackedWeight(words, scales, k, n, 4) as own, M.PackedWeight.wrap_device(wd, sd, k, n, 4) as borrowed:
+        assert np.array_equal(own.gemv(x).view(np.uint32), borrowed.gemv(x).view(np.uint32))
+    # the borrowed buffers are still the caller's after the handle is gone
+    assert np.array_equal(wd.download(np.uint32, words.shape), words)
