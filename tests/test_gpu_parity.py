@@ -388,3 +388,19 @@ def test_forward_in_the_ambient_dtype_is_the_f32_block_between_exact_widening_an
     assert np.array_equal(bits(m.forward_typed(x32, M.F32, 2, True)), bits(m.forward(x32, 2, True)))
     with pytest.raises(M.MoeError, match="F32, F16 or BF16"):
         m._check(m._lib.mummu_moe_forward_typed(m._h, 0, bits16.ctypes.data, M.Q8_0, 6, 2, 1, got.ctypes.data))
+
+
+def test_gate_energy_with_rows_wider_than_the_default_lds_window():
+    # 4 rows of 4096 f32 are 64 KB of LDS: above the 48 KB a launch gets without asking
+    H, I, E = 4096, 64, 2
+    g = np.random.Generator(np.random.PCG64(5))
+    gate = (g.standard_normal((E, I, H), dtype=np.float32) * 0.02).astype(np.float32)
+    up, down = gate.copy(), (g.standard_normal((E, H, I), dtype=np.float32) * 0.02).astype(np.float32)
+    router = (g.standard_normal((E, H), dtype=np.float32) * 0.02).astype(np.float32)
+    x = g.standard_normal((5, H), dtype=np.float32)
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, 1), max_tokens=8) as m:
+        m.load_layer(0, router, M.F32, gate, M.F32, up, M.F32, down, M.F32)
+        got = m.gate_energy(0, 1, x)
+    pre = x.astype(np.float64) @ gate[1].astype(np.float64).T
+    want = ((pre / (1.0 + np.exp(-pre))) ** 2).sum(axis=1)
+    assert np.all(np.abs(got - want) <= 1e-5 * want)
