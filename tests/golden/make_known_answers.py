@@ -35,6 +35,35 @@ def q6_k_block():
     return b
 
 
+def q4_0_block():
+    # f16 d = 2, qs[0] = 0x31 (low nibble 1 -> element 0, high nibble 3 -> element 16)
+    return f16(2.0) + [0x31] + [0] * 15
+
+
+def q4_1_block():
+    # f16 d = 2, f16 m = 1, qs[0] = 0x31
+    return f16(2.0) + f16(1.0) + [0x31] + [0] * 15
+
+
+def q5_0_block():
+    # f16 d = 1, qh = 1 | 1 << 16 (little endian), qs[0] = 0x21
+    return f16(1.0) + [1, 0, 1, 0] + [0x21] + [0] * 15
+
+
+def q5_1_block():
+    # f16 d = 1, f16 m = 1, qh = 1, qs[0] = 0x01
+    return f16(1.0) + f16(1.0) + [1, 0, 0, 0] + [0x01] + [0] * 15
+
+
+def q5_k_block():
+    # d = 1, dmin = 1, scales[0] = 2 (sub 0 scale), scales[1] = 3 (sub 1 scale), scales[4] = 1 (sub 0 min),
+    # qh[0] = 1 (element 0 gets +16), ql[0] = 0x21 (low 1 -> element 0, high 2 -> element 32)
+    b = [0] * 176
+    b[0:2], b[2:4] = f16(1.0), f16(1.0)
+    b[4], b[5], b[8], b[16], b[48] = 2, 3, 1, 1, 0x21
+    return b
+
+
 def main():
     stable = [-1000.0] * 48
     stable[5], stable[16 + 9], stable[16 + 3], stable[32 + 15] = 1000.0, 999.0, 998.0, 30.0
@@ -48,6 +77,11 @@ def main():
             {"cite": "gguf.rs:2395-2405", "type": 8, "bytes": q8_0_block(), "count": 32, "expect": {"0": -8.0, "16": 0.0, "31": 7.5}},
             {"cite": "gguf.rs:2407-2429", "type": 12, "bytes": q4_k_block(), "count": 256,
              "expect": {"0": 1.5, "1": -0.5, "32": 15.0, "128": 3.0}},
+            {"cite": "gguf.rs:2549-2560", "type": 2, "bytes": q4_0_block(), "count": 32, "expect": {"0": -14.0, "16": -10.0, "1": -16.0}},
+            {"cite": "gguf.rs:2562-2569", "type": 3, "bytes": q4_1_block(), "count": 32, "expect": {"0": 3.0, "16": 7.0, "1": 1.0}},
+            {"cite": "gguf.rs:2572-2582", "type": 6, "bytes": q5_0_block(), "count": 32, "expect": {"0": 1.0, "16": 2.0, "1": -16.0}},
+            {"cite": "gguf.rs:2584-2592", "type": 7, "bytes": q5_1_block(), "count": 32, "expect": {"0": 18.0, "16": 1.0}},
+            {"cite": "gguf.rs:2638-2652", "type": 13, "bytes": q5_k_block(), "count": 256, "expect": {"0": 33.0, "1": -1.0, "32": 6.0}},
             {"cite": "gguf.rs:2431-2447", "type": 14, "bytes": q6_k_block(), "count": 256, "expect": {"0": 62.0, "32": -32.0, "64": 0.0}},
         ],
         "codec_refused": [

@@ -102,6 +102,115 @@ def np_dequant_q4_k(raw):
     return ((ds * q).astype(np.float32) - mins).astype(np.float32).reshape(-1)
 
 
+def _f16col(b, off):
+    return b[:, off:off + 2].copy().view(np.float16).astype(np.float32)
+
+
+def _k4_scales(s):
+    """The 6-bit (scale, min) pairs of a Q4_K / Q5_K super-block from its 12 packed bytes."""
+    sc = np.empty((s.shape[0], 8), dtype=np.float32)
+    mn = np.empty((s.shape[0], 8), dtype=np.float32)
+    for j in range(8):
+        if j < 4:
+            sc[:, j] = s[:, j] & 63
+            mn[:, j] = s[:, j + 4] & 63
+        else:
+            sc[:, j] = (s[:, j + 4] & 0x0F) | ((s[:, j - 4] >> 6) << 4)
+            mn[:, j] = (s[:, j + 4] >> 4) | ((s[:, j] >> 6) << 4)
+    return sc, mn
+
+
+def np_dequant_q5_k(raw):
+    # 176 B: d, dmin, 12 B scales, 32 B fifth bits (bit 2c / 2c+1 of byte l: chunk c, low / high nibble), 128 B nibbles
+    b = raw.reshape(-1, 176)
+    d, dmin = _f16col(b, 0), _f16col(b, 2)
+    sc, mn = _k4_scales(b[:, 4:16])
+    qh = b[:, 16:48]
+    qs = b[:, 48:].reshape(-1, 4, 32)
+    q = np.empty((b.shape[0], 8, 32), dtype=np.float32)
+    for c in range(4):
+        q[:, 2 * c] = (qs[:, c] & 0x0F) + 16 * ((qh >> (2 * c)) & 1)
+        q[:, 2 * c + 1] = (qs[:, c] >> 4) + 16 * ((qh >> (2 * c + 1)) & 1)
+    ds = (d * sc)[:, :, None]
+    mins = (dmin * mn)[:, :, None]
+    return ((ds * q).astype(np.float32) - mins).astype(np.float32).reshape(-1)
+
+
+def np_dequant_q6_k(raw):
+    # 210 B: 128 B low nibbles, 64 B two-bit tops, 16 signed scales (one per 16 elements), d
+    b = raw.reshape(-1, 210)
+    ql = b[:, 0:128].reshape(-1, 2, 64)
+    qh = b[:, 128:192].reshape(-1, 2, 32)
+    sc = b[:, 192:208].view(np.int8).astype(np.float32).reshape(-1, 2, 8)
+    d = _f16col(b, 208)
+    out = np.empty((b.shape[0], 2, 4, 32), dtype=np.float32)
+    for g in range(4):  # elements 32g .. 32g+31 of a 128-element half
+        lo = ql[:, :, (g & 1) * 32:(g & 1) * 32 + 32]
+        lo = (lo >> 4) if g >= 2 else (lo & 0x0F)
+        q = (lo | (((qh >> (2 * g)) & 3) << 4)).astype(np.int16) - 32
+        s = np.repeat(sc[:, :, 2 * g:2 * g + 2], 16, axis=2)  # scale index l / 16 + 2g
+        out[:, :, g] = ((d[:, :, None] * s).astype(np.float32) * q.astype(np.float32)).astype(np.float32)
+    return out.reshape(-1)
+
+
+def _legacy_codes(b, qs_off, qh_off=None):
+    """Elements 0..15 are the low nibbles, 16..31 the high ones; bit j of qh tops element j."""
+    qs = b[:, qs_off:qs_off + 16]
+    q = np.concatenate([qs & 0x0F, qs >> 4], axis=1).astype(np.uint32)
+    if qh_off is not None:
+        qh = b[:, qh_off:qh_off + 4].copy().view(np.uint32)
+        q |= ((qh >> np.arange(32, dtype=np.uint32)[None, :]) & 1) << 4
+    return q.astype(np.float32)
+
+
+def np_dequant_legacy(dtype, raw):
+    b = raw.reshape(-1, synth.BLOCK_BYTES[dtype])
+    d = _f16col(b, 0)
+    if dtype == synth.Q4_0:
+        return (d * (_legacy_codes(b, 2) - 8.0)).astype(np.float32).reshape(-1)
+    if dtype == synth.Q5_0:
+        return (d * (_legacy_codes(b, 6, 2) - 16.0)).astype(np.float32).reshape(-1)
+    m = _f16col(b, 2)
+    q = _legacy_codes(b, 4) if dtype == synth.Q4_1 else _legacy_codes(b, 8, 4)
+    return ((d * q).astype(np.float32) + m).astype(np.float32).reshape(-1)
+
+
+NP_DECODERS = {
+    synth.Q5_K: np_dequant_q5_k, synth.Q6_K: np_dequant_q6_k,
+    synth.Q4_0: lambda r: np_dequant_legacy(synth.Q4_0, r), synth.Q4_1: lambda r: np_dequant_legacy(synth.Q4_1, r),
+    synth.Q5_0: lambda r: np_dequant_legacy(synth.Q5_0, r), synth.Q5_1: lambda r: np_dequant_legacy(synth.Q5_1, r),
+}
+
+
+@pytest.mark.parametrize("dtype", sorted(NP_DECODERS), ids=lambda t: f"type{t}")
+def test_the_other_block_types_match_an_independent_numpy_dequantizer_bit_for_bit(dtype):
+    # sane synthetic blocks, then raw random bytes (any f16 pattern as a scale: finite outputs compared as bits)
+    raw = synth.synth_blocks(dtype, 200, synth.SplitMix64(11 + dtype))
+    assert np.array_equal(orc.dequantize(dtype, raw).view(np.uint32), NP_DECODERS[dtype](raw).view(np.uint32))
+    g = np.random.Generator(np.random.PCG64(dtype))
+    raw = g.integers(0, 256, size=synth.BLOCK_BYTES[dtype] * 64, dtype=np.uint8)
+    with np.errstate(all="ignore"):
+        a, b = orc.dequantize(dtype, raw), NP_DECODERS[dtype](raw)
+    fin = np.isfinite(b)
+    assert np.array_equal(a[fin].view(np.uint32), b[fin].view(np.uint32))
+    assert np.array_equal(np.isnan(a), np.isnan(b))
+
+
+def test_the_reference_known_answers_hold_for_the_numpy_decoders_too():
+    # gguf.rs:2549-2592, 2638-2652, 2431-2447: the same hand-computed blocks, so the second opinion is itself pinned
+    import json
+    import os
+    golden = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_known_answers.json")))
+    seen = set()
+    for case in golden["codec"]:
+        if case["type"] in NP_DECODERS:
+            out = NP_DECODERS[case["type"]](np.array(case["bytes"], dtype=np.uint8))
+            for i, v in case["expect"].items():
+                assert out[int(i)] == np.float32(v), (case["cite"], i)
+            seen.add(case["type"])
+    assert seen == set(NP_DECODERS)
+
+
 @pytest.mark.parametrize("seed", [1, 0x5EED])
 def test_q4_k_and_q8_0_match_an_independent_numpy_dequantizer_bit_for_bit(seed):
     rng = synth.SplitMix64(seed)
