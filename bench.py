@@ -9,8 +9,10 @@ layer banks (16 x 226.5 MB) and over a pool of distinct tokens, so that no step 
 expert weights in the 256 MB Infinity Cache from an earlier step: a layer is revisited only
 after the other 15 have streamed >= 425 MB through the cache.
 
-The whole rotation is captured once in a HIP graph and replayed (the serving-loop form);
---no-graph times eager launches instead.
+The timed steps are replays of a HIP graph that holds one rotation (or the whole timed region,
+if that is shorter) - the serving-loop form; they start where the warm-up steps stopped, so no
+(layer, token batch) pair of the warm-up is read again.  --no-graph times eager launches instead.
+`steady` adds the median and p10 / p90 of the per-layer time over >= 200 event-timed replays.
 
 Prints ONE JSON line (the contract the round driver reads), including
   roofline      the dominant kernel against the 8 TB/s HBM peak, its duration
@@ -34,10 +36,30 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
-# same command (profiles/olmoe_q4k_decode_hbm_traffic.txt), each scaled by what the counter
-# reads for the library's 256 MiB copy kernel.  Only for the workload/batch they were taken on.
-PROFILED_TRAFFIC = {("olmoe_q4k_decode", 1, "gate_up"): 19146025}
+# kernel-timing slot -> name of the kernel in the rocprofv3 summaries
+PROFILE_KERNEL_NAMES = {"gate_up": "gate_up_q_kernel", "down_combine": "down_combine_q_kernel"}
+
+
+def profiled_traffic(workload, tokens, slot):
+    """HBM bytes per launch of the dominant kernel, read from the committed summary of the rocprofv3 FETCH_SIZE /
+    WRITE_SIZE counter runs of this same command (profiles/<workload>_hbm_traffic.txt, column "traffic B": each
+    counter scaled by what it reads for the library's 256 MiB copy kernel).  None for a workload or batch size
+    no summary was taken on."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt" if tokens == 1 else f"{workload}_bt{tokens}_hbm_traffic.txt")
+    name = PROFILE_KERNEL_NAMES.get(slot)
+    if name is None or not os.path.exists(path):
+        return None
+    column = None
+    for line in open(path):
+        if line.startswith("kernel ") and "traffic B" in line:
+            head = line.split("  ")
+            column = [c.strip() for c in head if c.strip()].index("traffic B")
+        elif column is not None and line.startswith(name):
+            # the kernel name holds template arguments with spaces: count the numeric fields from the right
+            fields = line[line.index(">") + 1:].split() if ">" in line else line.split()[1:]
+            return int(float(fields[column - 1]))
+    return None
+
 
 WORKLOADS = {
     # name: (hidden, inter, experts, top_k, norm, bank type, router type)
@@ -60,8 +82,8 @@ BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "F32": 0, "Q6_K": 14, "Q5_1": 7, 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--steps", type=int, default=4096)
+    ap.add_argument("--warmup", type=int, default=256)
     ap.add_argument("--workload", default="olmoe_q4k_decode", choices=sorted(WORKLOADS))
     ap.add_argument("--tokens", type=int, default=1, help="tokens per step (decode batch)")
     ap.add_argument("--layers", type=int, default=16, help="distinct layer banks the steps rotate over")
@@ -167,26 +189,35 @@ def main() -> int:
             moe.forward_device(s % L, x_dev[s % pool], n, k, norm, out_dev)
 
     use_graph = not args.no_graph
-    graph = None
-    steps_per_launch = 1
-    if use_graph:
-        steps_per_launch = period if period <= 1024 else L
-        if args.stack:
-            steps_per_launch = min(pool, 16)
-        moe.graph_begin()
-        for s in range(steps_per_launch):
-            step(s)
-        graph = moe.graph_end()
+    layers_per_step = L if args.stack else 1
+    rotation = min(pool, 16) if args.stack else period  # steps after which the (layer, token batch) sequence repeats
+    first = args.warmup  # the timed steps go on where the warm-up stopped: none of its (layer, token batch) pairs is re-read
 
-    def run(nsteps, s0=0):
+    def capture(s_begin, count):
+        moe.graph_begin()
+        for s in range(s_begin, s_begin + count):
+            step(s)
+        return moe.graph_end()
+
+    # The timed region is EXACTLY args.steps steps: whole replays of one graph holding `per_graph` consecutive steps,
+    # plus one replay of a shorter graph for what is left over.  A graph is never longer than the timed region, so
+    # a short run (--steps 20) is still a graph replay.
+    per_graph = max(1, min(rotation if rotation <= 1024 else L, args.steps))
+    graph = tail_graph = None
+    replays, left = divmod(args.steps, per_graph)
+    if use_graph:
+        graph = capture(first, per_graph)
+        tail_graph = capture(first + replays * per_graph, left) if left else None
+
+    def timed_steps():
         if graph is not None:
-            for _ in range(nsteps // steps_per_launch):
+            for _ in range(replays):
                 graph.launch()
-            for s in range(nsteps % steps_per_launch):
-                step(s)
+            if tail_graph is not None:
+                tail_graph.launch()
         else:
-            for s in range(nsteps):
-                step(s0 + s)
+            for s in range(first, first + args.steps):
+                step(s)
 
     # one plain copy of known size on the same stream (untimed): under `rocprofv3 --pmc
     # FETCH_SIZE` / `WRITE_SIZE` its dispatch calibrates the counters the roofline's `traffic`
@@ -197,16 +228,46 @@ def main() -> int:
     M.synchronize()
     del probe_src, probe_dst
 
-    run(args.warmup)
+    # warm-up: args.warmup eager steps (steps 0 .. warmup-1), then, untimed, one replay of each graph so that its
+    # first-launch upload is not inside the timed region.  That replay reads the same pairs as the timed one will,
+    # per_graph steps earlier: with every step streaming `layer_bytes` of distinct weights, what a step needs has
+    # been pushed out of the 256 MB Infinity Cache again when (per_graph - 1) * layer_bytes exceeds it (`cache_cold`).
+    for s in range(args.warmup):
+        step(s)
+    if graph is not None:
+        graph.launch()
+        if tail_graph is not None:
+            tail_graph.launch()
     M.synchronize()
     moe.check()
     moe.timer_start()
     t0 = time.perf_counter()
-    run(args.steps)
+    timed_steps()
     ev_ms = moe.timer_stop()
     M.synchronize()
     wall = time.perf_counter() - t0
     moe.check()
+
+    ms_per_step = wall * 1e3 / args.steps / layers_per_step  # per layer
+    value = n * args.steps * layers_per_step / wall
+
+    # steady state: >= 200 replays of a graph over one whole rotation, each replay timed on the device between two
+    # HIP events (no host synchronisation in between): median and p10 / p90 of the per-layer time
+    steady = None
+    if use_graph:
+        rot_graph = graph if per_graph == rotation else capture(first, min(rotation, 1024))
+        rot_steps = per_graph if per_graph == rotation else min(rotation, 1024)
+        reps = max(200, -(-2048 // rot_steps))
+        rot_graph.launch()
+        M.synchronize()
+        us = np.sort(rot_graph.launch_timed(reps).astype(np.float64)) * 1e3 / (rot_steps * layers_per_step)
+        moe.check()
+        steady = {"steps": reps * rot_steps, "replays": reps, "steps_per_replay": rot_steps,
+                  "us_per_layer_p10": round(float(np.percentile(us, 10)), 3), "us_per_layer_p50": round(float(np.percentile(us, 50)), 3),
+                  "us_per_layer_p90": round(float(np.percentile(us, 90)), 3), "us_per_layer_min": round(float(us[0]), 3),
+                  "us_per_layer_max": round(float(us[-1]), 3)}
+        if rot_graph is not graph:
+            rot_graph.close()
 
     layers_per_step = L if args.stack else 1
     ms_per_step = wall * 1e3 / args.steps / layers_per_step  # per layer
@@ -259,10 +320,16 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
-                   "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "shared_inter": args.shared_inter, "hip_graph": use_graph, "steps_per_graph_launch": steps_per_launch,
+                   "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "shared_inter": args.shared_inter,
+                   "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
+                   "graph_replays_timed": (replays + (1 if left else 0)) if graph is not None else 0,
+                   "first_timed_step": first,
+                   "cache_cold": bool((per_graph - 1) * layer_bytes * layers_per_step > 256e6) if graph is not None else
+                                 bool(min(L, args.steps) * layer_bytes > 256e6),
                    "mean_distinct_experts_per_step": round(mean_distinct, 3)},
         "us_per_layer": round(ms_per_step * 1e3, 3),
         "event_ms_per_step": round(ev_ms / args.steps / layers_per_step, 6),
+        "steady": steady,
         "layer_algorithmic_bytes": int(layer_bytes),
         "layer_hbm_gbs": round(layer_gbs, 1),
         "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4),
@@ -270,7 +337,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1) if achieved else None,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
-                     "traffic": PROFILED_TRAFFIC.get((args.workload, n, dom)),
+                     "traffic": profiled_traffic(args.workload, n, dom),
                      "algorithmic_bytes_per_launch": int(gu_bytes), "avg_launch_us": round(gu_us, 3) if gu_us else None},
         "mfma": mfma,
         "device": M.device_name(),

@@ -58,7 +58,8 @@ enum mummu_status {
     MUMMU_ERR_ARG = 11,       /* null pointer or otherwise unusable argument */
     MUMMU_ERR_IO = 12,        /* a file cannot be opened, read or mapped, or ends inside its header */
     MUMMU_ERR_GGUF = 13,      /* the GGUF container breaks one of the reader's rules (gguf.rs:1226-1376) */
-    MUMMU_ERR_SAFETENSORS = 14 /* a safetensors header, index or expert group breaks a rule (safetensors.rs:180-320, 600-740) */
+    MUMMU_ERR_SAFETENSORS = 14, /* a safetensors header, index or expert group breaks a rule (safetensors.rs:180-320, 600-740) */
+    MUMMU_ERR_STALE = 15      /* a captured graph outlived the device buffers it points into (see mummu_graph_launch) */
 };
 
 /* Router arithmetic.  0: SparseMoe / SparseMoePerExpert (nn/moe.rs:144-150: f32 softmax,
@@ -355,11 +356,22 @@ MUMMU_API int mummu_device_synchronize(void);
 MUMMU_API int mummu_device_name(char *buf, size_t len);
 
 /* HIP-graph capture of whatever *_device calls are issued between begin and end on the
- * handle's own stream; launch replays it there. */
+ * handle's own stream; launch replays it there.  No counterpart in the reference.
+ *
+ * A captured graph holds raw pointers into the handle's workspace and weight buffers.  The
+ * *_device entry points never reallocate (they return MUMMU_ERR_TOKENS beyond max_tokens), but a
+ * host-pointer call with more tokens than the workspace holds regrows it, and loading a layer or a
+ * shared expert again replaces its buffers.  Either makes every graph captured before it stale:
+ * mummu_graph_launch then returns MUMMU_ERR_STALE and enqueues nothing; capture the graph again.
+ * graph_exec is an opaque library object (not a hipGraphExec_t); free it with mummu_graph_destroy. */
 MUMMU_API void *mummu_moe_stream(mummu_moe *h);
 MUMMU_API int mummu_graph_begin(mummu_moe *h);
 MUMMU_API int mummu_graph_end(mummu_moe *h, void **graph_exec);
 MUMMU_API int mummu_graph_launch(mummu_moe *h, void *graph_exec);
+/* `reps` replays enqueued back to back, a HIP event between neighbours, one synchronisation at the
+ * end: ms[i] = device milliseconds of replay i (1 <= reps <= 65536).  For benchmarks that report
+ * percentiles over replays. */
+MUMMU_API int mummu_graph_launch_timed(mummu_moe *h, void *graph_exec, int reps, float *ms);
 MUMMU_API void mummu_graph_destroy(void *graph_exec);
 
 /* HIP-event stopwatch on the handle's stream: elapsed milliseconds between start and stop. */

@@ -19,10 +19,10 @@ BLOCKS = {F32: (1, 4), F16: (1, 2), BF16: (1, 2), Q4_0: (32, 18), Q4_1: (32, 20)
 ROUTER_SPARSE_MOE, ROUTER_QWEN4EXP = 0, 1
 
 (OK, ERR_CONFIG, ERR_TYPE, ERR_BLOCKS, ERR_TOPK, ERR_SHAPE, ERR_NONFINITE, ERR_RANGE, ERR_NOT_LOADED, ERR_TOKENS,
- ERR_DEVICE, ERR_ARG, ERR_IO, ERR_GGUF, ERR_SAFETENSORS) = range(15)
+ ERR_DEVICE, ERR_ARG, ERR_IO, ERR_GGUF, ERR_SAFETENSORS, ERR_STALE) = range(16)
 
 STATUS_NAMES = ["ok", "config", "type", "blocks", "topk", "shape", "nonfinite", "range", "not_loaded", "tokens",
-                "device", "arg", "io", "gguf", "safetensors"]
+                "device", "arg", "io", "gguf", "safetensors", "stale"]
 
 
 class Config(C.Structure):
@@ -101,6 +101,7 @@ SIGNATURES = {
     "mummu_graph_begin": (_I, [_P]),
     "mummu_graph_end": (_I, [_P, C.POINTER(_P)]),
     "mummu_graph_launch": (_I, [_P, _P]),
+    "mummu_graph_launch_timed": (_I, [_P, _P, _I, C.POINTER(C.c_float)]),
     "mummu_graph_destroy": (None, [_P]),
     "mummu_timer_start": (_I, [_P]),
     "mummu_timer_stop": (_I, [_P, C.POINTER(C.c_float)]),

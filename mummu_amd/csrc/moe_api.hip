@@ -50,6 +50,12 @@ struct TimedLaunch {
     int slot;
 };
 
+// What mummu_graph_end hands out: the executable graph and the handle generation it was captured under.
+struct CapturedGraph {
+    hipGraphExec_t exec;
+    uint64_t generation;
+};
+
 }  // namespace
 
 namespace mummu {
@@ -89,6 +95,10 @@ struct mummu_moe {
     int32_t *sh_sorted = nullptr, *sh_tiles = nullptr, *sh_ntiles = nullptr;  // its one-expert work list
     int sh_max_tiles = 0;
 
+    // bumped whenever a device buffer a captured graph may point into is freed (workspace regrown, a layer's or
+    // a shared expert's weights replaced); a graph remembers the value it was captured under
+    uint64_t generation = 0;
+
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing = false;
     std::vector<TimedLaunch> timed;
@@ -115,6 +125,7 @@ bool router_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16; }
 size_t row_bytes_of(int t, int in_dim) { return (size_t)(in_dim / block_elems(t)) * (size_t)block_bytes(t); }
 
 void free_ws(mummu_moe *h) {
+    h->generation++;
     void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1],
                     h->xq.hi, h->xq.lo, h->xq.scale, h->xq.sum, h->actq.hi, h->actq.lo, h->actq.scale, h->actq.sum,
                     h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->act16, h->disp_scratch};
@@ -143,6 +154,7 @@ void free_ws(mummu_moe *h) {
 int ensure_shared_ws(mummu_moe *h) {
     if (h->sh_inter_max == 0 || h->sh_ws_tokens >= h->ws_tokens) return MUMMU_OK;
     HIPCHK(h, hipDeviceSynchronize());
+    h->generation++;
     void *sh[] = {h->sh_act, h->sh_y, h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, h->sh_actq.sum,
                   h->sh_act16, h->sh_sorted, h->sh_tiles, h->sh_ntiles};
     for (void *p : sh)
@@ -434,6 +446,31 @@ bool decode_three_launches(const mummu_moe *h, const Layer &L, int64_t n, int k)
     return !(n > 8 && router_fused_supported(E)) && want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k);
 }
 
+// What the three-launch decode form keeps between its launches: the router's logits, the routing the gate/up kernel
+// publishes, and the 16-bit activations of the block's input and of the experts' hidden rows.
+struct DecodeScratch {
+    float *logits;    // [n, E]
+    int32_t *ids;     // [n, k]
+    float *weights;   // [n, k]
+    QAct xq, actq;    // [n, H] and [n*k, I rounded up to 16]
+};
+
+// The two launches after the router's: gate/up with the routing inside, then down + combine.
+int decode_tail(mummu_moe *h, const Layer &L, const DecodeScratch &ws, int n, int k, int norm, const float *residual, float *out,
+                hipStream_t s) {
+    const ExpertBanks b = banks_of(h, L);
+    RouteInline route;
+    route.logits = ws.logits;
+    route.flavour = h->cfg.router_flavour;
+    route.norm = norm;
+    route.ids = ws.ids;
+    route.weights = ws.weights;
+    route.hits = L.hits;
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up_routed(b, ws.xq, route, n, k, ws.actq, h->flags, s));
+    LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, ws.actq, ws.ids, ws.weights, n, k, residual, out, s));
+    return MUMMU_OK;
+}
+
 // norm_gamma != nullptr (only where decode_three_launches holds): x is the raw residual stream and the
 // first launch applies the layer's RmsNorm itself.
 int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
@@ -459,16 +496,8 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
         const ExpertBanks b = banks_of(h, L);
         if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
             // ... and the gate/up kernel routes by itself: one launch less on the decode path
-            RouteInline route;
-            route.logits = h->logits;
-            route.flavour = h->cfg.router_flavour;
-            route.norm = norm;
-            route.ids = h->ids;
-            route.weights = h->weights;
-            route.hits = L.hits;
-            LAUNCH(h, K_GATE_UP, s, launch_gate_up_routed(b, h->xq, route, (int)n, k, h->actq, h->flags, s));
-            LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, h->actq, h->ids, h->weights, (int)n, k, residual, out, s));
-            return MUMMU_OK;
+            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq};
+            return decode_tail(h, L, ws, (int)n, k, norm, residual, out, s);
         }
         if (!batched && float_decode_fused(b, k)) {
             // float banks: the same two fusions
@@ -714,6 +743,7 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
 
     Layer &L = h->layers[layer];
     HIPCHK(h, hipDeviceSynchronize());
+    if (L.loaded) h->generation++;
     void *old[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits, L.sh_gate, L.sh_up, L.sh_down, L.sh_gatevec};
     for (void *p : old)
         if (p) (void)hipFree(p);
@@ -768,6 +798,7 @@ int mummu_moe_load_shared_expert(mummu_moe *h, int layer, int inter, const void 
     if (is_quant_type(down_type) && inter % 16) return fail(h, MUMMU_ERR_BLOCKS, "shared expert width must be a multiple of 16 for a quantized down matrix");
     Layer &L = h->layers[layer];
     HIPCHK(h, hipDeviceSynchronize());
+    h->generation++;  // a graph captured before this call does not run the shared expert (or points at the old one)
     void *old[] = {L.sh_gate, L.sh_up, L.sh_down, L.sh_gatevec};
     for (void *p : old)
         if (p) (void)hipFree(p);
@@ -1233,18 +1264,60 @@ int mummu_graph_end(mummu_moe *h, void **graph_exec) {
     hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
     (void)hipGraphDestroy(g);
     if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
-    *graph_exec = (void *)ex;
+    std::lock_guard<std::mutex> lock(h->mu);
+    *graph_exec = (void *)new CapturedGraph{ex, h->generation};
+    return MUMMU_OK;
+}
+
+// A captured graph holds raw pointers into the handle's workspace and weights: refuse to replay it once any of
+// them has been freed.
+static int graph_usable(mummu_moe *h, const CapturedGraph *g) {
+    if (g->generation != h->generation)
+        return fail(h, MUMMU_ERR_STALE, "this graph was captured before the handle's workspace grew or weights were reloaded; "
+                                        "it points at freed device memory - capture it again");
     return MUMMU_OK;
 }
 
 int mummu_graph_launch(mummu_moe *h, void *graph_exec) {
     if (!h || !graph_exec) return fail(h, MUMMU_ERR_ARG, "null argument");
-    HIPCHK(h, hipGraphLaunch((hipGraphExec_t)graph_exec, h->stream));
+    const CapturedGraph *g = (const CapturedGraph *)graph_exec;
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = graph_usable(h, g);
+    if (rc) return rc;
+    HIPCHK(h, hipGraphLaunch(g->exec, h->stream));
+    return MUMMU_OK;
+}
+
+int mummu_graph_launch_timed(mummu_moe *h, void *graph_exec, int reps, float *ms) {
+    if (!h || !graph_exec || !ms) return fail(h, MUMMU_ERR_ARG, "null argument");
+    if (reps < 1 || reps > 65536) return fail(h, MUMMU_ERR_ARG, "reps must be in 1..=65536");
+    const CapturedGraph *g = (const CapturedGraph *)graph_exec;
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = graph_usable(h, g);
+    if (rc) return rc;
+    std::vector<hipEvent_t> ev((size_t)reps + 1, nullptr);
+    hipError_t e = hipSuccess;
+    for (auto &x : ev)
+        if (e == hipSuccess) e = hipEventCreate(&x);
+    // all replays are enqueued back to back with an event between neighbours; one synchronisation at the end
+    if (e == hipSuccess) e = hipEventRecord(ev[0], h->stream);
+    for (int i = 0; i < reps && e == hipSuccess; i++) {
+        e = hipGraphLaunch(g->exec, h->stream);
+        if (e == hipSuccess) e = hipEventRecord(ev[(size_t)i + 1], h->stream);
+    }
+    if (e == hipSuccess) e = hipEventSynchronize(ev[(size_t)reps]);
+    for (int i = 0; i < reps && e == hipSuccess; i++) e = hipEventElapsedTime(&ms[i], ev[(size_t)i], ev[(size_t)i + 1]);
+    for (auto x : ev)
+        if (x) (void)hipEventDestroy(x);
+    if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("timed graph replay: ") + hipGetErrorString(e));
     return MUMMU_OK;
 }
 
 void mummu_graph_destroy(void *graph_exec) {
-    if (graph_exec) (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+    if (!graph_exec) return;
+    CapturedGraph *g = (CapturedGraph *)graph_exec;
+    (void)hipGraphExecDestroy(g->exec);
+    delete g;
 }
 
 int mummu_timer_start(mummu_moe *h) {

@@ -362,6 +362,13 @@ class Graph:
     def launch(self):
         self._moe._check(self._moe._lib.mummu_graph_launch(self._moe._h, self._g))
 
+    def launch_timed(self, reps: int) -> np.ndarray:
+        """`reps` replays back to back, device milliseconds of each (HIP events between neighbours)."""
+        ms = np.zeros(reps, dtype=np.float32)
+        self._moe._check(self._moe._lib.mummu_graph_launch_timed(self._moe._h, self._g, reps,
+                                                                 ms.ctypes.data_as(C.POINTER(C.c_float))))
+        return ms
+
     def close(self):
         if self._g:
             self._moe._lib.mummu_graph_destroy(self._g)

@@ -4,13 +4,12 @@ expert geometry), through the C ABI, against the CPU oracle on the same seeded i
   C1  OLMoE f32, 16 tokens                      (float GEMV path, tolerance 1e-5)
   C2  OLMoE f16, 512 tokens, uniform router      (dispatch + grouped MFMA GEMM, 2e-3)
   C3  OLMoE Q4_K experts, f16 router, 1/4/8 tok  (packed integer GEMV, 2e-3)
-  C4  16-layer OLMoE stack, RmsNorm + residual, Q8_0, decode 1 token and prefill
+  C4  16-layer OLMoE stack, RmsNorm + residual, Q8_0, decode 1 token and prefill 256 tokens
   C5  Qwen3-A3B shape, Q4_K, 64 tokens, Zipf-skewed routing, norm_topk_prob=true
 
 Routing ids must be bit-exact; outputs are held to the stated relative error measured as the
-reference measures it (experts.rs:1264-1271).  Full-size f64 references are computed for a
-subset of tokens where the whole batch would take the oracle too long; every token is still
-compared with the oracle's f32 result.
+reference measures it (experts.rs:1264-1271), every token and every element against the f64
+product of the dequantized weights.
 """
 import numpy as np
 import pytest
@@ -81,9 +80,11 @@ def test_c2_olmoe_f16_prefill_512_tokens_grouped_gemm():
     out, ids, w, _ = orc.moe_forward(banks, router, orc.F16, x, k, False)
     assert np.array_equal(r.ids, ids.astype(np.int32)) and np.array_equal(bits(r.weights), bits(w))
     assert int(hits.sum()) == n * k and hits.tolist() == np.bincount(ids.reshape(-1), minlength=E).tolist()
-    rows = np.r_[0:12, 250:256, 500:512]
-    check_rows(got, banks, ids, w, x, rows, 2e-3)
-    # every token against the oracle's f32 result, scaled by the row's magnitude
+    # every token, every element, by the reference's measure: all 4096 assignments, so every row position of
+    # every tile of the grouped GEMM is checked
+    check_rows(got, banks, ids, w, x, slice(0, n), 2e-3)
+    check_rows(got_97, banks, ids, w, x, slice(0, 97), 2e-3)
+    # and against the oracle's f32 result, scaled by the row's magnitude
     scale = np.sqrt((out.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     assert (np.abs(got - out) / scale).max() <= 2e-2
     assert np.abs(got - out).mean() / np.abs(out).mean() <= 2e-3
@@ -175,8 +176,11 @@ def c4_layers(L, seed):
     return layers
 
 
-def run_c4(L, n, seed):
-    """GPU stack vs the oracle run layer by layer.  Returns (got, gpu ids [L,n,k], want, oracle ids,
+def run_c4(L, n, seed, layer_tol=None):
+    """GPU stack vs the oracle run layer by layer.  With `layer_tol` every layer is also run on its own
+    on the ORACLE's input to that layer and every element of its output is held to `layer_tol` of the f64
+    reference by the reference's measure (experts.rs:1264-1271) - identical inputs, so no error carried
+    over from the layers before.  Returns (got, gpu ids [L,n,k], want, oracle ids,
     oracle routing margins [L,n]): margin = the smallest relative gap (p_j - p_{j+1}) / p_j between
     neighbours among the oracle's k+1 most probable experts - the slack before either the selected
     set or the slot order can change."""
@@ -199,6 +203,8 @@ def run_c4(L, n, seed):
             assert np.array_equal(bits(r.weights), bits(w))
             p = np.sort(np.exp(lg.astype(np.float64) - lg.max(axis=1, keepdims=True)), axis=1)[:, ::-1]
             margins.append(((p[:, :k] - p[:, 1:k + 1]) / p[:, :k]).min(axis=1))
+            if layer_tol is not None:
+                check_rows(m.forward(h2, k, False, layer=l), banks, ids, w, h2, slice(0, n), layer_tol)
             oids.append(ids.astype(np.int32))
             cur = (cur + moe).astype(np.float32)
     return got, gids, cur, np.stack(oids), np.stack(margins)
@@ -230,8 +236,11 @@ def test_c4_sixteen_layer_q8_0_stack_decode():
     check_stack(*run_c4(16, 1, 400), tol=2e-3)  # integer GEMV with 16-bit activations: far inside
 
 
-def test_c4_q8_0_stack_prefill_256_tokens_two_layers():
-    check_stack(*run_c4(2, 256, 500), tol=9e-3)
+def test_c4_sixteen_layer_q8_0_stack_prefill_256_tokens():
+    # the configuration as stated: 16 layers, 256 tokens.  Layer by layer on identical inputs every element is
+    # inside 2e-3 by the reference's measure; the residual stream after 16 layers, where each layer's rounding
+    # feeds the next, is held per row (see check_stack for the unit)
+    check_stack(*run_c4(16, 256, 500, layer_tol=2e-3), tol=9e-3)
 
 
 @pytest.mark.parametrize("H,I,E,k,gt", [(2048, 256, 64, 8, M.Q4_K), (512, 128, 8, 2, M.Q8_0), (1280, 128, 16, 4, M.Q5_0),
@@ -277,7 +286,7 @@ def test_c4_q8_0_prefill_layer_against_the_f64_reference():
         got = m.forward(x, k, False)
     banks = orc.LayerBanks(H, I, E, gate, up, down, orc.Q8_0)
     _, ids, w, _ = orc.moe_forward(banks, router, orc.F16, x, k, False)
-    check_rows(got, banks, ids, w, x, np.r_[0:10, 120:130, 246:256], 2e-3)
+    check_rows(got, banks, ids, w, x, slice(0, 256), 2e-3)
 
 
 def test_c5_qwen3_a3b_shape_q4k_zipf_routing():

@@ -404,3 +404,46 @@ def test_gate_energy_with_rows_wider_than_the_default_lds_window():
     pre = x.astype(np.float64) @ gate[1].astype(np.float64).T
     want = ((pre / (1.0 + np.exp(-pre))) ** 2).sum(axis=1)
     assert np.all(np.abs(got - want) <= 1e-5 * want)
+
+
+def test_a_graph_is_refused_once_the_buffers_it_points_into_are_gone():
+    # a captured graph holds raw workspace and weight pointers: a host call that regrows the workspace, or a reload
+    # of the layer, must make launch fail with MUMMU_ERR_STALE instead of replaying over freed memory
+    from mummu_amd import _lib
+    H, I, E, k = 256, 64, 8, 2
+    rng = synth.SplitMix64(77)
+    banks = [synth.synth_bank(synth.Q8_0, ne, rng) for ne in ([H, I, E], [H, I, E], [I, H, E])]
+    router = rng.normal(E * H, 0.0, 0.05).astype(np.float16).reshape(E, H)
+    x = rng.normal(2 * H).reshape(2, H)
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=4) as m:
+        m.load_layer(0, router, M.F16, banks[0], M.Q8_0, banks[1], M.Q8_0, banks[2], M.Q8_0)
+        want = m.forward(x, k, False)
+        xd, od = M.DeviceBuffer.from_array(x), M.DeviceBuffer(x.nbytes)
+
+        def capture():
+            m.graph_begin()
+            m.forward_device(0, xd, 2, k, False, od)
+            return m.graph_end()
+
+        g = capture()
+        g.launch()
+        m.check()
+        assert np.array_equal(bits(od.download(np.float32, x.shape)), bits(want))
+        ms = g.launch_timed(3)
+        assert ms.shape == (3,) and np.all(ms > 0)
+        m.forward(rng.normal(64 * H).reshape(64, H), k, False)  # 64 tokens > max_tokens: the workspace is regrown
+        with pytest.raises(M.MoeError) as e:
+            g.launch()
+        assert e.value.code == _lib.ERR_STALE
+        with pytest.raises(M.MoeError):
+            g.launch_timed(2)
+        g.close()
+        g = capture()  # captured again, it runs
+        g.launch()
+        m.check()
+        assert np.array_equal(bits(od.download(np.float32, x.shape)), bits(want))
+        m.load_layer(0, router, M.F16, banks[0], M.Q8_0, banks[1], M.Q8_0, banks[2], M.Q8_0)  # same bytes, new buffers
+        with pytest.raises(M.MoeError) as e:
+            g.launch()
+        assert e.value.code == _lib.ERR_STALE
+        g.close()
