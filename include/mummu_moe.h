@@ -196,6 +196,20 @@ MUMMU_API int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, in
  * reported synchronously here; mummu_moe_check() reads the flag back. */
 MUMMU_API int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_t n_tokens, int top_k,
                                        int norm_topk_prob, float *out_dev, void *stream);
+/* mummu_moe_forward_device for callers that cannot allocate device memory and do not want a workspace that was
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments, same result bits.  What its three kernels hand to one another (router logits, the
+ * routing, the 16-bit activations) lives in one static device array of MUMMU_NOALLOC_SCRATCH_BYTES that every GPU
+ * the library runs on holds until the process ends; the call itself calls no hipMalloc / hipFree and no allocating
+ * library routine.  Limits: the decode form only - at most MUMMU_NOALLOC_MAX_TOKENS tokens, block-quantized
+ * gate / up / down banks, hidden a multiple of 64, top_k <= 16, no shared expert on the layer, kernel timing off -
+ * and a call whose intermediate data would not fit the array is refused (MUMMU_ERR_TOKENS / MUMMU_ERR_CONFIG, with
+ * a message).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two
+ * handles, two threads) race; issue them on one stream.  mummu_moe_last_routing does not see this call's routing. */
+#define MUMMU_NOALLOC_SCRATCH_BYTES (4u << 20)
+#define MUMMU_NOALLOC_MAX_TOKENS 8
+MUMMU_API int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const float *x_dev, int64_t n_tokens, int top_k,
+                                               int norm_topk_prob, float *out_dev, void *stream);
 /* ExpertExec::run_tensor_resident (nn/moe.rs:360-371, DeviceExpert's at :470-501): the SwiGLU of one expert on rows
  * that are already on this device, the result left there; only enqueues on `stream`.  rows <= max_tokens. */
 MUMMU_API int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_dev, int64_t rows, int hidden,

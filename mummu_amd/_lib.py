@@ -88,6 +88,7 @@ SIGNATURES = {
     "mummu_dequantize": (_I, [_I, _P, _SZ, _P]),
     "mummu_moe_dequantize_expert": (_I, [_P, _I, _I, _I, _P]),
     "mummu_moe_forward_device": (_I, [_P, _I, _P, _I64, _I, _I, _P, _P]),
+    "mummu_moe_forward_device_noalloc": (_I, [_P, _I, _P, _I64, _I, _I, _P, _P]),
     "mummu_moe_stack_forward_device": (_I, [_P, _P, _I64, _I, _I, _P, _P]),
     "mummu_moe_check": (_I, [_P, _P]),
     "mummu_moe_last_routing": (_I, [_P, _I64, _I, _P, _P]),

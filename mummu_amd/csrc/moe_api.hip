@@ -62,6 +62,11 @@ namespace mummu {
 thread_local LaunchTiming g_launch_timing;
 }
 
+// Scratch of the entry point that allocates nothing (mummu_moe_forward_device_noalloc): what its three kernels hand to one
+// another lives here instead of in hipMalloc'ed workspace.  Every GPU holds its own copy until the process ends.  In host
+// code this name is only a stand-in for the symbol: the address kernels are given comes from hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[MUMMU_NOALLOC_SCRATCH_BYTES];
+
 struct mummu_moe {
     mummu_moe_config cfg{};
     std::vector<Layer> layers;
@@ -119,6 +124,26 @@ int fail(mummu_moe *h, int code, const std::string &msg) {
         if (e_ != hipSuccess)                                                                              \
             return fail(h, MUMMU_ERR_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_));            \
     } while (0)
+
+// The device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+unsigned char *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(mummu_moe *h, unsigned char **out) {
+    int dev = -1;
+    HIPCHK(h, hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(h, MUMMU_ERR_DEVICE, "device index " + std::to_string(dev) + " out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        HIPCHK(h, hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(h, MUMMU_ERR_DEVICE, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_scratch_ptr[dev] = (unsigned char *)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MUMMU_OK;
+}
 
 bool bank_type_ok(int t) { return block_elems(t) > 0; }  // F32, F16, BF16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K
 bool router_type_ok(int t) { return t == T_F32 || t == T_F16 || t == T_BF16; }
@@ -691,6 +716,11 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     if (hipMalloc(&h->flags, sizeof(int32_t) * kFlagWords) != hipSuccess) return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(flags) failed"));
     int rc = reset_flags(h);
     if (rc) return bail(rc);
+    {
+        // resolve the static scratch's address on this device now, outside any stream capture
+        unsigned char *unused = nullptr;
+        if ((rc = static_scratch(h, &unused))) return bail(rc);
+    }
     rc = ensure_ws(h, cfg->max_tokens, (int64_t)cfg->max_tokens * cfg->num_experts_per_tok, cfg->num_experts);
     if (rc) return bail(rc);
     *out = h;
@@ -1166,6 +1196,51 @@ int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_
     if ((rc = check_device_call(h, n, top_k, x_dev, out_dev))) return rc;
     if (n == 0) return MUMMU_OK;
     return forward_impl(h, layer, x_dev, n, top_k, norm, nullptr, out_dev, (hipStream_t)stream);
+}
+
+int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const float *x_dev, int64_t n, int top_k, int norm, float *out_dev,
+                                     void *stream) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    int rc = check_layer(h, layer);
+    if (rc) return rc;
+    if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
+    if (!x_dev || !out_dev) return fail(h, MUMMU_ERR_ARG, "null device pointer");
+    if (((uintptr_t)x_dev & 15) || ((uintptr_t)out_dev & 15)) return fail(h, MUMMU_ERR_ARG, "device buffers must be 16-byte aligned");
+    if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
+    if (n == 0) return MUMMU_OK;
+    if (h->timing) return fail(h, MUMMU_ERR_ARG, "kernel timing creates events; disable it for the call that allocates nothing");
+    const Layer &L = h->layers[layer];
+    if (L.sh_loaded) return fail(h, MUMMU_ERR_CONFIG, "the call that allocates nothing does not serve a layer with a shared expert");
+    if (n > MUMMU_NOALLOC_MAX_TOKENS || !decode_three_launches(h, L, n, top_k))
+        return fail(h, n > MUMMU_NOALLOC_MAX_TOKENS ? MUMMU_ERR_TOKENS : MUMMU_ERR_CONFIG,
+                    "the call that allocates nothing serves the decode form only: at most " + std::to_string(MUMMU_NOALLOC_MAX_TOKENS) +
+                        " tokens, block-quantized banks, hidden a multiple of 64, top_k <= 16");
+    // carve the static array: every piece starts on a 256-byte boundary
+    const size_t E = (size_t)h->cfg.num_experts, H = (size_t)h->cfg.hidden_size, I = (size_t)h->cfg.expert_intermediate_size;
+    const size_t nn = (size_t)n, na = nn * (size_t)top_k, xe = nn * H, ae = na * ((I + 15) / 16 * 16);
+    const size_t want[] = {sizeof(float) * nn * E, sizeof(int32_t) * na, sizeof(float) * na,
+                           xe, xe, sizeof(float) * (xe / 16), sizeof(int32_t) * (xe / 16),
+                           ae, ae, sizeof(float) * (ae / 16), sizeof(int32_t) * (ae / 16)};
+    size_t off[sizeof(want) / sizeof(want[0]) + 1] = {0};
+    for (size_t i = 0; i < sizeof(want) / sizeof(want[0]); i++) off[i + 1] = (off[i] + want[i] + 255) / 256 * 256;
+    const size_t need = off[sizeof(want) / sizeof(want[0])];
+    if (need > MUMMU_NOALLOC_SCRATCH_BYTES)
+        return fail(h, MUMMU_ERR_TOKENS, "this call needs " + std::to_string(need) + " bytes between its kernels; the static scratch holds " +
+                                             std::to_string((size_t)MUMMU_NOALLOC_SCRATCH_BYTES));
+    unsigned char *base = nullptr;
+    if ((rc = static_scratch(h, &base))) return rc;
+    DecodeScratch ws;
+    ws.logits = (float *)(base + off[0]);
+    ws.ids = (int32_t *)(base + off[1]);
+    ws.weights = (float *)(base + off[2]);
+    ws.xq = QAct{(int8_t *)(base + off[3]), (int8_t *)(base + off[4]), (float *)(base + off[5]), (int32_t *)(base + off[6])};
+    ws.actq = QAct{(int8_t *)(base + off[7]), (int8_t *)(base + off[8]), (float *)(base + off[9]), (int32_t *)(base + off[10])};
+    hipStream_t s = (hipStream_t)stream;
+    // the kernels write every word of the scratch they later read (nothing in it has to start at zero)
+    LAUNCH(h, K_ROUTER_LOGITS, s,
+           launch_router_logits(x_dev, L.router, L.router_type, ws.logits, (int)n, (int)H, (int)E, ws.xq, s, nullptr, h->cfg.rms_norm_eps, nullptr));
+    return decode_tail(h, L, ws, (int)n, top_k, norm, nullptr, out_dev, s);
 }
 
 int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_dev, int64_t rows, int hidden, float *out_dev,

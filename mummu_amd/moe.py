@@ -297,6 +297,13 @@ class SparseMoe:
         self._check(self._lib.mummu_moe_forward_device(self._h, layer, x_dev.ptr, n, top_k, int(norm_topk_prob),
                                                        out_dev.ptr, self.stream))
 
+    def forward_device_noalloc(self, layer: int, x_dev: "DeviceBuffer", n: int, top_k: int, norm_topk_prob: bool,
+                               out_dev: "DeviceBuffer"):
+        """forward_device through the entry point that allocates nothing: the kernels' intermediate data lives in the
+        library's static device array (decode form only; see include/mummu_moe.h)."""
+        self._check(self._lib.mummu_moe_forward_device_noalloc(self._h, layer, x_dev.ptr, n, top_k, int(norm_topk_prob),
+                                                               out_dev.ptr, self.stream))
+
     def expert_run_device(self, layer: int, expert: int, x_dev: "DeviceBuffer", rows: int, out_dev: "DeviceBuffer"):
         """ExpertExec::run_tensor_resident (nn/moe.rs:360-371): rows already on the device, result left there."""
         self._check(self._lib.mummu_expert_run_device(self._h, layer, expert, x_dev.ptr, rows, self.config.hidden_size,
