@@ -210,6 +210,17 @@ MUMMU_API int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_d
 #define MUMMU_NOALLOC_MAX_TOKENS 8
 MUMMU_API int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const float *x_dev, int64_t n_tokens, int top_k,
                                                int norm_topk_prob, float *out_dev, void *stream);
+/* A decode step of ONE token on block-quantized banks takes two launches where the device allows it: router + routing +
+ * gate/up in one kernel whose workgroups pass the router logits to one another through the L2 of the XCD they share,
+ * then down + combine.  No counterpart in the reference.  enable = 0: always three launches (router logits in a launch
+ * of their own); 1 (default): two launches at one token; 2: two launches at every size the kernel takes (up to 8
+ * tokens; slower than three from 2 tokens on).  spin_ticks bounds how long a workgroup waits for the others' logits, in
+ * 10 ns units (default 5000), before it computes them itself - the result has the same bits either way, and with
+ * spin_ticks = 0 no workgroup looks for the others' logits at all.  _state reports whether the two-launch form is in
+ * use on this device (it is not when workgroups with equal ids modulo 8 do not share an XCD) and returns-and-clears
+ * the number of workgroups that gave up waiting. */
+MUMMU_API int mummu_moe_set_router_exchange(mummu_moe *h, int enable, unsigned spin_ticks);
+MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbacks);
 /* ExpertExec::run_tensor_resident (nn/moe.rs:360-371, DeviceExpert's at :470-501): the SwiGLU of one expert on rows
  * that are already on this device, the result left there; only enqueues on `stream`.  rows <= max_tokens. */
 MUMMU_API int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_dev, int64_t rows, int hidden,

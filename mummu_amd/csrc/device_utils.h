@@ -33,13 +33,16 @@ constexpr int kWave = 64;
 
 // Phase marks for kernel timing studies.  A normal build compiles them away; with
 // -DMUMMU_TRACE every wave stores the constant 100 MHz wall clock at each mark into a caller-provided buffer
-// (8 slots per wave), set per translation unit through mummu_trace_set_<unit>().
+// (16 slots per wave), set per translation unit through mummu_trace_set_<unit>().
 #ifdef MUMMU_TRACE
 static __device__ long long *g_trace_buf = nullptr;
+#ifndef MUMMU_TRACE_MASK
+#define MUMMU_TRACE_MASK 0xFFFF  // which of the 16 marks are compiled in (every mark costs a clock read and a store)
+#endif
 #define MUMMU_PHASE(ph)                                                                                           \
     do {                                                                                                          \
-        if (g_trace_buf && (threadIdx.x & 63) == 0)                                                               \
-            g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + \
+        if (((MUMMU_TRACE_MASK >> (ph)) & 1) && g_trace_buf && (threadIdx.x & 63) == 0)                           \
+            g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16 + \
                         (ph)] = wall_clock64();                                                                       \
     } while (0)
 #define MUMMU_TRACE_UNIT(name)                                                                      \
@@ -60,7 +63,7 @@ static __device__ long long *g_trace_buf = nullptr;
         tm_acc_[7] = tm_last_;                                                                                    \
         if (g_trace_buf && (threadIdx.x & 63) == 0)                                                               \
             for (int i_ = 0; i_ < 8; i_++)                                                                        \
-                g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + i_] = tm_acc_[i_]; \
+                g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16 + i_] = tm_acc_[i_]; \
     } while (0)
 #else
 #define MUMMU_PHASE(ph) do { } while (0)
@@ -272,6 +275,26 @@ __device__ inline void dispatch_group(int g, F &&f) {
     case 2: f(std::integral_constant<int, 2>{}); break;
     default: f(std::integral_constant<int, 1>{}); break;
     }
+}
+
+// Maximum of a signed integer over the wave, every lane gets it.  The four steps inside a 16-lane row are single
+// v_max_i32 instructions reading their first operand through DPP (written as such: left to itself the compiler makes a
+// move and a maximum of each; the s_nop covers the two wait states a DPP read needs after a write of the same
+// register), then the two lane swaps across rows.  Non-negative finite floats order like their bit patterns, so this
+// also serves as their maximum.
+__device__ inline int wave_max_i32(int v) {
+    asm("s_nop 1\n\tv_max_i32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_i32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_i32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_i32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf"
+        : "+v"(v));
+    // (the swaps return unsigned words: compare them as the signed values they are)
+    auto a = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    const int a0 = (int)a[0], a1 = (int)a[1];
+    v = a0 > a1 ? a0 : a1;
+    auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    const int b0 = (int)b[0], b1 = (int)b[1];
+    return b0 > b1 ? b0 : b1;
 }
 
 // Maximum over the wave, every lane gets it: four DPP steps inside each 16-lane row, then the

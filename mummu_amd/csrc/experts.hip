@@ -58,57 +58,16 @@ static hipError_t with_bank_type(int type, F &&f) {
 #undef MUMMU_TYPE_CASE
 }
 
-// ------------------------------------------------------------------------------------------
-// gate/up, quantized banks: NIT iterations of rows_per_it rows per wave; the workgroup's
-// rows_per_block = waves*NIT*rows_per_it output rows are a whole number of 16-element
-// activation blocks, quantized for the down projection in the epilogue.
-// ------------------------------------------------------------------------------------------
-// RJN > 0: the kernel routes by itself, RJN experts per lane of the routing wave (see RouteInline).
-template <int WT, int UPL, int NIT, bool ACTQ, int RJN = 0>
-__global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restrict__ gate,
-                                                         const uint8_t *__restrict__ up, QAct xq,
-                                                         const int32_t *__restrict__ ids, int k, int fixed_expert,
-                                                         int hidden, int inter, int n_experts,
-                                                         float *__restrict__ act, QAct actq,
-                                                         int32_t *__restrict__ flags, RouteInline route) {
-    constexpr bool ROUTE = RJN > 0;
-    constexpr int JN = ROUTE ? RJN : 1;
-    extern __shared__ float s_act[];  // rows_per_block floats
-    __shared__ __attribute__((aligned(16))) RouteScratch<JN> s_route;
-    __shared__ int s_ids[64];
-    __shared__ float s_w[64];
-    MUMMU_PHASE(0);
+// The gate/up products of one (token, expert) assignment `a` for this workgroup's tile of output rows, given the
+// lane's share `la` of the token's 16-bit activations: NIT iterations of rows_per_it rows per wave, then
+// silu(gate) * up per row, written as f32 (act) or staged in LDS (s_act, rows_per_block floats) and re-quantized to
+// 16-bit blocks for the down product (ACTQ).
+template <int WT, int UPL, int NIT, bool ACTQ>
+__device__ __forceinline__ void gate_up_tile(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, int e, int a,
+                                             const LaneAct<UPL> &la, const RowSplit &rs, int hidden, int inter,
+                                             float *__restrict__ act, const QAct &actq, float *s_act) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.z;  // grid = (slot, row tile, token)
-    const int a = t * gridDim.x + blockIdx.x;
-    const RowSplit rs = row_split(hidden);
     const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
-    LaneAct<UPL> la;  // the token's activations do not depend on the routing: fetch them first
-    load_lane_act<WT, UPL>(xq, (size_t)t, hidden, unit0, rs.units, la);
-    if (ROUTE) {
-        // wave 0 routes token t from its logits; everybody else already has the activations coming
-        if (wave == 0) {
-            float l[JN];
-#pragma unroll
-            for (int j = 0; j < JN; j++) l[j] = lane + 64 * j < n_experts ? route.logits[(size_t)t * n_experts + lane + 64 * j] : 0.0f;
-            route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
-            wave_lds_sync();
-            if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
-                const int id = s_ids[lane];
-                route.ids[(size_t)t * k + lane] = id;
-                route.weights[(size_t)t * k + lane] = s_w[lane];
-                if (route.hits) atomicAdd(&route.hits[id], 1ULL);
-            }
-            MUMMU_PHASE(6);
-        }
-        __syncthreads();
-        MUMMU_PHASE(7);
-    }
-    const int e = ROUTE ? s_ids[blockIdx.x] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
-    if ((unsigned)e >= (unsigned)n_experts) {
-        if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
-        return;
-    }
     const int rows_per_wave = NIT * rs.rows_per_it;
     const int rows_per_block = rows_per_wave * (blockDim.x >> 6);
     const int block_row0 = blockIdx.y * rows_per_block;
@@ -188,6 +147,352 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     MUMMU_PHASE(5);
 }
 
+// ------------------------------------------------------------------------------------------
+// gate/up, quantized banks: NIT iterations of rows_per_it rows per wave; the workgroup's
+// rows_per_block = waves*NIT*rows_per_it output rows are a whole number of 16-element
+// activation blocks, quantized for the down projection in the epilogue.
+// ------------------------------------------------------------------------------------------
+// RJN > 0: the kernel routes by itself, RJN experts per lane of the routing wave (see RouteInline).
+template <int WT, int UPL, int NIT, bool ACTQ, int RJN = 0>
+__global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restrict__ gate,
+                                                         const uint8_t *__restrict__ up, QAct xq,
+                                                         const int32_t *__restrict__ ids, int k, int fixed_expert,
+                                                         int hidden, int inter, int n_experts,
+                                                         float *__restrict__ act, QAct actq,
+                                                         int32_t *__restrict__ flags, RouteInline route) {
+    constexpr bool ROUTE = RJN > 0;
+    constexpr int JN = ROUTE ? RJN : 1;
+    extern __shared__ float s_act[];  // rows_per_block floats
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> s_route;
+    __shared__ int s_ids[64];
+    __shared__ float s_w[64];
+    MUMMU_PHASE(0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.z;  // grid = (slot, row tile, token)
+    const int a = t * gridDim.x + blockIdx.x;
+    const RowSplit rs = row_split(hidden);
+    const int unit0 = lane & (rs.group - 1);
+    LaneAct<UPL> la;  // the token's activations do not depend on the routing: fetch them first
+    load_lane_act<WT, UPL>(xq, (size_t)t, hidden, unit0, rs.units, la);
+    if (ROUTE) {
+        // wave 0 routes token t from its logits; everybody else already has the activations coming
+        if (wave == 0) {
+            float l[JN];
+#pragma unroll
+            for (int j = 0; j < JN; j++) l[j] = lane + 64 * j < n_experts ? route.logits[(size_t)t * n_experts + lane + 64 * j] : 0.0f;
+            route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
+            wave_lds_sync();
+            if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
+                const int id = s_ids[lane];
+                route.ids[(size_t)t * k + lane] = id;
+                route.weights[(size_t)t * k + lane] = s_w[lane];
+                if (route.hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&route.hits[id], 1ULL);
+            }
+            MUMMU_PHASE(6);
+        }
+        __syncthreads();
+        MUMMU_PHASE(7);
+    }
+    const int e = ROUTE ? s_ids[blockIdx.x] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
+    if ((unsigned)e >= (unsigned)n_experts) {
+        if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
+        return;
+    }
+    gate_up_tile<WT, UPL, NIT, ACTQ>(gate, up, e, a, la, rs, hidden, inter, act, actq, s_act);
+}
+
+// ------------------------------------------------------------------------------------------
+// Decode, first of two launches: router logits, routing and gate/up in ONE kernel.
+//
+// The grid is the gate/up grid (slot, row tile, token).  Workgroups are dealt to the chip's 8 XCDs round-robin
+// by linear id, and the workgroups of one XCD share its L2.  Those of one token on one XCD split the token's E
+// router rows between them (a wave per row, the fixed summation order of router.hip), publish each logit as a
+// 16-byte record in a table of their XCD, and wave 0 of every workgroup collects the E records of its XCD before it
+// routes.  Producer and consumer sit behind the same L2, so a plain store followed by a device-scope load (which
+// bypasses the CU's own L1) sees the record within a fraction of a microsecond, where a round trip through memory
+// between XCDs costs about as much as a kernel launch.  The table is indexed by the XCD the workgroup actually runs
+// on (read from the hardware id register): a workgroup never looks for records on another XCD.
+//
+// A record = {logit bits, epoch low, epoch high, check word}.  The epoch is a 64-bit counter in device memory that the
+// launch after this one increments (down_combine), so records of earlier launches never match and the table needs no
+// clearing.  The wait is bounded (spin_ticks of the 100 MHz clock): a wave that does not find its records - workgroups
+// placed otherwise than assumed, or a tiny spin_ticks from a test - computes the missing logits itself, same bits.
+//
+// Every wave also loads the token's f32 row: with a gamma it is normalised first (RmsNorm, the RmsNorm kernel's bits),
+// wave c quantizes the c-th 512-element chunk to the 16-bit blocks of QAct into LDS, which feed the integer dots.
+// hidden <= 2048 and a multiple of 64; (slots * row tiles) a multiple of 8.
+// ------------------------------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ inline u32x4 load_device_scope_b128(const u32x4 *p) {
+    u32x4 r;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p) : "memory");
+    return r;
+}
+
+__device__ inline unsigned xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u; }  // HW_REG_XCC_ID[3:0]
+
+__device__ inline u32x4 exchange_record(float logit, unsigned long long epoch, unsigned what) {
+    u32x4 r;
+    r.x = __float_as_uint(logit);
+    r.y = (unsigned)epoch;
+    r.z = (unsigned)(epoch >> 32);
+    r.w = r.x ^ r.y ^ r.z ^ what ^ 0x5A5A5A5Au;
+    return r;
+}
+
+// 8 consecutive activations of one lane (half a 16-element block; the partner lane holds the other half) -> their hi / lo
+// bytes, the block's scale and integer sum: the arithmetic of quantize16, bit for bit.
+__device__ inline void quantize_half_block(const float (&v)[8], uint2 &hi, uint2 &lo, float &scale, int &sum) {
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+    m = fmaxf(m, dpp_move<0xB1>(m));  // the partner lane
+    const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
+    uint32_t hw[2] = {0u, 0u}, lw[2] = {0u, 0u};
+    sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        int xq = (int)__builtin_rintf(__fmul_rn(v[i], inv));
+        xq = xq > 32512 ? 32512 : (xq < -32512 ? -32512 : xq);
+        const int l = ((xq + 128) & 255) - 128;
+        const int h = (xq - l) >> 8;
+        hw[i >> 2] |= (uint32_t)(h & 255) << (8 * (i & 3));
+        lw[i >> 2] |= (uint32_t)(l & 255) << (8 * (i & 3));
+        sum += xq;
+    }
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, false);
+    hi = make_uint2(hw[0], hw[1]);
+    lo = make_uint2(lw[0], lw[1]);
+    scale = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
+}
+
+// load_lane_act from the workgroup's LDS copy of one token's 16-bit row (UPL = 1: hidden <= 2048).
+template <int WT>
+__device__ inline void load_lane_act_lds(const int8_t *s_hi, const int8_t *s_lo, const float *s_scale, const int *s_sum, int unit0,
+                                         int units, LaneAct<1> &a) {
+    const bool on = unit0 < units;
+    int e0, e1;
+    unit_halves<WT>(on ? unit0 : 0, e0, e1);
+    const int4 h0 = *(const int4 *)(s_hi + e0), h1 = *(const int4 *)(s_hi + e1);
+    const int4 l0 = *(const int4 *)(s_lo + e0), l1 = *(const int4 *)(s_lo + e1);
+    a.xh[0][0] = h0.x; a.xh[0][1] = h0.y; a.xh[0][2] = h0.z; a.xh[0][3] = h0.w;
+    a.xh[0][4] = h1.x; a.xh[0][5] = h1.y; a.xh[0][6] = h1.z; a.xh[0][7] = h1.w;
+    a.xl[0][0] = l0.x; a.xl[0][1] = l0.y; a.xl[0][2] = l0.z; a.xl[0][3] = l0.w;
+    a.xl[0][4] = l1.x; a.xl[0][5] = l1.y; a.xl[0][6] = l1.z; a.xl[0][7] = l1.w;
+    a.s[0][0] = on ? s_scale[e0 >> 4] : 0.0f;
+    a.s[0][1] = on ? s_scale[e1 >> 4] : 0.0f;
+    a.sx[0][0] = on ? s_sum[e0 >> 4] : 0;
+    a.sx[0][1] = on ? s_sum[e1 >> 4] : 0;
+    a.fsx[0][0] = __fmul_rn(a.s[0][0], (float)a.sx[0][0]);
+    a.fsx[0][1] = __fmul_rn(a.s[0][1], (float)a.sx[0][1]);
+}
+
+template <int RT>
+__device__ __forceinline__ float router_logit_of(const void *__restrict__ w, int e, const WaveRow &x, int hidden, int lane) {
+    WaveRouterRow wr;
+    wave_router_row_load<RT>(w, (size_t)e * (size_t)hidden, hidden, lane, wr);
+    return wave_router_dot(x, wr, hidden, lane);
+}
+
+__device__ __forceinline__ float router_logit_any(const void *__restrict__ w, int wtype, int e, const WaveRow &x, int hidden, int lane) {
+    if (wtype == T_F16) return router_logit_of<T_F16>(w, e, x, hidden, lane);
+    if (wtype == T_BF16) return router_logit_of<T_BF16>(w, e, x, hidden, lane);
+    return router_logit_of<T_F32>(w, e, x, hidden, lane);
+}
+
+template <int WT, int NIT, int RJN>
+__global__ __launch_bounds__(256) void gate_up_fused_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, int k,
+                                                            int hidden, int inter, int n_experts, QAct actq,
+                                                            int32_t *__restrict__ flags, RouteInline route, RouterExchange rx) {
+    constexpr int JN = RJN;
+    extern __shared__ float s_dyn[];  // [rows_per_block] gate/up results, then the token's 16-bit row
+    __shared__ __attribute__((aligned(16))) RouteScratch<JN> s_route;
+    __shared__ int s_ids[64];
+    __shared__ float s_w[64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.z;  // grid = (slot, row tile, token)
+    const int a = t * gridDim.x + blockIdx.x;
+    const RowSplit rs = row_split(hidden);
+    const int unit0 = lane & (rs.group - 1);
+    const int rows_per_block = NIT * rs.rows_per_it * (blockDim.x >> 6);
+    float *s_act = s_dyn;
+    int8_t *s_xhi = (int8_t *)(s_dyn + rows_per_block);
+    int8_t *s_xlo = s_xhi + hidden;
+    float *s_xscale = (float *)(s_xlo + hidden);
+    int *s_xsum = (int *)(s_xscale + hidden / 16);
+    MUMMU_PHASE(0);
+
+    // which router rows this workgroup computes: the workgroups of token t on one XCD are those with the same linear id
+    // modulo 8; `mine` counts them in linear order
+    const int per_token = gridDim.x * gridDim.y;             // a multiple of 8
+    const int per_xcd = per_token >> 3;
+    const int mine = (blockIdx.y * gridDim.x + blockIdx.x) >> 3;
+    const int rows_each = (n_experts + per_xcd - 1) / per_xcd;
+    const int row_begin = mine * rows_each;
+    const int row_end = row_begin + rows_each < n_experts ? row_begin + rows_each : n_experts;
+
+    // every load that does not depend on anything goes out first: the epoch, the token's row, this wave's router row.
+    // A wave with a router row (or with a gamma: the sum of squares runs over the whole row) and wave 0 take the whole row,
+    // the others only the 512-element chunk they quantize (chunk = wave: four waves, at most four chunks).
+    const unsigned long long epoch = *rx.epoch;
+    const float *xr = rx.x + (size_t)t * (size_t)hidden;
+    const int my_row = row_begin + wave, my_end = row_end;
+    const bool whole_row = rx.gamma != nullptr || my_row < my_end || wave == 0;  // (wave 0: it may have to compute missing logits)
+    const int qbase = lane * 8 + 512 * wave;
+    const bool qon = qbase < hidden;  // hidden % 64 == 0: the two lanes of a 16-element block are on or off together
+    WaveRow xrow;
+    f32x4 qa, qb;
+    if (whole_row) {
+        wave_row_load(xr, hidden, lane, xrow);
+    } else {
+        qa = ((const f32x4 *)(xr + (qon ? qbase : 0)))[0];
+        qb = ((const f32x4 *)(xr + (qon ? qbase : 0)))[1];
+    }
+    WaveRouterRow wrow;
+    if (my_row < my_end) {
+        const size_t at = (size_t)my_row * (size_t)hidden;
+        if (rx.wtype == T_F16) wave_router_row_load<T_F16>(rx.w, at, hidden, lane, wrow);
+        else if (rx.wtype == T_BF16) wave_router_row_load<T_BF16>(rx.w, at, hidden, lane, wrow);
+        else wave_router_row_load<T_F32>(rx.w, at, hidden, lane, wrow);
+    }
+    if (rx.gamma != nullptr) {
+        const float r = wave_row_rms_scale(xrow, hidden, lane, rx.eps);
+        wave_row_normalise(xrow, r, rx.gamma, hidden, lane);
+        if (rx.xnorm_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
+            float *xo = rx.xnorm_out + (size_t)t * (size_t)hidden;
+#pragma unroll
+            for (int c = 0; c < kWaveRowChunks; c++) {
+                const int base = lane * 8 + 512 * c;
+                if (base >= hidden) continue;
+                ((f32x4 *)(xo + base))[0] = xrow.a[c];
+                ((f32x4 *)(xo + base))[1] = xrow.b[c];
+            }
+        }
+    }
+    u32x4 *table = (u32x4 *)rx.slots + ((size_t)xcc_id() * kExchangeTokens + (size_t)t) * (size_t)n_experts;
+    // this wave's router row (more rows than waves: the remaining ones in further rounds, each with its own loads)
+    if (my_row < my_end) {
+        const float logit = wave_router_dot(xrow, wrow, hidden, lane);
+        if (lane == 0) table[my_row] = exchange_record(logit, epoch, (unsigned)(t * n_experts + my_row));
+    }
+    for (int row = row_begin + wave + (blockDim.x >> 6); row < row_end; row += blockDim.x >> 6) {
+        const float logit = router_logit_any(rx.w, rx.wtype, row, xrow, hidden, lane);
+        if (lane == 0) table[row] = exchange_record(logit, epoch, (unsigned)(t * n_experts + row));
+    }
+    MUMMU_PHASE(8);
+    // this wave's chunk of the row into LDS as 16-bit blocks (lane pairs hold the 16-element blocks)
+    if (whole_row) {
+        qa = xrow.a[0];
+        qb = xrow.b[0];
+#pragma unroll
+        for (int cc = 1; cc < kWaveRowChunks; cc++) {
+            qa = wave == cc ? xrow.a[cc] : qa;
+            qb = wave == cc ? xrow.b[cc] : qb;
+        }
+    }
+    if (512 * wave < hidden) {
+        const float v[8] = {qon ? qa.x : 0.0f, qon ? qa.y : 0.0f, qon ? qa.z : 0.0f, qon ? qa.w : 0.0f,
+                            qon ? qb.x : 0.0f, qon ? qb.y : 0.0f, qon ? qb.z : 0.0f, qon ? qb.w : 0.0f};
+        uint2 hi, lo;
+        float scale;
+        int sum;
+        quantize_half_block(v, hi, lo, scale, sum);
+        if (qon) {
+            *(uint2 *)(s_xhi + qbase) = hi;
+            *(uint2 *)(s_xlo + qbase) = lo;
+            if ((lane & 1) == 0) {
+                s_xscale[qbase >> 4] = scale;
+                s_xsum[qbase >> 4] = sum;
+            }
+            if (rx.xq_out.hi != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
+                // one workgroup per token also leaves the row in global memory (the shared expert's launches read it)
+                *(uint2 *)(rx.xq_out.hi + (size_t)t * (size_t)hidden + qbase) = hi;
+                *(uint2 *)(rx.xq_out.lo + (size_t)t * (size_t)hidden + qbase) = lo;
+                if ((lane & 1) == 0) {
+                    rx.xq_out.scale[(size_t)t * (size_t)(hidden / 16) + (qbase >> 4)] = scale;
+                    rx.xq_out.sum[(size_t)t * (size_t)(hidden / 16) + (qbase >> 4)] = sum;
+                }
+            }
+        }
+    }
+    MUMMU_PHASE(9);
+    if (wave == 0) {
+        // collect the E logits of token t from this XCD's table
+        float l[JN];
+        bool have[JN];
+#pragma unroll
+        for (int j = 0; j < JN; j++) {
+            l[j] = 0.0f;
+            have[j] = lane + 64 * j >= n_experts;
+        }
+        const unsigned long long t_begin = wall_clock64();
+        bool complete = false;
+        while (rx.spin_ticks != 0u) {  // (a bound of 0: do not look at the table at all)
+            bool all = true;
+#pragma unroll
+            for (int j = 0; j < JN; j++) {
+                if (have[j]) continue;
+                const int e = lane + 64 * j;
+                const u32x4 r = load_device_scope_b128(table + e);
+                const u32x4 want = exchange_record(__uint_as_float(r.x), epoch, (unsigned)(t * n_experts + e));
+                if (r.y == want.y && r.z == want.z && r.w == want.w) {
+                    l[j] = __uint_as_float(r.x);
+                    have[j] = true;
+                } else {
+                    all = false;
+                }
+            }
+            if (__all(all)) {
+                complete = true;
+                break;
+            }
+            if (wall_clock64() - t_begin >= (unsigned long long)rx.spin_ticks) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        MUMMU_PHASE(10);
+        if (!complete) {
+            // records that never came: compute those logits here (the same function of the same row: the same bits)
+            if (lane == 0 && rx.fallbacks != nullptr) atomicAdd(rx.fallbacks, 1ULL);
+#pragma unroll
+            for (int j = 0; j < JN; j++) {
+                unsigned long long missing = __ballot(!have[j]);
+                while (missing != 0ull) {
+                    const int src = (int)__builtin_ctzll(missing);
+                    missing &= missing - 1ull;
+                    const float v = router_logit_any(rx.w, rx.wtype, src + 64 * j, xrow, hidden, lane);
+                    if (lane == src) l[j] = v;
+                }
+            }
+        }
+        if (rx.logits_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
+#pragma unroll
+            for (int j = 0; j < JN; j++)
+                if (lane + 64 * j < n_experts) rx.logits_out[(size_t)t * n_experts + lane + 64 * j] = l[j];
+        }
+        route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
+        wave_lds_sync();
+        if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
+            const int id = s_ids[lane];
+            route.ids[(size_t)t * k + lane] = id;
+            route.weights[(size_t)t * k + lane] = s_w[lane];
+            if (route.hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&route.hits[id], 1ULL);
+        }
+        MUMMU_PHASE(11);
+    }
+    __syncthreads();
+    MUMMU_PHASE(7);
+    LaneAct<1> la;
+    load_lane_act_lds<WT>(s_xhi, s_xlo, s_xscale, s_xsum, unit0, rs.units, la);
+    MUMMU_PHASE(14);
+    const int e = s_ids[blockIdx.x];
+    if ((unsigned)e >= (unsigned)n_experts) {
+        if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
+        return;
+    }
+    gate_up_tile<WT, 1, NIT, true>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act);
+}
+
 // gate/up, float banks.  RJN > 0: the kernel routes by itself (see RouteInline), RJN experts per lane
 // of the routing wave.
 template <int WT, int VEC, int RJN = 0>
@@ -214,7 +519,7 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gate_up_f_kernel(
                 const int id = s_ids[lane];
                 route.ids[(size_t)t * k + lane] = id;
                 route.weights[(size_t)t * k + lane] = s_w[lane];
-                if (route.hits) atomicAdd(&route.hits[id], 1ULL);
+                if (route.hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&route.hits[id], 1ULL);
             }
         }
         __syncthreads();
@@ -365,8 +670,11 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_f_kernel(const uint8_t *
 template <int WT, int UPL, int NIT, int KPW, int kDcWaves = 4>
 __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
     const uint8_t *down /* not __restrict__: the code fences below must order its loads */, QAct actq, const int32_t *__restrict__ ids, const float *__restrict__ weights,
-    int k, int hidden, int inter, int n_experts, const float *__restrict__ residual, float *__restrict__ out) {
+    int k, int hidden, int inter, int n_experts, const float *__restrict__ residual, float *__restrict__ out,
+    unsigned long long *epoch_bump) {
     constexpr int KMAX = kDcWaves * KPW;
+    // the launch before this one (gate_up_fused_kernel) has finished with the epoch: move it on for the next
+    if (epoch_bump != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *epoch_bump = *epoch_bump + 1ULL;
     extern __shared__ float s_mem[];  // [KMAX][rows_per_block] row sums, then [KMAX] weights
     MUMMU_PHASE(0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -694,6 +1002,47 @@ hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInlin
     });
 }
 
+bool gate_up_fused_supported(const ExpertBanks &b, int k, int n_tokens, const RouterExchange &rx) {
+    if (!gate_up_routes_inline(b, k) || !down_combine_supported(b, k)) return false;
+    if (n_tokens < 1 || n_tokens > kExchangeTokens || b.hidden % 64 != 0 || b.hidden > 512 * kWaveRowChunks) return false;
+    if (rx.wtype != T_F32 && rx.wtype != T_F16 && rx.wtype != T_BF16) return false;
+    if ((((uintptr_t)rx.x | (uintptr_t)rx.w | (uintptr_t)rx.gamma | (uintptr_t)rx.xnorm_out | (uintptr_t)rx.slots) & 15) != 0) return false;
+    if (rx.x == nullptr || rx.w == nullptr || rx.slots == nullptr || rx.epoch == nullptr) return false;
+    if (rx.xnorm_out != nullptr && rx.gamma == nullptr) return false;
+    const RowSplit rs = row_split(b.hidden);
+    const int rpb = 4 * 4 * rs.rows_per_it;  // four waves, NIT = 4
+    const int tiles = (b.inter + rpb - 1) / rpb;
+    return (k * tiles) % 8 == 0;  // a token's workgroups spread evenly over the 8 XCDs
+}
+
+template <int WT>
+static hipError_t launch_gate_up_fused_t(const ExpertBanks &b, const RouterExchange &rx, const RouteInline &route, int n_tokens,
+                                         int k, QAct actq, int32_t *flags, hipStream_t s) {
+    constexpr int NIT = 4;
+    const RowSplit rs = row_split(b.hidden);
+    const int rpb = 4 * NIT * rs.rows_per_it;
+    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(256);
+    const size_t lds = sizeof(float) * (size_t)rpb + 2 * (size_t)b.hidden + 8 * (size_t)(b.hidden / 16);
+#define MUMMU_GUX(JN) \
+    launch_kernel(gate_up_fused_kernel<WT, NIT, JN>, grid, block, lds, s, b.gate, b.up, k, b.hidden, b.inter, b.n_experts, actq, flags, route, rx)
+    if (b.n_experts <= 64) MUMMU_GUX(1);
+    else if (b.n_experts <= 128) MUMMU_GUX(2);
+    else MUMMU_GUX(8);
+#undef MUMMU_GUX
+    return hipGetLastError();
+}
+
+hipError_t launch_gate_up_fused(const ExpertBanks &b, const RouterExchange &rx, const RouteInline &route, int n_tokens, int k,
+                                QAct actq, int32_t *flags, hipStream_t s) {
+    if (n_tokens <= 0) return hipSuccess;
+    if (!gate_up_fused_supported(b, k, n_tokens, rx)) return hipErrorInvalidValue;
+    return with_bank_type(b.gate_type, [&](auto tag) {
+        constexpr int WT = decltype(tag)::value;
+        if constexpr (is_quant_type(WT)) return launch_gate_up_fused_t<WT>(b, rx, route, n_tokens, k, actq, flags, s);
+        else return hipErrorInvalidValue;
+    });
+}
+
 template <int WT>
 static hipError_t launch_down_t(const ExpertBanks &b, const float *act, QAct actq, const int32_t *ids, int n_assign,
                                 int k, int fixed_expert, float *y, hipStream_t s) {
@@ -744,7 +1093,7 @@ bool down_combine_supported(const ExpertBanks &b, int k) {
 
 template <int WT>
 static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n,
-                                        int k, const float *residual, float *out, hipStream_t s) {
+                                        int k, const float *residual, float *out, hipStream_t s, unsigned long long *epoch_bump) {
     const RowSplit rs = row_split(b.inter);
     const int upl = (rs.units + 63) / 64;
 #define MUMMU_DC(UPL, NIT, KPW, WAVES)                                                                             \
@@ -753,7 +1102,7 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
         dim3 grid(n, (b.hidden + rpb - 1) / rpb), block(64 * (WAVES));                                             \
         const size_t lds = sizeof(float) * (size_t)((WAVES) * (KPW)) * (size_t)(rpb + 1);                          \
         launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW, WAVES>, grid, block, lds, s, b.down, actq, ids, weights, k, \
-                      b.hidden, b.inter, b.n_experts, residual, out);                                              \
+                      b.hidden, b.inter, b.n_experts, residual, out, epoch_bump);                                  \
     } while (0)
     // two experts per wave (one for top_k <= 4), as many waves as that takes
     if (upl == 1) {
@@ -772,12 +1121,12 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
 }
 
 hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,
-                               const float *residual, float *out, hipStream_t s) {
+                               const float *residual, float *out, hipStream_t s, unsigned long long *epoch_bump) {
     if (n <= 0) return hipSuccess;
     if (!down_combine_supported(b, k)) return hipErrorInvalidValue;
     return with_bank_type(b.down_type, [&](auto tag) {
         constexpr int WT = decltype(tag)::value;
-        if constexpr (is_quant_type(WT)) return launch_down_combine_t<WT>(b, actq, ids, weights, n, k, residual, out, s);
+        if constexpr (is_quant_type(WT)) return launch_down_combine_t<WT>(b, actq, ids, weights, n, k, residual, out, s, epoch_bump);
         else return hipErrorInvalidValue;
     });
 }

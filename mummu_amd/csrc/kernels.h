@@ -71,6 +71,30 @@ struct RouteInline {
 bool gate_up_routes_inline(const ExpertBanks &b, int k);
 hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInline &route, int n_tokens, int k, QAct actq,
                                  int32_t *flags, hipStream_t s);
+// Router logits, routing and gate/up in ONE launch (the first of the two launches of a decode step): the workgroups
+// of a token that share an XCD split the router's rows and pass the logits to one another through a table in that
+// XCD's L2 (see gate_up_fused_kernel).  x is the block's f32 input [n, hidden]; with gamma it is the raw residual
+// stream and RmsNorm(x) = (x * r) * gamma is what the block sees (xnorm_out, nullable, also receives those rows).
+constexpr int kExchangeTokens = 8;  // tokens per launch the table holds
+constexpr int kExchangeXcds = 16;   // the hardware id has four bits
+struct RouterExchange {
+    const float *x = nullptr;
+    const void *w = nullptr;  // router weights [E, hidden], F32 / F16 / BF16
+    int wtype = 0;
+    const float *gamma = nullptr;
+    float eps = 0.0f;
+    float *xnorm_out = nullptr;
+    void *slots = nullptr;                      // router_exchange_bytes(E) bytes, 256-byte aligned
+    const unsigned long long *epoch = nullptr;  // incremented by the launch that follows (launch_down_combine)
+    float *logits_out = nullptr;                // nullable [n, E]
+    QAct xq_out;                                // nullable (hi == nullptr): the token rows as 16-bit blocks, for a later launch
+    unsigned spin_ticks = 5000;                 // bound of the wait for the other workgroups' records, 10 ns units
+    unsigned long long *fallbacks = nullptr;    // nullable: += 1 per workgroup that gave up waiting and computed the logits itself
+};
+inline size_t router_exchange_bytes(int n_experts) { return (size_t)kExchangeXcds * kExchangeTokens * (size_t)n_experts * 16; }
+bool gate_up_fused_supported(const ExpertBanks &b, int k, int n_tokens, const RouterExchange &rx);
+hipError_t launch_gate_up_fused(const ExpertBanks &b, const RouterExchange &rx, const RouteInline &route, int n_tokens, int k,
+                                QAct actq, int32_t *flags, hipStream_t s);
 // The same pair for float banks (F32 / F16 / BF16 gate/up and down, at most 512 experts, top_k <= 16):
 // gate/up with the routing inside writes act [n*k, inter] f32, then down + combine in one launch.
 bool float_decode_fused(const ExpertBanks &b, int k);
@@ -88,8 +112,9 @@ hipError_t launch_combine(const float *y, const int32_t *ids, const float *weigh
                           int hidden, const float *residual, float *out, hipStream_t s);
 // down + combine in one launch (no y round trip): quantized down bank and top_k <= 16.
 bool down_combine_supported(const ExpertBanks &b, int k);
+// epoch_bump (nullable): the 64-bit counter of the router exchange, incremented once by this launch.
 hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *ids, const float *weights, int n, int k,
-                               const float *residual, float *out, hipStream_t s);
+                               const float *residual, float *out, hipStream_t s, unsigned long long *epoch_bump = nullptr);
 
 
 // out[t, :] = [residual[t, :] +] (out[t, :] + y[t, :] * sigmoid(<gate_vec, x[t, :]>)), every operation

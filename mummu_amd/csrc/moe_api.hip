@@ -100,6 +100,14 @@ struct mummu_moe {
     int32_t *sh_sorted = nullptr, *sh_tiles = nullptr, *sh_ntiles = nullptr;  // its one-expert work list
     int sh_max_tiles = 0;
 
+    // router exchange of the two-launch decode form (gate_up_fused_kernel): the per-XCD logit table, its epoch counter
+    // and the count of workgroups that gave up waiting; xcd_round_robin says the device deals workgroups to 8 XCDs by
+    // linear id modulo 8, which is what makes the exchange worth using
+    void *xslots = nullptr;
+    unsigned long long *xstate = nullptr;  // [0] epoch, [1] fallbacks
+    bool xcd_round_robin = false;
+    int router_exchange = 1;
+    unsigned spin_ticks = 5000;
     // bumped whenever a device buffer a captured graph may point into is freed (workspace regrown, a layer's or
     // a shared expert's weights replaced); a graph remembers the value it was captured under
     uint64_t generation = 0;
@@ -478,6 +486,8 @@ struct DecodeScratch {
     int32_t *ids;     // [n, k]
     float *weights;   // [n, k]
     QAct xq, actq;    // [n, H] and [n*k, I rounded up to 16]
+    void *xslots = nullptr;                  // router exchange table (router_exchange_bytes(E)), or null: three launches
+    unsigned long long *xstate = nullptr;    // [0] its epoch, [1] its fallback counter
 };
 
 // The two launches after the router's: gate/up with the routing inside, then down + combine.
@@ -493,6 +503,43 @@ int decode_tail(mummu_moe *h, const Layer &L, const DecodeScratch &ws, int n, in
     route.hits = L.hits;
     LAUNCH(h, K_GATE_UP, s, launch_gate_up_routed(b, ws.xq, route, n, k, ws.actq, h->flags, s));
     LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, ws.actq, ws.ids, ws.weights, n, k, residual, out, s));
+    return MUMMU_OK;
+}
+
+// The decode step in two launches where the device and the shapes allow it: router + routing + gate/up in one kernel
+// (the workgroups exchange the logits inside it), then down + combine.  *done = false: not taken, nothing launched.
+int decode_two_launches(mummu_moe *h, const Layer &L, const DecodeScratch &ws, const float *x, int n, int k, int norm,
+                        const float *residual, float *out, hipStream_t s, const float *norm_gamma, float *xnorm_out, bool *done) {
+    *done = false;
+    if (!h->router_exchange || !h->xcd_round_robin || ws.xslots == nullptr || ws.xstate == nullptr) return MUMMU_OK;
+    // measured on the OLMoE shape (Q4_K): one token 18.1 us against 18.4 in three launches, but 23.6 / 40.2 / 69.5 us
+    // against 22.8 / 36.6 / 57.2 at 2 / 4 / 8 tokens - every workgroup repeats the router wait, and the fused kernel
+    // keeps fewer waves per CU.  So one token only, unless a caller asks for it at every size (tests do).
+    if (n > 1 && h->router_exchange < 2) return MUMMU_OK;
+    const ExpertBanks b = banks_of(h, L);
+    RouterExchange rx;
+    rx.x = x;
+    rx.w = L.router;
+    rx.wtype = L.router_type;
+    rx.gamma = norm_gamma;
+    rx.eps = h->cfg.rms_norm_eps;
+    rx.xnorm_out = xnorm_out;
+    rx.slots = ws.xslots;
+    rx.epoch = ws.xstate;
+    rx.logits_out = ws.logits;
+    rx.spin_ticks = h->spin_ticks;
+    rx.fallbacks = ws.xstate + 1;
+    if (L.sh_loaded) rx.xq_out = ws.xq;  // the shared expert's kernels multiply the same 16-bit rows
+    if (!gate_up_fused_supported(b, k, n, rx)) return MUMMU_OK;
+    RouteInline route;
+    route.flavour = h->cfg.router_flavour;
+    route.norm = norm;
+    route.ids = ws.ids;
+    route.weights = ws.weights;
+    route.hits = L.hits;
+    LAUNCH(h, K_GATE_UP, s, launch_gate_up_fused(b, rx, route, n, k, ws.actq, h->flags, s));
+    LAUNCH(h, K_DOWN_COMBINE, s, launch_down_combine(b, ws.actq, ws.ids, ws.weights, n, k, residual, out, s, ws.xstate));
+    *done = true;
     return MUMMU_OK;
 }
 
@@ -515,13 +562,19 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
                                    h->ids, h->weights, batched ? nullptr : L.hits, h->flags, xq, s));
         return run_experts(h, L, x, want_xq, n, k, residual, out, s, batched);
     } else {
+        if (want_xq) {
+            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, h->xslots, h->xstate};
+            bool done = false;
+            const int rc = decode_two_launches(h, L, ws, x, (int)n, k, norm, residual, out, s, norm_gamma, xnorm_out, &done);
+            if (rc || done) return rc;
+        }
         // few tokens: the router rows are spread over as many CUs as there are experts
         LAUNCH(h, K_ROUTER_LOGITS, s,
                launch_router_logits(x, L.router, L.router_type, h->logits, (int)n, H, E, xq, s, norm_gamma, h->cfg.rms_norm_eps, xnorm_out));
         const ExpertBanks b = banks_of(h, L);
         if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
             // ... and the gate/up kernel routes by itself: one launch less on the decode path
-            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq};
+            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, nullptr, nullptr};
             return decode_tail(h, L, ws, (int)n, k, norm, residual, out, s);
         }
         if (!batched && float_decode_fused(b, k)) {
@@ -606,6 +659,38 @@ int check_device_call(mummu_moe *h, int64_t n, int k, const void *a, const void 
         return fail(h, MUMMU_ERR_TOKENS, std::to_string(n) + " tokens x top_k " + std::to_string(k) +
                                              " exceeds the workspace (max_tokens " + std::to_string(h->ws_tokens) + ", pairs " +
                                              std::to_string(h->ws_assign) + ")");
+    return MUMMU_OK;
+}
+
+// Do workgroups whose linear ids agree modulo 8 run on one XCD?  (The router exchange splits its work on that
+// assumption; it stays correct without it, only slow, so it is switched off then.)  Probed with the launch shape of the
+// decode kernels.
+__global__ __launch_bounds__(256) void xcd_probe_kernel(int *out) {
+    if (threadIdx.x == 0)
+        out[blockIdx.y * gridDim.x + blockIdx.x] = (int)(__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u);  // HW_REG_XCC_ID[3:0]
+}
+
+int probe_xcd_round_robin(mummu_moe *h) {
+    constexpr int kProbe = 512;
+    int *d = nullptr;
+    HIPCHK(h, hipMalloc((void **)&d, sizeof(int) * kProbe));
+    std::vector<int> got(kProbe);
+    bool rr = true;
+    hipError_t e = hipSuccess;
+    for (int rep = 0; rep < 2 && e == hipSuccess; rep++) {
+        launch_kernel(xcd_probe_kernel, dim3(8, kProbe / 8), dim3(256), 0, h->stream, d);
+        e = hipMemcpyAsync(got.data(), d, sizeof(int) * kProbe, hipMemcpyDeviceToHost, h->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
+        for (int i = 0; i < kProbe && e == hipSuccess; i++) rr = rr && got[i] == got[i & 7];
+    }
+    (void)hipFree(d);
+    if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("XCD probe: ") + hipGetErrorString(e));
+    if (getenv("MUMMU_DEBUG")) {
+        fprintf(stderr, "[mummu] XCD of workgroups 0..15:");
+        for (int i = 0; i < 16; i++) fprintf(stderr, " %d", got[i]);
+        fprintf(stderr, "  -> same XCD for equal id mod 8: %s\n", rr ? "yes" : "no");
+    }
+    h->xcd_round_robin = rr;
     return MUMMU_OK;
 }
 
@@ -717,6 +802,16 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     int rc = reset_flags(h);
     if (rc) return bail(rc);
     {
+        // the router exchange: table and state, and whether workgroups land on the XCDs the way it assumes
+        const size_t xb = router_exchange_bytes(cfg->num_experts);
+        if (hipMalloc(&h->xslots, xb) != hipSuccess || hipMalloc((void **)&h->xstate, 256) != hipSuccess)
+            return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(router exchange) failed"));
+        if (hipMemset(h->xslots, 0, xb) != hipSuccess || hipMemset(h->xstate, 0, 256) != hipSuccess)
+            return bail(fail(h, MUMMU_ERR_DEVICE, "hipMemset(router exchange) failed"));
+        if ((rc = probe_xcd_round_robin(h))) return bail(rc);
+        if (const char *e = getenv("MUMMU_ROUTER_EXCHANGE")) h->router_exchange = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
+    }
+    {
         // resolve the static scratch's address on this device now, outside any stream capture
         unsigned char *unused = nullptr;
         if ((rc = static_scratch(h, &unused))) return bail(rc);
@@ -736,6 +831,8 @@ void mummu_moe_destroy(mummu_moe *h) {
             if (p) (void)hipFree(p);
     }
     free_ws(h);
+    if (h->xslots) (void)hipFree(h->xslots);
+    if (h->xstate) (void)hipFree(h->xstate);
     if (h->flags) (void)hipFree(h->flags);
     for (auto &t : h->timed) {
         (void)hipEventDestroy(t.start);
@@ -1219,9 +1316,10 @@ int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const float *x_dev
     // carve the static array: every piece starts on a 256-byte boundary
     const size_t E = (size_t)h->cfg.num_experts, H = (size_t)h->cfg.hidden_size, I = (size_t)h->cfg.expert_intermediate_size;
     const size_t nn = (size_t)n, na = nn * (size_t)top_k, xe = nn * H, ae = na * ((I + 15) / 16 * 16);
-    const size_t want[] = {sizeof(float) * nn * E, sizeof(int32_t) * na, sizeof(float) * na,
+    // (the exchange state comes first: its epoch must keep its place - and its value - from call to call)
+    const size_t want[] = {256, sizeof(float) * nn * E, sizeof(int32_t) * na, sizeof(float) * na,
                            xe, xe, sizeof(float) * (xe / 16), sizeof(int32_t) * (xe / 16),
-                           ae, ae, sizeof(float) * (ae / 16), sizeof(int32_t) * (ae / 16)};
+                           ae, ae, sizeof(float) * (ae / 16), sizeof(int32_t) * (ae / 16), router_exchange_bytes((int)E)};
     size_t off[sizeof(want) / sizeof(want[0]) + 1] = {0};
     for (size_t i = 0; i < sizeof(want) / sizeof(want[0]); i++) off[i + 1] = (off[i] + want[i] + 255) / 256 * 256;
     const size_t need = off[sizeof(want) / sizeof(want[0])];
@@ -1231,13 +1329,21 @@ int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const float *x_dev
     unsigned char *base = nullptr;
     if ((rc = static_scratch(h, &base))) return rc;
     DecodeScratch ws;
-    ws.logits = (float *)(base + off[0]);
-    ws.ids = (int32_t *)(base + off[1]);
-    ws.weights = (float *)(base + off[2]);
-    ws.xq = QAct{(int8_t *)(base + off[3]), (int8_t *)(base + off[4]), (float *)(base + off[5]), (int32_t *)(base + off[6])};
-    ws.actq = QAct{(int8_t *)(base + off[7]), (int8_t *)(base + off[8]), (float *)(base + off[9]), (int32_t *)(base + off[10])};
+    ws.xstate = (unsigned long long *)(base + off[0]);
+    ws.logits = (float *)(base + off[1]);
+    ws.ids = (int32_t *)(base + off[2]);
+    ws.weights = (float *)(base + off[3]);
+    ws.xq = QAct{(int8_t *)(base + off[4]), (int8_t *)(base + off[5]), (float *)(base + off[6]), (int32_t *)(base + off[7])};
+    ws.actq = QAct{(int8_t *)(base + off[8]), (int8_t *)(base + off[9]), (float *)(base + off[10]), (int32_t *)(base + off[11])};
+    ws.xslots = base + off[12];
     hipStream_t s = (hipStream_t)stream;
-    // the kernels write every word of the scratch they later read (nothing in it has to start at zero)
+    {
+        bool done = false;
+        rc = decode_two_launches(h, L, ws, x_dev, (int)n, top_k, norm, nullptr, out_dev, s, nullptr, nullptr, &done);
+        if (rc || done) return rc;
+    }
+    // the kernels write every word of the scratch they later read; the exchange's epoch counts on from whatever the
+    // array holds (it starts at zero with the process), so nothing has to be cleared between calls
     LAUNCH(h, K_ROUTER_LOGITS, s,
            launch_router_logits(x_dev, L.router, L.router_type, ws.logits, (int)n, (int)H, (int)E, ws.xq, s, nullptr, h->cfg.rms_norm_eps, nullptr));
     return decode_tail(h, L, ws, (int)n, top_k, norm, nullptr, out_dev, s);
@@ -1323,6 +1429,28 @@ int mummu_device_name(char *buf, size_t len) {
 }
 
 void *mummu_moe_stream(mummu_moe *h) { return h ? (void *)h->stream : nullptr; }
+
+int mummu_moe_set_router_exchange(mummu_moe *h, int enable, unsigned spin_ticks) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    h->router_exchange = enable < 0 ? 0 : (enable > 2 ? 2 : enable);
+    h->spin_ticks = spin_ticks;
+    return MUMMU_OK;
+}
+
+int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbacks) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    std::lock_guard<std::mutex> lock(h->mu);
+    if (usable) *usable = h->router_exchange && h->xcd_round_robin;
+    if (fallbacks) {
+        HIPCHK(h, hipDeviceSynchronize());
+        unsigned long long v = 0, zero = 0;
+        HIPCHK(h, hipMemcpy(&v, h->xstate + 1, sizeof(v), hipMemcpyDeviceToHost));
+        HIPCHK(h, hipMemcpy(h->xstate + 1, &zero, sizeof(zero), hipMemcpyHostToDevice));
+        *fallbacks = v;
+    }
+    return MUMMU_OK;
+}
 
 int mummu_graph_begin(mummu_moe *h) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");

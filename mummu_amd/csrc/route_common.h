@@ -41,6 +41,100 @@ __device__ inline void load_w8(const void *w, size_t i, float (&o)[8]) {
 }
 
 // ---------------------------------------------------------------------------------------
+// One token's activation row held by one wave in the router's layout: lane l owns elements 8l .. 8l+7 of
+// every 512-element chunk (hidden <= 512 * kWaveRowChunks, hidden % 8 == 0, 16-byte aligned rows).  Every load
+// of the row goes out at once.  Lanes whose slice lies past the row's end re-read its first elements and never
+// use them.
+// ---------------------------------------------------------------------------------------
+constexpr int kWaveRowChunks = 4;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));  // (a first-class vector type: arrays of it stay in registers)
+
+struct WaveRow {
+    f32x4 a[kWaveRowChunks], b[kWaveRowChunks];
+};
+
+__device__ __forceinline__ void wave_row_load(const float *__restrict__ xr, int hidden, int lane, WaveRow &r) {
+#pragma unroll
+    for (int c = 0; c < kWaveRowChunks; c++) {
+        const int base = lane * 8 + 512 * c;
+        const int at = base < hidden ? base : 0;
+        r.a[c] = ((const f32x4 *)(xr + at))[0];
+        r.b[c] = ((const f32x4 *)(xr + at))[1];
+    }
+}
+
+// 1 / sqrt(mean(x^2) + eps): the sum of squares as 512 strided partials (element i -> partial i mod 512, fused
+// multiply-adds in ascending i), each lane's eight folded ((a0+a4)+(a1+a5))+((a2+a6)+(a3+a7)), then the pairwise
+// tree over the lanes - the order the RmsNorm kernel and the router kernel use.  Every lane gets the result.
+__device__ __forceinline__ float wave_row_rms_scale(const WaveRow &r, int hidden, int lane, float eps) {
+    float a2[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int c = 0; c < kWaveRowChunks; c++) {
+        if (lane * 8 + 512 * c >= hidden) continue;
+        const float xv[8] = {r.a[c].x, r.a[c].y, r.a[c].z, r.a[c].w, r.b[c].x, r.b[c].y, r.b[c].z, r.b[c].w};
+#pragma unroll
+        for (int j = 0; j < 8; j++) a2[j] = __builtin_fmaf(xv[j], xv[j], a2[j]);
+    }
+    float ss = __fadd_rn(__fadd_rn(__fadd_rn(a2[0], a2[4]), __fadd_rn(a2[1], a2[5])),
+                         __fadd_rn(__fadd_rn(a2[2], a2[6]), __fadd_rn(a2[3], a2[7])));
+    ss = wave_sum(ss);
+    return __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, (float)hidden), eps)));
+}
+
+// x <- (x * rs) * gamma, two roundings per element.
+__device__ __forceinline__ void wave_row_normalise(WaveRow &r, float rs, const float *__restrict__ gamma, int hidden, int lane) {
+    f32x4 ga[kWaveRowChunks], gb[kWaveRowChunks];
+#pragma unroll
+    for (int c = 0; c < kWaveRowChunks; c++) {
+        const int base = lane * 8 + 512 * c;
+        const int at = base < hidden ? base : 0;
+        ga[c] = ((const f32x4 *)(gamma + at))[0];
+        gb[c] = ((const f32x4 *)(gamma + at))[1];
+    }
+#pragma unroll
+    for (int c = 0; c < kWaveRowChunks; c++) {
+        r.a[c].x = __fmul_rn(__fmul_rn(r.a[c].x, rs), ga[c].x);
+        r.a[c].y = __fmul_rn(__fmul_rn(r.a[c].y, rs), ga[c].y);
+        r.a[c].z = __fmul_rn(__fmul_rn(r.a[c].z, rs), ga[c].z);
+        r.a[c].w = __fmul_rn(__fmul_rn(r.a[c].w, rs), ga[c].w);
+        r.b[c].x = __fmul_rn(__fmul_rn(r.b[c].x, rs), gb[c].x);
+        r.b[c].y = __fmul_rn(__fmul_rn(r.b[c].y, rs), gb[c].y);
+        r.b[c].z = __fmul_rn(__fmul_rn(r.b[c].z, rs), gb[c].z);
+        r.b[c].w = __fmul_rn(__fmul_rn(r.b[c].w, rs), gb[c].w);
+    }
+}
+
+// A router row's weights in the same layout (all loads at once) ...
+struct WaveRouterRow {
+    float w[kWaveRowChunks][8];
+};
+
+template <int WT>
+__device__ __forceinline__ void wave_router_row_load(const void *__restrict__ w, size_t wrow, int hidden, int lane, WaveRouterRow &r) {
+#pragma unroll
+    for (int c = 0; c < kWaveRowChunks; c++) {
+        const int base = lane * 8 + 512 * c;
+        load_w8<WT>(w, wrow + (size_t)(base < hidden ? base : 0), r.w[c]);
+    }
+}
+
+// ... and the logit <x, w> in the router's fixed order (the file comment of router.hip): every lane gets it.
+__device__ __forceinline__ float wave_router_dot(const WaveRow &x, const WaveRouterRow &wr, int hidden, int lane) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int c = 0; c < kWaveRowChunks; c++) {
+        if (lane * 8 + 512 * c >= hidden) continue;  // (never adds: keeps -0 partials impossible either way)
+        const float xv[8] = {x.a[c].x, x.a[c].y, x.a[c].z, x.a[c].w, x.b[c].x, x.b[c].y, x.b[c].z, x.b[c].w};
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(xv[j], wr.w[c][j], acc[j]);
+    }
+    const float s = __fadd_rn(__fadd_rn(__fadd_rn(acc[0], acc[4]), __fadd_rn(acc[1], acc[5])),
+                              __fadd_rn(__fadd_rn(acc[2], acc[6]), __fadd_rn(acc[3], acc[7])));
+    return wave_sum(s);
+}
+
+// ---------------------------------------------------------------------------------------
 // softmax -> top-k -> renormalise, one wave per token.  Lane l holds experts l, l+64, ...
 // Ties: strictly-greater wins, so the lower expert id keeps a tie and equal slots ascend
 // by id (experts.rs:557-573; the stable descending sort of nn/moe.rs:2143-2144).
@@ -147,7 +241,30 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         for (int j = 0; j < JN; j++) p[j] = __fmul_rn(p[j], scale);
     }
 
-    if (!ANY_K || k <= 16) {
+    MUMMU_PHASE(12);
+    if (JN == 1 && (!ANY_K || k <= 16)) {
+        // one expert per lane: the rounds run on the bit patterns (a probability is a non-negative finite float, so it
+        // orders like its bits; -1 marks a lane that is out of the running), and every lane remembers the slot it won
+        // instead of lane 0 writing each round's winner
+        int cand = lane < n_experts ? __float_as_int(p[0]) : -1;
+        int my_slot = -1;
+        auto round = [&](int s) {
+            const int best = wave_max_i32(cand);
+            const int win = (int)__builtin_ctzll(__ballot(cand == best));  // lowest expert id holding the maximum
+            my_slot = lane == win ? s : my_slot;
+            cand = lane == win ? -1 : cand;
+        };
+        if (k == 8) {  // the usual top-8 as straight-line code (a taken branch costs as much as half a round)
+#pragma unroll
+            for (int s = 0; s < 8; s++) round(s);
+        } else {
+            for (int s = 0; s < k; s++) round(s);
+        }
+        if (my_slot >= 0) {
+            sc.w[my_slot] = p[0];
+            sc.id[my_slot] = lane;
+        }
+    } else if (!ANY_K || k <= 16) {
         // k rounds of "largest remaining probability, lowest id on a tie": the wave maximum,
         // then the first lane (and, within a lane, the first expert) that holds it
         float cand[JN];
@@ -213,6 +330,7 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         }
     }
     wave_lds_sync();
+    MUMMU_PHASE(13);
 
     float denom = 1.0f;
     if (flavour == 0) {
@@ -235,7 +353,7 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         if (divide) wv = __fdiv_rn(wv, denom);
         ids[orow * k + s] = id;
         weights[orow * k + s] = wv;
-        if (hits) atomicAdd(&hits[id], 1ULL);
+        if (hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&hits[id], 1ULL);
     }
 }
 

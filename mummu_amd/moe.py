@@ -304,6 +304,17 @@ class SparseMoe:
         self._check(self._lib.mummu_moe_forward_device_noalloc(self._h, layer, x_dev.ptr, n, top_k, int(norm_topk_prob),
                                                                out_dev.ptr, self.stream))
 
+    def set_router_exchange(self, enable, spin_ticks: int = 5000):
+        """Two-launch decode form: 0 / False off, 1 / True at one token (default), 2 at every size it takes; and the
+        bound (10 ns units) of a workgroup's wait for the others' logits."""
+        self._check(self._lib.mummu_moe_set_router_exchange(self._h, int(enable), spin_ticks))
+
+    def router_exchange_state(self):
+        """(two-launch form in use on this device, workgroups that gave up waiting since the last call)."""
+        usable, fb = C.c_int(0), C.c_uint64(0)
+        self._check(self._lib.mummu_moe_router_exchange_state(self._h, C.byref(usable), C.byref(fb)))
+        return bool(usable.value), int(fb.value)
+
     def expert_run_device(self, layer: int, expert: int, x_dev: "DeviceBuffer", rows: int, out_dev: "DeviceBuffer"):
         """ExpertExec::run_tensor_resident (nn/moe.rs:360-371): rows already on the device, result left there."""
         self._check(self._lib.mummu_expert_run_device(self._h, layer, expert, x_dev.ptr, rows, self.config.hidden_size,

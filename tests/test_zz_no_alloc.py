@@ -25,7 +25,9 @@ def test_noalloc_forward_gives_the_bits_of_forward_device_on_two_calls_in_a_row(
     router = (g.standard_normal((E, H), dtype=np.float32) * np.float32(0.02)).astype(np.float16)
     with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=8) as m:
         m.load_layer(0, router, M.F16, gate, gt, up, gt, down, dt)
-        for n in (8, 3):  # the second call is smaller: whatever the first left in the static array must not leak in
+        # the second call is smaller: whatever the first left in the static array must not leak in; one token takes the
+        # two-launch form, whose logit table and epoch live in the static array as well
+        for n in (8, 3, 1, 1):
             x = g.standard_normal((n, H), dtype=np.float32)
             xd = M.DeviceBuffer.from_array(x)
             want_d, got_d = M.DeviceBuffer(x.nbytes), M.DeviceBuffer(x.nbytes)
