@@ -215,6 +215,39 @@ def test_a_random_block_with_a_shared_expert_matches_the_composition(seed):
     assert err <= tol, f"{what}: max relative error {err:.3e} > {tol}"
 
 
+def test_known_limit_of_the_16_bit_activations_a_hidden_row_with_one_element_standing_out():
+    # The documented limit of the block-scaled 16-bit activations (include/mummu_moe.h, "Arithmetic of block-quantized
+    # banks"): draw 7 has a token whose gate pre-activations are all far below zero, so its hidden row is ~1e-15 except
+    # for one or two elements ~0.2; every other element of their blocks shares their scale and keeps only a few bits.
+    # The token's outputs are ~1e5 times smaller than the batch's; against THEIR OWN magnitude (the reference's
+    # measure, unchanged) the worst element is a few 1e-3 off - above the 2e-3 bar, below the 1e-2 this test pins -
+    # and against 1 % of the batch's typical magnitude it is far inside the bar.  If the first number moves up, the
+    # arithmetic got worse; if it drops under 2e-3, the floor in the random draws can go.
+    seed = 7
+    gt, dt, sgt, sdt, H, I, IS, E, k, n, flavour, gated = draw_shared(seed)
+    gate, up, down = bank(gt, [H, I, E], 11 * seed + 1), bank(gt, [H, I, E], 11 * seed + 2), bank(dt, [I, H, E], 11 * seed + 3)
+    sgate, sup, sdown = bank(sgt, [H, IS, 1], 11 * seed + 4), bank(sgt, [H, IS, 1], 11 * seed + 5), bank(sdt, [IS, H, 1], 11 * seed + 6)
+    router = normal((E, H), 11 * seed + 7, 0.05)
+    gate_vec = normal((H,), 11 * seed + 8, 0.2) if gated else None
+    x = normal((n, H), 11 * seed + 9)
+    norm = flavour == M.ROUTER_QWEN4EXP or bool(seed & 1)
+    with M.SparseMoe(M.SparseMoeConfig(H, I, E, k), max_tokens=n, router_flavour=flavour) as m:
+        m.load_layer(0, router, M.F32, gate, gt, up, gt, down, dt)
+        m.load_shared_expert(0, IS, sgate, sgt, sup, sgt, sdown, sdt, gate_vec)
+        got = m.forward(x, k, norm)
+    banks = orc.LayerBanks(H, I, E, gate, up, down, gt, gt, dt)
+    shared = orc.LayerBanks(H, IS, 1, sgate, sup, sdown, sgt, sgt, sdt)
+    _, _, _, full, mag = reference(banks, shared, router, orc.F32, gate_vec, x, k, norm, flavour)
+    own = orc.rel_err(got, full, mag)
+    floored = orc.rel_err(got, full, np.maximum(mag, 1e-2 * np.median(mag)))
+    worst_token = int(np.unravel_index(np.argmax(own), own.shape)[0])
+    assert own.max() <= 1e-2, f"the known limit moved: {own.max():.3e} (token {worst_token})"
+    assert floored.max() <= 2e-3
+    # the limit only ever shows on outputs far below the batch's typical size
+    over = own > 2e-3
+    assert not over.any() or mag[over].max() <= 1e-2 * np.median(mag)
+
+
 @pytest.mark.parametrize("sgt", [M.Q8_0, M.F32], ids=["quantized-shared", "float-shared"])
 def test_decode_stack_with_a_shared_expert_and_the_norm_inside_the_router_launch(sgt):
     # up to 8 tokens the stack normalises inside the router launch and hands the normalised rows to the shared
