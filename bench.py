@@ -37,7 +37,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # kernel-timing slot -> name of the kernel in the rocprofv3 summaries
-PROFILE_KERNEL_NAMES = {"gate_up": "gate_up_q_kernel", "down_combine": "down_combine_q_kernel"}
+PROFILE_KERNEL_NAMES = {"gate_up": ("gate_up_fused_kernel", "gate_up_q_kernel"), "down_combine": ("down_combine_q_kernel",)}
 
 
 def profiled_traffic(workload, tokens, slot):
@@ -46,15 +46,15 @@ def profiled_traffic(workload, tokens, slot):
     counter scaled by what it reads for the library's 256 MiB copy kernel).  None for a workload or batch size
     no summary was taken on."""
     path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt" if tokens == 1 else f"{workload}_bt{tokens}_hbm_traffic.txt")
-    name = PROFILE_KERNEL_NAMES.get(slot)
-    if name is None or not os.path.exists(path):
+    names = PROFILE_KERNEL_NAMES.get(slot)
+    if names is None or not os.path.exists(path):
         return None
     column = None
     for line in open(path):
         if line.startswith("kernel ") and "traffic B" in line:
             head = line.split("  ")
             column = [c.strip() for c in head if c.strip()].index("traffic B")
-        elif column is not None and line.startswith(name):
+        elif column is not None and line.startswith(names):
             # the kernel name holds template arguments with spaces: count the numeric fields from the right
             fields = line[line.index(">") + 1:].split() if ">" in line else line.split()[1:]
             return int(float(fields[column - 1]))
@@ -93,6 +93,9 @@ def main() -> int:
     ap.add_argument("--shared-inter", type=int, default=0,
                     help="also give every layer a shared expert of this intermediate width with a sigmoid gate "
                          "(Qwen-style block; same bank types); the CPU baseline leg is skipped")
+    ap.add_argument("--no-steady", action="store_true",
+                    help="leave out the event-timed replays behind `steady` (rocprofv3's kernel trace has crashed inside "
+                         "hipGraphLaunch between event records; the profile commands pass this)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--seed", type=int, default=1234)
@@ -254,7 +257,7 @@ def main() -> int:
     # steady state: >= 200 replays of a graph over one whole rotation, each replay timed on the device between two
     # HIP events (no host synchronisation in between): median and p10 / p90 of the per-layer time
     steady = None
-    if use_graph:
+    if use_graph and not args.no_steady:
         rot_graph = graph if per_graph == rotation else capture(first, min(rotation, 1024))
         rot_steps = per_graph if per_graph == rotation else min(rotation, 1024)
         reps = max(200, -(-2048 // rot_steps))
@@ -283,7 +286,9 @@ def main() -> int:
     per_kernel_us = {name: (tot / cnt * 1e3 if cnt else None) for name, (tot, cnt) in kt.items()}
     layer_bytes = mean_distinct * expert_bytes + router_bytes + n * H * 8
     # the dominant kernel and the bytes one launch of it has to move
-    kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes + n * E * 4,
+    # at one token the gate/up launch is the fused one where the device allows it: it also reads the router and the f32 row
+    fused = n == 1 and moe.router_exchange_state()[0]
+    kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes + (router_bytes + n * H * 4 if fused else n * E * 4),
                     "down_combine": mean_distinct * (expert_bytes - gate_up_expert_bytes),
                     "down": mean_distinct * (expert_bytes - gate_up_expert_bytes),
                     "gemm_gate_up": mean_distinct * gate_up_expert_bytes}
@@ -326,7 +331,8 @@ def main() -> int:
                    "first_timed_step": first,
                    "cache_cold": bool((per_graph - 1) * layer_bytes * layers_per_step > 256e6) if graph is not None else
                                  bool(min(L, args.steps) * layer_bytes > 256e6),
-                   "mean_distinct_experts_per_step": round(mean_distinct, 3)},
+                   "mean_distinct_experts_per_step": round(mean_distinct, 3),
+                   "launches_per_step": {k_: int(round(cnt / max(probe_steps * (L if args.stack else 1), 1))) for k_, (tot, cnt) in kt.items() if cnt}},
         "us_per_layer": round(ms_per_step * 1e3, 3),
         "event_ms_per_step": round(ev_ms / args.steps / layers_per_step, 6),
         "steady": steady,
