@@ -20,6 +20,8 @@
 //                    integer sums are exact, C = 256*C_hi + C_lo, and the f32 accumulator takes
 //                    s * sum_blocks(d_block * C).  Q4_K's offset term -dmin*m*sum(x) is one
 //                    v_mfma_f32_32x32x2_f32 per K step over the per-block activation sums.
+#include <type_traits>
+
 #include "device_utils.h"
 #include "kernels.h"
 
@@ -839,6 +841,335 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Q4_K banks on the f16 units
+// ---------------------------------------------------------------------------------------
+// A Q4_K weight is d * (sc * q) - dmin * m with q < 16 and sc, m < 64 per 32 elements and d, dmin per 256.
+// sc * q < 1024 is an exact half, so the matrix cores can sum x * (sc * q) over a whole run of
+// sub-blocks with no vector work in between; the f32 accumulator takes d * that sum once per 128
+// elements.  Activations come as pairs of halfs (HAct): the two products of a K step go into the
+// same accumulator.  The offset term is one more instruction per 128 elements: the sums of the four
+// 32-element blocks (hi and lo halfs, K = 8) against the four m.  Per output element and 128 elements
+// of K that leaves three vector operations where the int8 form spends fourteen.
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+// Only the activation tile goes through LDS.  Wave w owns output columns 32w..32w+31 for every row of the
+// tile, so the weights of those columns are its own: lane (column c, K group g) reads 16 of the 32 quant
+// bytes of a 64-element step of row c straight into registers (low nibbles: elements 16g..16g+15, high
+// nibbles: 32+16g..), turns them into its four B operands and never stores them anywhere.  The K index of
+// an instruction therefore maps to element (kk/2)*32 + 16g + (kk%2)*8 + i of the step, and the A operands
+// are read from the tile at that offset.  The activation tile is double-buffered (one barrier per step),
+// loads run two steps (weights) and one step (activations) ahead of their use.
+template <bool GATE_UP, int MT>
+struct HTileLds {
+    static constexpr int BM = 32 * MT;
+    static constexpr int kRow = 2 * kLds;                     // LDS row (bytes): 64 halfs + 8 of padding
+    static constexpr int kBuf = 2 * BM * kRow;                // hi and lo planes of one K step
+    static constexpr int kC = GATE_UP ? BM * kLdsC * 4 : 0;   // f32 staging of the epilogue (aliases the tiles)
+    static constexpr int kBytes = 2 * kBuf > kC ? 2 * kBuf : kC;
+};
+
+// Two biased halfs 1024 + byte from bytes 0, 1 (or 2, 3) of t.
+__device__ inline half2v biased_pair(uint32_t t, bool upper) {
+    const uint32_t u = __builtin_amdgcn_perm(0x64646464u, t, upper ? 0x04030402u : 0x04010400u);
+    half2v h;
+    __builtin_memcpy(&h, &u, 4);
+    return h;
+}
+
+// GATE_UP: A = the token rows of a_in gathered through `sorted`; the epilogue writes silu(g)*u in sorted
+//          order, as HAct (OUT_H: the down banks are Q4_K too) or in the int8 kernels' QAct64.
+// else   : A = a_in rows in sorted order; y[pos, n] = f32 sum.
+// WM: the workgroup has 4 WM waves; wave w owns columns 32 (w % 4) .. +31 of row blocks (w / 4) * MT / WM .. of the
+// tile.  With two waves to a column block each expands the weights of its columns itself (twice the vector work
+// in the workgroup) and keeps half the accumulators, which is what lets two workgroups share a CU without spills.
+template <bool GATE_UP, int MT, int WM, bool OUT_H>
+__global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
+    const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, HAct a_in, const int32_t *__restrict__ sorted, int k_slots,
+    const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim, HAct act_h, QAct64 act_q,
+    float *__restrict__ y_out) {
+    using L = HTileLds<GATE_UP, MT>;
+    constexpr int NB = GATE_UP ? 2 : 1, BM = L::BM, kRow = L::kRow;
+    constexpr int MW = MT / WM, NT = 256 * WM;   // row blocks per wave, threads
+    static_assert(MT % WM == 0, "row blocks split evenly over the wave rows");
+    __shared__ __attribute__((aligned(16))) uint8_t s_raw[L::kBytes];
+    __shared__ __attribute__((aligned(16))) float s_as[2][BM];         // activation scale of a 128-element run, per tile row
+    __shared__ __attribute__((aligned(8))) _Float16 s_sum[2][BM][8];   // its four block sums: hi halfs, then lo halfs
+    auto s_a = [&](int buf, int plane, int row) -> _Float16 * {
+        return (_Float16 *)(s_raw + (size_t)buf * L::kBuf + ((size_t)plane * BM + row) * kRow);
+    };
+
+    int tile, slab;
+    if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
+    const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int n0 = slab * kBN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t row_bytes = gemm_row_bytes(T_Q4_K, in_dim);
+    const int col = 32 * (wave & 3) + (lane & 31), g = lane >> 5;
+    const int row0 = 32 * MW * (wave >> 2);   // first tile row of this wave
+
+    // Addresses are a uniform base plus a 32-bit byte offset per lane (an expert's bank and the activation planes
+    // are far below 4 GB).  Rows past the tile's end read its last row and columns past the matrix its last column:
+    // their products are never stored.
+    const int b_out = n0 + col < out_dim ? n0 + col : out_dim - 1;
+    const uint8_t *b_base[NB];
+    b_base[0] = w0 + (size_t)e * (size_t)out_dim * row_bytes;
+    if (GATE_UP) b_base[NB - 1] = w1 + (size_t)e * (size_t)out_dim * row_bytes;
+    const uint32_t b_off = (uint32_t)b_out * (uint32_t)row_bytes + 16u * (uint32_t)g;
+
+    auto source_row = [&](int r) -> int {
+        r = r < rows ? r : rows - 1;
+        return GATE_UP ? sorted[p0 + r] / k_slots : p0 + r;
+    };
+    // activation tile: thread -> (plane, row, 8 halfs), passes of 16 WM rows
+    constexpr int A_PASSES = 2 * MT / WM, A_ROWS = 16 * WM;
+    const int a_plane = tid / (NT / 2), a_chunk = tid & 7;
+    const uint8_t *a_base = (const uint8_t *)(a_plane ? a_in.lo : a_in.hi);
+    uint32_t a_off[A_PASSES], a_lds[A_PASSES];
+#pragma unroll
+    for (int p = 0; p < A_PASSES; p++) {
+        const int r = A_ROWS * p + ((tid >> 3) & (A_ROWS - 1));
+        a_off[p] = ((uint32_t)source_row(r) * (uint32_t)in_dim + (uint32_t)a_chunk * 8u) * 2u;
+        a_lds[p] = (uint32_t)(((size_t)a_plane * BM + r) * kRow + a_chunk * 16);
+    }
+    // block sums and scales of a 128-element run: thread -> (row tid / 4, block tid % 4)
+    // (threads past 4 BM repeat rows, and all four threads of a row store its scale: the same values twice, and no
+    // branch in the loop body - with basic blocks in it the compiler sinks one step's arithmetic into the next and
+    // keeps both steps' accumulators alive)
+    const int m_row = (tid >> 2) & (BM - 1), m_blk = tid & 3;
+    const uint32_t src_m = (uint32_t)source_row(m_row);
+    const uint32_t sum_off = (src_m * (uint32_t)(in_dim / 32) + (uint32_t)m_blk) * 4u;
+    const uint32_t scale_off = src_m * (uint32_t)(in_dim / 128) * 4u;
+
+    float16v acc[NB][MW], c1[NB][MW];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int m = 0; m < MW; m++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[b][m][r] = c1[b][m][r] = 0.0f;
+
+    // weights: the raw bytes of the step being multiplied and of the next one, the header of the current
+    // super-block and, during its last step, of the next
+    u32x4 raw[2][NB], rh[NB], rh_next[NB];
+    auto load_b = [&](int k0, int st, u32x4 (&dst)[NB]) {
+        const uint32_t o = b_off + (uint32_t)(k0 >> 8) * 144u;
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            dst[b] = *(const u32x4 *)(b_base[b] + (o + 16u + (uint32_t)st * 32u));
+            if (st == 0) rh_next[b] = *(const u32x4 *)(b_base[b] + (o - 16u * (uint32_t)g));
+        }
+    };
+    // activations of one step in registers, then into a tile
+    u32x4 ra[A_PASSES];
+    float rsum = 0.0f, rscale = 0.0f;
+    auto load_a = [&](int k0, int st) {
+#pragma unroll
+        for (int p = 0; p < A_PASSES; p++) ra[p] = *(const u32x4 *)(a_base + (a_off[p] + (uint32_t)k0 * 2u));
+        if ((st & 1) == 0) {
+            rsum = *(const float *)((const uint8_t *)a_in.ssum + (sum_off + (uint32_t)(k0 >> 5) * 4u));
+            rscale = *(const float *)((const uint8_t *)a_in.scale + (scale_off + (uint32_t)(k0 >> 7) * 4u));
+        }
+    };
+    auto store_a = [&](int buf, int st, int pair_buf) {
+#pragma unroll
+        for (int p = 0; p < A_PASSES; p++) *(u32x4 *)(s_raw + (size_t)buf * L::kBuf + a_lds[p]) = ra[p];
+        if ((st & 1) == 0) {
+            const _Float16 h = (_Float16)rsum;
+            s_sum[pair_buf][m_row][m_blk] = h;
+            s_sum[pair_buf][m_row][4 + m_blk] = (_Float16)__fsub_rn(rsum, (float)h);
+            s_as[pair_buf][m_row] = rscale;
+        }
+    };
+
+    const float16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    // one 64-element step: st = which step of the super-block, buf = which tile holds its activations
+    auto multiply = [&](int st, int buf, const u32x4 (&rw)[NB]) {
+        half2v ml2[NB], al2[NB], mh2[NB], ah2[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            uint32_t scp, mnp;
+            k4_scale_min_both(rh[b][1], rh[b][2], rh[b][3], st, scp, mnp);
+            const float sc_lo = (float)(scp & 0xFFu), sc_hi = (float)((scp >> 8) & 0xFFu);
+            // low nibbles: (1024 + q) * sc - 1024 sc; high nibbles, left in place: (1024 + 16 q) * (sc / 16) - 64 sc
+            const _Float16 ml = (_Float16)sc_lo, al = (_Float16)__fmul_rn(-1024.0f, sc_lo);
+            const _Float16 mh = (_Float16)__fmul_rn(0.0625f, sc_hi), ah = (_Float16)__fmul_rn(-64.0f, sc_hi);
+            ml2[b] = half2v{ml, ml};
+            al2[b] = half2v{al, al};
+            mh2[b] = half2v{mh, mh};
+            ah2[b] = half2v{ah, ah};
+        }
+        const uint8_t *tile = s_raw + (size_t)buf * L::kBuf + (size_t)(row0 + (lane & 31)) * kRow + 32 * g;
+        // the A operands of instruction group kk + 1 are read from the tile before group kk is issued
+        half8 a_hi[2][MW], a_lo[2][MW];
+        auto read_a = [&](int kk) {
+            const int a_byte = (kk >> 1) * 64 + (kk & 1) * 16;  // element (kk/2)*32 + 16g + (kk%2)*8 of the step
+#pragma unroll
+            for (int m = 0; m < MW; m++) {
+                a_hi[kk & 1][m] = *(const half8 *)(tile + (size_t)(32 * m) * kRow + a_byte);
+                a_lo[kk & 1][m] = *(const half8 *)(tile + (size_t)(BM + 32 * m) * kRow + a_byte);
+            }
+        };
+        read_a(0);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            if (kk < 3) read_a(kk + 1);
+            half8 bfrag[NB];
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const uint32_t w_a = (kk & 1) ? rw[b][2] : rw[b][0], w_b = (kk & 1) ? rw[b][3] : rw[b][1];
+                const uint32_t mask = kk < 2 ? 0x0F0F0F0Fu : 0xF0F0F0F0u;
+                const half2v mul = kk < 2 ? ml2[b] : mh2[b], add = kk < 2 ? al2[b] : ah2[b];
+                half2v f[4];
+                f[0] = __builtin_elementwise_fma(biased_pair(w_a & mask, false), mul, add);
+                f[1] = __builtin_elementwise_fma(biased_pair(w_a & mask, true), mul, add);
+                f[2] = __builtin_elementwise_fma(biased_pair(w_b & mask, false), mul, add);
+                f[3] = __builtin_elementwise_fma(biased_pair(w_b & mask, true), mul, add);
+                __builtin_memcpy(&bfrag[b], f, 16);
+            }
+#pragma unroll
+            for (int m = 0; m < MW; m++) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[kk & 1][m], bfrag[b], ((st & 1) == 0 && kk == 0) ? zero : c1[b][m], 0, 0, 0);
+                    c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[kk & 1][m], bfrag[b], c1[b][m], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // the 128 elements just summed into c1 -> acc; pair: which half of the super-block
+    auto fold = [&](int pair, int pair_buf) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const float d = half_bits_to_float((uint16_t)(rh[b][0] & 0xFFFFu));
+            const float ndmin = -half_bits_to_float((uint16_t)(rh[b][0] >> 16));
+            uint32_t sc0, mn0, sc1, mn1;
+            k4_scale_min_both(rh[b][1], rh[b][2], rh[b][3], 2 * pair, sc0, mn0);
+            k4_scale_min_both(rh[b][1], rh[b][2], rh[b][3], 2 * pair + 1, sc1, mn1);
+            const half4v bm = {(_Float16)(float)(mn0 & 0xFFu), (_Float16)(float)((mn0 >> 8) & 0xFFu), (_Float16)(float)(mn1 & 0xFFu),
+                               (_Float16)(float)((mn1 >> 8) & 0xFFu)};
+#pragma unroll
+            for (int m = 0; m < MW; m++) {
+                const half4v am = *(const half4v *)&s_sum[pair_buf][row0 + 32 * m + (lane & 31)][4 * g];
+                const float16v c2 = __builtin_amdgcn_mfma_f32_32x32x8f16(am, bm, zero, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float4 s4 = *(const float4 *)&s_as[pair_buf][row0 + 32 * m + 8 * j + 4 * g];
+                    const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int r = 4 * j + i;
+                        const float u = fmaf(ndmin, c2[r], __fmul_rn(d, c1[b][m][r]));
+                        acc[b][m][r] = fmaf(u, sr[i], acc[b][m][r]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);  // (one 32 x 32 block at a time: scheduled together they do not fit the registers)
+            }
+        }
+    };
+
+    // prologue: step 0 into tile 0
+    load_b(0, 0, raw[0]);
+    load_a(0, 0);
+    store_a(0, 0, 0);
+    __syncthreads();
+    MUMMU_TIMER_DECL;
+    // (one step as a generic lambda over a compile-time step index: the register sets are picked by constants)
+    auto step = [&](int sb0, auto st_c) {
+        constexpr int st = decltype(st_c)::value;
+        // (after the last step the "next" one is step 0 again: loaded and stored like any other, never multiplied;
+        // no branch in the loop body)
+        const int k_next = (st == 3 && sb0 + 256 >= in_dim) ? 0 : sb0 + kBK * (st + 1);
+        MUMMU_TIMER_MARK(0);
+        if (st == 0) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) rh[b] = rh_next[b];
+        }
+        // the next step: weights into the other set of registers, activations into registers
+        load_b(k_next, (st + 1) & 3, raw[(st + 1) & 1]);
+        load_a(k_next, (st + 1) & 3);
+        MUMMU_CODE_FENCE();  // (the loads stay here, a whole step ahead of their first use)
+        MUMMU_TIMER_MARK(1);
+        multiply(st, st & 1, raw[st & 1]);
+        MUMMU_TIMER_MARK(2);
+        if (st & 1) fold(st >> 1, (st >> 1) & 1);
+        MUMMU_TIMER_MARK(3);
+        MUMMU_CODE_FENCE();
+        // ... and into the tile that the step before this one was read from
+        store_a((st + 1) & 1, (st + 1) & 3, (((st + 1) & 3) >> 1) & 1);
+        MUMMU_TIMER_MARK(4);
+        __syncthreads();
+        MUMMU_TIMER_MARK(5);
+    };
+    for (int sb0 = 0; sb0 < in_dim; sb0 += 256) {
+        step(sb0, std::integral_constant<int, 0>{});
+        step(sb0, std::integral_constant<int, 1>{});
+        step(sb0, std::integral_constant<int, 2>{});
+        step(sb0, std::integral_constant<int, 3>{});
+    }
+    MUMMU_TIMER_STORE;
+
+    if (GATE_UP) {
+        // stage silu(g)*u of the whole tile as f32 (over the activation tiles, no longer needed), then store it in the
+        // form the down product reads
+        float *s_c = (float *)s_raw;
+#pragma unroll
+        for (int m = 0; m < MW; m++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                s_c[(row0 + 32 * m + acc_row(r, lane)) * kLdsC + col] = __fmul_rn(det_silu(acc[0][m][r]), acc[NB - 1][m][r]);
+        __syncthreads();
+        if (OUT_H) {
+            const int grp = tid >> 5, l32 = tid & 31;
+#pragma unroll
+            for (int pass = 0; pass < BM / (NT / 32); pass++) {
+                const int row = pass * (NT / 32) + grp;
+                const float4 v = *(const float4 *)&s_c[row * kLdsC + 4 * l32];
+                const bool active = row < rows && n0 < out_dim;
+                hact_store128(active ? v : make_float4(0.f, 0.f, 0.f, 0.f), active, act_h, (size_t)(p0 + row), out_dim, n0 + 4 * l32);
+            }
+        } else {
+            const int grp = tid >> 4, l16 = tid & 15;
+#pragma unroll
+            for (int pass = 0; pass < 2 * BM / (NT / 16); pass++) {
+                const int task = pass * (NT / 16) + grp, row = task >> 1, cb = task & 1;
+                const float4 v = *(const float4 *)&s_c[row * kLdsC + cb * 64 + 4 * l16];
+                const bool active = row < rows && n0 + cb * 64 < out_dim;
+                quantize_store64(active ? v : make_float4(0.f, 0.f, 0.f, 0.f), active, act_q, (size_t)(p0 + row), out_dim,
+                                 n0 + cb * 64 + 4 * l16);
+            }
+        }
+    } else {
+        const int n = n0 + col;
+        if (n < out_dim) {
+#pragma unroll
+            for (int m = 0; m < MW; m++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = row0 + 32 * m + acc_row(r, lane);
+                    if (row < rows) y_out[(size_t)(p0 + row) * (size_t)out_dim + (size_t)n] = acc[0][m][r];
+                }
+        }
+    }
+}
+
+// x [n, d] f32 -> HAct: one 32-lane group per 128-element block.
+__global__ __launch_bounds__(256) void quantize_rows_h_kernel(const float *__restrict__ x, int d, HAct q) {
+    const int row = blockIdx.y;
+    const int elem0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    const bool active = elem0 < d;
+    const float4 v = active ? *(const float4 *)(x + (size_t)row * (size_t)d + elem0) : make_float4(0.f, 0.f, 0.f, 0.f);
+    hact_store128(v, active, q, (size_t)row, d, elem0);
+}
+
+hipError_t launch_quantize_rows_h(const float *x, int n, int d, HAct q, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (d % 128 != 0) return hipErrorInvalidValue;
+    launch_kernel(quantize_rows_h_kernel, dim3((d + 1023) / 1024, n), dim3(256), 0, s, x, d, q);
+    return hipGetLastError();
+}
+
 // x [n, d] f32 -> QAct64: one 16-lane row per 64-element block.
 __global__ __launch_bounds__(256) void quantize_rows64_kernel(const float *__restrict__ x, int d, QAct64 q) {
     const int row = blockIdx.y;
@@ -906,6 +1237,35 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
     return hipGetLastError();
 }
 
+bool grouped_gemm_q4k_f16(const ExpertBanks &b) {
+    return b.gate_type == T_Q4_K && b.up_type == T_Q4_K && b.hidden % 256 == 0 && b.inter % 128 == 0;
+}
+
+bool grouped_gemm_q4k_f16_down(const ExpertBanks &b) {
+    return grouped_gemm_q4k_f16(b) && b.down_type == T_Q4_K && b.inter % 256 == 0 && b.hidden % 128 == 0;
+}
+
+template <bool GATE_UP>
+static hipError_t launch_gemm_q4k_f16(const uint8_t *w0, const uint8_t *w1, HAct a_in, const int32_t *sorted, int k_slots,
+                                      const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
+                                      int out_dim, HAct act_h, QAct64 act_q, bool out_h, float *y_out, hipStream_t s) {
+    dim3 grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
+#define MUMMU_H(MT, WM, OUT_H)                                                                                           \
+    launch_kernel(grouped_gemm_q4k_f16_kernel<GATE_UP, MT, WM, OUT_H>, grid, dim3(256 * WM), 0, s, w0, w1, a_in, sorted, k_slots, \
+                  tiles, n_tiles, in_dim, out_dim, act_h, act_q, y_out)
+    if (tile_rows == 64) {
+        if (out_h) MUMMU_H(2, 1, true);
+        else MUMMU_H(2, 1, false);
+    } else if (tile_rows == 32) {
+        if (out_h) MUMMU_H(1, 1, true);
+        else MUMMU_H(1, 1, false);
+    } else {
+        return hipErrorInvalidValue;
+    }
+#undef MUMMU_H
+    return hipGetLastError();
+}
+
 template <bool GATE_UP>
 static hipError_t launch_gemm_f32(const uint8_t *w0, const uint8_t *w1, const float *a_in, const int32_t *sorted, int k_slots,
                                   const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int in_dim,
@@ -942,10 +1302,17 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const fl
     return hipGetLastError();
 }
 
-hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
+hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, HAct xh, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
-                               float *act32, QAct64 actq, hipStream_t s) {
+                               float *act32, QAct64 actq, HAct acth, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (xh.hi != nullptr) {
+        if (!grouped_gemm_q4k_f16(b)) return hipErrorInvalidValue;
+        const bool out_h = acth.hi != nullptr;
+        if (out_h && !grouped_gemm_q4k_f16_down(b)) return hipErrorInvalidValue;
+        return launch_gemm_q4k_f16<true>(b.gate, b.up, xh, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden, b.inter,
+                                         acth, actq, out_h, nullptr, s);
+    }
     if (b.gate_type == T_F32)
         return launch_gemm_f32<true>(b.gate, b.up, x, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden, b.inter, act32,
                                      nullptr, s);
@@ -973,9 +1340,14 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     }
 }
 
-hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, int n_assign,
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, HAct acth, int n_assign,
                             const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (acth.hi != nullptr) {
+        if (!grouped_gemm_q4k_f16_down(b)) return hipErrorInvalidValue;
+        return launch_gemm_q4k_f16<false>(b.down, nullptr, acth, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter, b.hidden,
+                                          HAct(), QAct64(), false, y, s);
+    }
     if (b.down_type == T_F32)
         return launch_gemm_f32<false>(b.down, nullptr, act32, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter, b.hidden,
                                       nullptr, y, s);

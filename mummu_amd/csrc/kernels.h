@@ -154,10 +154,18 @@ bool grouped_gemm_quantized(const ExpertBanks &b);
 int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts);
 // x [n, d] f32 -> QAct64 (d % 64 == 0).
 hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s);
-hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, const int32_t *sorted, int k_slots,
+// Q4_K banks can take the f16 units instead, against activations held as pairs of halfs (HAct: xh tokens x
+// hidden, acth A x inter in sorted order): gate and up both Q4_K ..., ... and the down bank as well.  The
+// launchers below take that form when xh.hi / acth.hi are given (pass HAct() for the int8 form); with a
+// down bank of another type the gate/up launch still writes actq.
+bool grouped_gemm_q4k_f16(const ExpertBanks &b);
+bool grouped_gemm_q4k_f16_down(const ExpertBanks &b);
+// x [n, d] f32 -> HAct (d % 128 == 0).
+hipError_t launch_quantize_rows_h(const float *x, int n, int d, HAct q, hipStream_t s);
+hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, HAct xh, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
-                               float *act32, QAct64 actq, hipStream_t s);
-hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, int n_assign,
+                               float *act32, QAct64 actq, HAct acth, hipStream_t s);
+hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, HAct acth, int n_assign,
                             const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s);
 
 }  // namespace mummu

@@ -91,6 +91,7 @@ struct mummu_moe {
     // batches at least this large take dispatch + grouped GEMM (measured crossovers on the OLMoE shape:
     // the 16-bit float decode kernels lose from 7 tokens on, the f32 ones from 10, the integer ones from 19)
     int gemm_min_f16 = 7, gemm_min_quant = 19, gemm_min_f32 = 10;
+    int gemm_q4k_f16 = 1;        // Q4_K banks of the batched path on the f16 units (0: the int8 form)
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
@@ -446,14 +447,21 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         // the 16-bit activation buffers, viewed in the batched path's 64-element-block layout
         const QAct64 xq64{h->xq.hi, h->xq.lo, h->xq.scale, (float *)h->xq.sum};
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
-        if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
+        // Q4_K banks on the f16 units: x as pairs of halfs in the (not yet written) buffer of the down product's
+        // output, the activations between the two products in the f16 and f32 activation buffers
+        const bool hf = h->gemm_q4k_f16 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
+        const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum} : HAct();
+        const HAct acth = hf_down ? HAct{(_Float16 *)h->act16, (_Float16 *)h->act, h->actq.scale, (float *)h->actq.sum} : HAct();
+        if (hf) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows_h(x, (int)n, b.hidden, xh, s));
+        else if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
         LAUNCH(h, K_DISPATCH, s,
                launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch,
                                count_hits ? L.hits : nullptr, h->flags, s));
         LAUNCH(h, K_GEMM_GATE_UP, s,
-               launch_gemm_gate_up(b, x, xq64, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, h->act, actq64, s));
+               launch_gemm_gate_up(b, x, xq64, xh, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, h->act, actq64,
+                                   acth, s));
         LAUNCH(h, K_GEMM_DOWN, s,
-               launch_gemm_down(b, h->act16, h->act, actq64, na, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
+               launch_gemm_down(b, h->act16, h->act, actq64, acth, na, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
         LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, h->inv, (int)n, k, b.hidden, residual, out, s));
         return MUMMU_OK;
     }
@@ -633,12 +641,18 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
         const QAct64 actq64{h->sh_actq.hi, h->sh_actq.lo, h->sh_actq.scale, (float *)h->sh_actq.sum};
         LAUNCH(h, K_SHARED, s, launch_identity_tiles((int)n, tile_rows, h->sh_sorted, h->sh_tiles, h->sh_ntiles, s));
         // (the routed path may have left the 16-bit activations in the decode layout, or not made them)
-        if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, H, xq64, s));
+        // (Q4_K on the f16 units as in the routed path; the routed products are done with their output buffer)
+        const bool hf = h->gemm_q4k_f16 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
+        const HAct xh = hf ? HAct{(_Float16 *)h->sh_y, (_Float16 *)h->sh_y + (size_t)n * H, h->xq.scale, (float *)h->xq.sum} : HAct();
+        const HAct acth = hf_down ? HAct{(_Float16 *)h->sh_act16, (_Float16 *)h->sh_act, h->sh_actq.scale, (float *)h->sh_actq.sum} : HAct();
+        if (hf) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows_h(x, (int)n, H, xh, s));
+        else if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, H, xq64, s));
         LAUNCH(h, K_SHARED, s,
-               launch_gemm_gate_up(b, x, xq64, h->sh_sorted, 1, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_act16,
-                                   h->sh_act, actq64, s));
+               launch_gemm_gate_up(b, x, xq64, xh, h->sh_sorted, 1, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_act16,
+                                   h->sh_act, actq64, acth, s));
         LAUNCH(h, K_SHARED, s,
-               launch_gemm_down(b, h->sh_act16, h->sh_act, actq64, (int)n, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_y, s));
+               launch_gemm_down(b, h->sh_act16, h->sh_act, actq64, acth, (int)n, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows,
+                                h->sh_y, s));
     } else {
         // the routed decode kernels leave x in the 16-bit decode layout when their own banks are quantized;
         // otherwise (float routed banks, or the batched path's layout) it is made here
@@ -780,6 +794,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     mummu_moe *h = new mummu_moe();
     h->cfg = *cfg;
     // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
+    if (const char *e = getenv("MUMMU_GEMM_Q4K_F16")) h->gemm_q4k_f16 = atoi(e) != 0;
     if (const char *e = getenv("MUMMU_GEMM_MIN_TOKENS")) {
         const int v = atoi(e);
         if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = h->gemm_min_f32 = v;

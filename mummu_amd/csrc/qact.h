@@ -101,4 +101,55 @@ __device__ inline void quantize_store64(float4 v, bool active, const QAct64 &q, 
     }
 }
 
+// Activations for the products of Q4_K banks on the f16 matrix units: every element as a pair of
+// halfs, x = scale * (hi + lo) with hi = f16(x / scale), lo = f16(x / scale - hi), one power-of-two
+// scale per 128 elements chosen so that the block's largest |x / scale| lies in [2^9, 2^10): 22
+// significant bits per element (elements more than 2^24 below their block's largest keep an absolute
+// error of 2^-25 of it), and sums of 32 scaled elements stay below 2^15, inside a half's range.
+//   hi, lo : f16 [rows][D]      scale : f32 [rows][D/128]      ssum : f32 [rows][D/32], sum of x / scale
+struct HAct {
+    _Float16 *hi = nullptr;
+    _Float16 *lo = nullptr;
+    float *scale = nullptr;
+    float *ssum = nullptr;
+};
+
+// Store 128 consecutive activations held four per lane in an aligned 32-lane group (lane i holds
+// elements 4i..4i+3; an inactive group holds zeros).  elem0: this lane's first element in the row.
+__device__ inline void hact_store128(float4 v, bool active, const HAct &q, size_t row, int d, int elem0) {
+    float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    m = fmaxf(m, dpp_move<0xB1>(m));
+    m = fmaxf(m, dpp_move<0x4E>(m));
+    m = fmaxf(m, dpp_move<0x141>(m));
+    m = fmaxf(m, dpp_move<0x140>(m));
+    m = fmaxf(m, __shfl_xor(m, 16, 64));
+    // m = f * 2^ex with f in [0.5, 1): x / scale = x * 2^(10 - ex)
+    int ex = (int)((__float_as_uint(m) >> 23) & 255u) - 126;
+    ex = ex < -116 ? -116 : ex;
+    const float inv = __uint_as_float((uint32_t)(137 - ex) << 23);
+    const float scale = __uint_as_float((uint32_t)(117 + ex) << 23);
+    const float f[4] = {__fmul_rn(v.x, inv), __fmul_rn(v.y, inv), __fmul_rn(v.z, inv), __fmul_rn(v.w, inv)};
+    _Float16 hi[4], lo[4];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        hi[i] = (_Float16)f[i];
+        lo[i] = (_Float16)__fsub_rn(f[i], (float)hi[i]);
+        sum = __fadd_rn(sum, f[i]);
+    }
+    // 32 elements = 8 lanes
+    sum = __fadd_rn(sum, dpp_move<0xB1>(sum));
+    sum = __fadd_rn(sum, dpp_move<0x4E>(sum));
+    sum = __fadd_rn(sum, dpp_move<0x141>(sum));
+    if (active) {
+        uint2 hw, lw;
+        __builtin_memcpy(&hw, hi, 8);
+        __builtin_memcpy(&lw, lo, 8);
+        *(uint2 *)(q.hi + row * (size_t)d + elem0) = hw;
+        *(uint2 *)(q.lo + row * (size_t)d + elem0) = lw;
+        if ((elem0 & 31) == 0) q.ssum[row * (size_t)(d / 32) + (elem0 >> 5)] = sum;
+        if ((elem0 & 127) == 0) q.scale[row * (size_t)(d / 128) + (elem0 >> 7)] = scale;
+    }
+}
+
 }  // namespace mummu
