@@ -885,7 +885,7 @@ __device__ inline half2v biased_pair(uint32_t t, bool upper) {
 // tile.  With two waves to a column block each expands the weights of its columns itself (twice the vector work
 // in the workgroup) and keeps half the accumulators, which is what lets two workgroups share a CU without spills.
 template <bool GATE_UP, int MT, int WM, bool OUT_H>
-__global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
+__global__ __launch_bounds__(256 * WM, GATE_UP ? 2 : 3) void grouped_gemm_q4k_f16_kernel(
     const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, HAct a_in, const int32_t *__restrict__ sorted, int k_slots,
     const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim, HAct act_h, QAct64 act_q,
     float *__restrict__ y_out) {
@@ -895,7 +895,7 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
     static_assert(MT % WM == 0, "row blocks split evenly over the wave rows");
     __shared__ __attribute__((aligned(16))) uint8_t s_raw[L::kBytes];
     __shared__ __attribute__((aligned(16))) float s_as[2][BM];         // activation scale of a 128-element run, per tile row
-    __shared__ __attribute__((aligned(8))) _Float16 s_sum[2][BM][8];   // its four block sums: hi halfs, then lo halfs
+    __shared__ __attribute__((aligned(16))) _Float16 s_sum[2][BM][GATE_UP ? 16 : 8];   // block sums of one fold: hi halfs, then lo halfs
     auto s_a = [&](int buf, int plane, int row) -> _Float16 * {
         return (_Float16 *)(s_raw + (size_t)buf * L::kBuf + ((size_t)plane * BM + row) * kRow);
     };
@@ -933,14 +933,21 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
         a_off[p] = ((uint32_t)source_row(r) * (uint32_t)in_dim + (uint32_t)a_chunk * 8u) * 2u;
         a_lds[p] = (uint32_t)(((size_t)a_plane * BM + r) * kRow + a_chunk * 16);
     }
-    // block sums and scales of a 128-element run: thread -> (row tid / 4, block tid % 4)
-    // (threads past 4 BM repeat rows, and all four threads of a row store its scale: the same values twice, and no
-    // branch in the loop body - with basic blocks in it the compiler sinks one step's arithmetic into the next and
-    // keeps both steps' accumulators alive)
+    // Activation scales.  ROW (the gate/up side: x comes from quantize_rows_h, one scale for the whole row): the
+    // scale is applied once, in the epilogue, and a super-block is folded into acc in one go.  Otherwise (the down
+    // side: the gate/up epilogue knows only its own 128 columns) every 128-element run has its own scale and is
+    // folded on its own.
+    // Block sums: thread -> (row tid / 4 of the tile, quarter tid % 4 of the run's blocks).  Threads past 4 BM
+    // repeat rows and all four threads of a row store its scale: the same values twice, and no branch in the
+    // loop body - with basic blocks in it the compiler sinks one step's arithmetic into the next and keeps both
+    // steps' accumulators alive.
+    constexpr bool ROW = GATE_UP;
+    constexpr int NSUM = ROW ? 8 : 4;          // block sums per fold
     const int m_row = (tid >> 2) & (BM - 1), m_blk = tid & 3;
     const uint32_t src_m = (uint32_t)source_row(m_row);
-    const uint32_t sum_off = (src_m * (uint32_t)(in_dim / 32) + (uint32_t)m_blk) * 4u;
+    const uint32_t sum_off = (src_m * (uint32_t)(in_dim / 32) + (uint32_t)m_blk * (ROW ? 2u : 1u)) * 4u;
     const uint32_t scale_off = src_m * (uint32_t)(in_dim / 128) * 4u;
+    if (ROW) s_as[0][m_row] = *(const float *)((const uint8_t *)a_in.scale + scale_off);
 
     float16v acc[NB][MW], c1[NB][MW];
 #pragma unroll
@@ -950,9 +957,11 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[b][m][r] = c1[b][m][r] = 0.0f;
 
-    // weights: the raw bytes of the step being multiplied and of the next one, the header of the current
-    // super-block and, during its last step, of the next
-    u32x4 raw[2][NB], rh[NB], rh_next[NB];
+    // weights: the raw bytes of the step being multiplied and of the next one; of the current super-block d | dmin
+    // and its eight scales and eight offsets as bytes (sub-blocks 0-3, 4-7); the header of the next super-block
+    // during this one's last step
+    u32x4 raw[2][NB], rh_next[NB];
+    uint32_t dd[NB], sc4[NB][2], mn4[NB][2];
     auto load_b = [&](int k0, int st, u32x4 (&dst)[NB]) {
         const uint32_t o = b_off + (uint32_t)(k0 >> 8) * 144u;
 #pragma unroll
@@ -961,25 +970,54 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
             if (st == 0) rh_next[b] = *(const u32x4 *)(b_base[b] + (o - 16u * (uint32_t)g));
         }
     };
+    // ggml get_scale_min_k4 for all eight sub-blocks at once
+    auto unpack_header = [&]() {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t y = rh_next[b][1], z = rh_next[b][2], w = rh_next[b][3];
+            dd[b] = rh_next[b][0];
+            sc4[b][0] = y & 0x3F3F3F3Fu;
+            mn4[b][0] = z & 0x3F3F3F3Fu;
+            sc4[b][1] = (w & 0x0F0F0F0Fu) | ((y >> 2) & 0x30303030u);
+            mn4[b][1] = ((w >> 4) & 0x0F0F0F0Fu) | ((z >> 2) & 0x30303030u);
+        }
+    };
     // activations of one step in registers, then into a tile
     u32x4 ra[A_PASSES];
-    float rsum = 0.0f, rscale = 0.0f;
+    float rsum[ROW ? 2 : 1] = {}, rscale = 0.0f;
     auto load_a = [&](int k0, int st) {
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) ra[p] = *(const u32x4 *)(a_base + (a_off[p] + (uint32_t)k0 * 2u));
-        if ((st & 1) == 0) {
-            rsum = *(const float *)((const uint8_t *)a_in.ssum + (sum_off + (uint32_t)(k0 >> 5) * 4u));
+        if (ROW) {
+            if (st == 0) {
+                const float2 v = *(const float2 *)((const uint8_t *)a_in.ssum + (sum_off + (uint32_t)(k0 >> 5) * 4u));
+                rsum[0] = v.x;
+                rsum[ROW ? 1 : 0] = v.y;
+            }
+        } else if ((st & 1) == 0) {
+            rsum[0] = *(const float *)((const uint8_t *)a_in.ssum + (sum_off + (uint32_t)(k0 >> 5) * 4u));
             rscale = *(const float *)((const uint8_t *)a_in.scale + (scale_off + (uint32_t)(k0 >> 7) * 4u));
         }
     };
-    auto store_a = [&](int buf, int st, int pair_buf) {
+    // sum_buf: which of the two sets of block sums (they alternate per fold)
+    auto store_a = [&](int buf, int st, int sum_buf) {
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) *(u32x4 *)(s_raw + (size_t)buf * L::kBuf + a_lds[p]) = ra[p];
-        if ((st & 1) == 0) {
-            const _Float16 h = (_Float16)rsum;
-            s_sum[pair_buf][m_row][m_blk] = h;
-            s_sum[pair_buf][m_row][4 + m_blk] = (_Float16)__fsub_rn(rsum, (float)h);
-            s_as[pair_buf][m_row] = rscale;
+        if (ROW) {
+            if (st == 0) {
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const float v = rsum[ROW ? i : 0];
+                    const _Float16 h = (_Float16)v;
+                    s_sum[sum_buf][m_row][2 * m_blk + i] = h;
+                    s_sum[sum_buf][m_row][8 + 2 * m_blk + i] = (_Float16)__fsub_rn(v, (float)h);
+                }
+            }
+        } else if ((st & 1) == 0) {
+            const _Float16 h = (_Float16)rsum[0];
+            s_sum[sum_buf][m_row][m_blk] = h;
+            s_sum[sum_buf][m_row][4 + m_blk] = (_Float16)__fsub_rn(rsum[0], (float)h);
+            s_as[sum_buf][m_row] = rscale;
         }
     };
 
@@ -989,9 +1027,9 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
         half2v ml2[NB], al2[NB], mh2[NB], ah2[NB];
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            uint32_t scp, mnp;
-            k4_scale_min_both(rh[b][1], rh[b][2], rh[b][3], st, scp, mnp);
-            const float sc_lo = (float)(scp & 0xFFu), sc_hi = (float)((scp >> 8) & 0xFFu);
+            // sub-blocks 2 st (the low nibbles) and 2 st + 1 (the high nibbles)
+            const uint32_t sw = sc4[b][st >> 1] >> (16 * (st & 1));
+            const float sc_lo = (float)(sw & 0xFFu), sc_hi = (float)((sw >> 8) & 0xFFu);
             // low nibbles: (1024 + q) * sc - 1024 sc; high nibbles, left in place: (1024 + 16 q) * (sc / 16) - 64 sc
             const _Float16 ml = (_Float16)sc_lo, al = (_Float16)__fmul_rn(-1024.0f, sc_lo);
             const _Float16 mh = (_Float16)__fmul_rn(0.0625f, sc_hi), ah = (_Float16)__fmul_rn(-64.0f, sc_hi);
@@ -1011,6 +1049,7 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
                 a_lo[kk & 1][m] = *(const half8 *)(tile + (size_t)(BM + 32 * m) * kRow + a_byte);
             }
         };
+        const bool first = ROW ? st == 0 : (st & 1) == 0;   // the step that starts a new sum in c1
         read_a(0);
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
@@ -1032,36 +1071,52 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
             for (int m = 0; m < MW; m++) {
 #pragma unroll
                 for (int b = 0; b < NB; b++) {
-                    c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[kk & 1][m], bfrag[b], ((st & 1) == 0 && kk == 0) ? zero : c1[b][m], 0, 0, 0);
+                    c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[kk & 1][m], bfrag[b], (first && kk == 0) ? zero : c1[b][m], 0, 0, 0);
                     c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[kk & 1][m], bfrag[b], c1[b][m], 0, 0, 0);
                 }
             }
         }
     };
-    // the 128 elements just summed into c1 -> acc; pair: which half of the super-block
-    auto fold = [&](int pair, int pair_buf) {
+    // what has been summed into c1 -> acc.  part: which 128-element run of the super-block (the whole of it with
+    // one scale per row); sum_buf: which set of block sums
+    auto fold = [&](int part, int sum_buf) {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            const float d = half_bits_to_float((uint16_t)(rh[b][0] & 0xFFFFu));
-            const float ndmin = -half_bits_to_float((uint16_t)(rh[b][0] >> 16));
-            uint32_t sc0, mn0, sc1, mn1;
-            k4_scale_min_both(rh[b][1], rh[b][2], rh[b][3], 2 * pair, sc0, mn0);
-            k4_scale_min_both(rh[b][1], rh[b][2], rh[b][3], 2 * pair + 1, sc1, mn1);
-            const half4v bm = {(_Float16)(float)(mn0 & 0xFFu), (_Float16)(float)((mn0 >> 8) & 0xFFu), (_Float16)(float)(mn1 & 0xFFu),
-                               (_Float16)(float)((mn1 >> 8) & 0xFFu)};
+            const float d = half_bits_to_float((uint16_t)(dd[b] & 0xFFFFu));
+            const float ndmin = -half_bits_to_float((uint16_t)(dd[b] >> 16));
+            // the block offsets m as halfs (exact), in the order of the block sums
+            _Float16 mh[NSUM];
+#pragma unroll
+            for (int j = 0; j < NSUM; j++) {
+                const uint32_t word = ROW ? mn4[b][j >> 2] : mn4[b][part];
+                mh[j] = (_Float16)(float)((word >> (8 * (j & 3))) & 0xFFu);
+            }
 #pragma unroll
             for (int m = 0; m < MW; m++) {
-                const half4v am = *(const half4v *)&s_sum[pair_buf][row0 + 32 * m + (lane & 31)][4 * g];
-                const float16v c2 = __builtin_amdgcn_mfma_f32_32x32x8f16(am, bm, zero, 0, 0, 0);
+                float16v c2;
+                if constexpr (ROW) {
+                    // K = 16: the eight sums' hi halfs from lanes 0-31, their lo halfs from lanes 32-63
+                    const half8 am = *(const half8 *)&s_sum[sum_buf][row0 + 32 * m + (lane & 31)][8 * g];
+                    half8 bm;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const float4 s4 = *(const float4 *)&s_as[pair_buf][row0 + 32 * m + 8 * j + 4 * g];
-                    const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+                    for (int j = 0; j < 8; j++) bm[j] = mh[j];
+                    c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bm, zero, 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int r = 4 * j + i;
-                        const float u = fmaf(ndmin, c2[r], __fmul_rn(d, c1[b][m][r]));
-                        acc[b][m][r] = fmaf(u, sr[i], acc[b][m][r]);
+                    for (int r = 0; r < 16; r++) acc[b][m][r] = fmaf(ndmin, c2[r], fmaf(d, c1[b][m][r], acc[b][m][r]));
+                } else {
+                    const half4v am = *(const half4v *)&s_sum[sum_buf][row0 + 32 * m + (lane & 31)][4 * g];
+                    const half4v bm = {mh[0], mh[1], mh[2], mh[3]};
+                    c2 = __builtin_amdgcn_mfma_f32_32x32x8f16(am, bm, zero, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float4 s4 = *(const float4 *)&s_as[sum_buf][row0 + 32 * m + 8 * j + 4 * g];
+                        const float sr[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int r = 4 * j + i;
+                            const float u = fmaf(ndmin, c2[r], __fmul_rn(d, c1[b][m][r]));
+                            acc[b][m][r] = fmaf(u, sr[i], acc[b][m][r]);
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);  // (one 32 x 32 block at a time: scheduled together they do not fit the registers)
@@ -1081,11 +1136,12 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
         // (after the last step the "next" one is step 0 again: loaded and stored like any other, never multiplied;
         // no branch in the loop body)
         const int k_next = (st == 3 && sb0 + 256 >= in_dim) ? 0 : sb0 + kBK * (st + 1);
+        // block sums alternate between two sets: per super-block with one scale per row, else per 128-element run
+        const int sb_par = (sb0 >> 8) & 1;
+        const int sum_buf = ROW ? sb_par : (st >> 1) & 1;
+        const int sum_buf_next = ROW ? (st == 3 ? sb_par ^ 1 : sb_par) : (((st + 1) & 3) >> 1) & 1;
         MUMMU_TIMER_MARK(0);
-        if (st == 0) {
-#pragma unroll
-            for (int b = 0; b < NB; b++) rh[b] = rh_next[b];
-        }
+        if (st == 0) unpack_header();
         // the next step: weights into the other set of registers, activations into registers
         load_b(k_next, (st + 1) & 3, raw[(st + 1) & 1]);
         load_a(k_next, (st + 1) & 3);
@@ -1093,11 +1149,11 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
         MUMMU_TIMER_MARK(1);
         multiply(st, st & 1, raw[st & 1]);
         MUMMU_TIMER_MARK(2);
-        if (st & 1) fold(st >> 1, (st >> 1) & 1);
+        if (ROW ? st == 3 : (st & 1) == 1) fold(st >> 1, sum_buf);
         MUMMU_TIMER_MARK(3);
         MUMMU_CODE_FENCE();
         // ... and into the tile that the step before this one was read from
-        store_a((st + 1) & 1, (st + 1) & 3, (((st + 1) & 3) >> 1) & 1);
+        store_a((st + 1) & 1, (st + 1) & 3, sum_buf_next);
         MUMMU_TIMER_MARK(4);
         __syncthreads();
         MUMMU_TIMER_MARK(5);
@@ -1118,7 +1174,12 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
         for (int m = 0; m < MW; m++)
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                s_c[(row0 + 32 * m + acc_row(r, lane)) * kLdsC + col] = __fmul_rn(det_silu(acc[0][m][r]), acc[NB - 1][m][r]);
+            {
+                // (one scale per row on this side: both products take it here)
+                const float sr = s_as[0][row0 + 32 * m + acc_row(r, lane)];
+                s_c[(row0 + 32 * m + acc_row(r, lane)) * kLdsC + col] =
+                    __fmul_rn(det_silu(__fmul_rn(sr, acc[0][m][r])), __fmul_rn(sr, acc[NB - 1][m][r]));
+            }
         __syncthreads();
         if (OUT_H) {
             const int grp = tid >> 5, l32 = tid & 31;
@@ -1154,19 +1215,32 @@ __global__ __launch_bounds__(256 * WM, 2) void grouped_gemm_q4k_f16_kernel(
     }
 }
 
-// x [n, d] f32 -> HAct: one 32-lane group per 128-element block.
+// x [n, d] f32 -> HAct with one scale per row: a workgroup per row finds the row's largest magnitude, then
+// stores the row 1024 elements at a time.
 __global__ __launch_bounds__(256) void quantize_rows_h_kernel(const float *__restrict__ x, int d, HAct q) {
-    const int row = blockIdx.y;
-    const int elem0 = (blockIdx.x * 256 + threadIdx.x) * 4;
-    const bool active = elem0 < d;
-    const float4 v = active ? *(const float4 *)(x + (size_t)row * (size_t)d + elem0) : make_float4(0.f, 0.f, 0.f, 0.f);
-    hact_store128(v, active, q, (size_t)row, d, elem0);
+    __shared__ float s_max[4];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float *xr = x + (size_t)row * (size_t)d;
+    float m = 0.0f;
+    for (int e0 = tid * 4; e0 < d; e0 += 1024) {
+        const float4 v = *(const float4 *)(xr + e0);
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+    m = wave_max(m);
+    if ((tid & 63) == 0) s_max[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    for (int e0 = tid * 4; e0 - tid * 4 < d; e0 += 1024) {   // (whole 32-lane groups run together: d is a multiple of 128)
+        const bool active = e0 < d;
+        const float4 v = active ? *(const float4 *)(xr + e0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        hact_store128(v, active, q, (size_t)row, d, e0, m);
+    }
 }
 
 hipError_t launch_quantize_rows_h(const float *x, int n, int d, HAct q, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     if (d % 128 != 0) return hipErrorInvalidValue;
-    launch_kernel(quantize_rows_h_kernel, dim3((d + 1023) / 1024, n), dim3(256), 0, s, x, d, q);
+    launch_kernel(quantize_rows_h_kernel, dim3(n), dim3(256), 0, s, x, d, q);
     return hipGetLastError();
 }
 

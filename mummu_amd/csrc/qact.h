@@ -102,10 +102,12 @@ __device__ inline void quantize_store64(float4 v, bool active, const QAct64 &q, 
 }
 
 // Activations for the products of Q4_K banks on the f16 matrix units: every element as a pair of
-// halfs, x = scale * (hi + lo) with hi = f16(x / scale), lo = f16(x / scale - hi), one power-of-two
-// scale per 128 elements chosen so that the block's largest |x / scale| lies in [2^9, 2^10): 22
-// significant bits per element (elements more than 2^24 below their block's largest keep an absolute
-// error of 2^-25 of it), and sums of 32 scaled elements stay below 2^15, inside a half's range.
+// halfs, x = scale * (hi + lo) with hi = f16(x / scale), lo = f16(x / scale - hi), and a power-of-two
+// scale chosen so that the largest |x / scale| it covers lies in [2^9, 2^10): 22 significant bits per
+// element (elements more than 2^24 below that largest one keep an absolute error of 2^-25 of it), and
+// sums of 32 scaled elements stay below 2^15, inside a half's range.  The scale array has one entry per
+// 128 elements; a producer that sees whole rows (quantize_rows_h) writes the same scale into all of a
+// row's entries, one that sees 128 columns at a time (the gate/up epilogue) a scale per entry.
 //   hi, lo : f16 [rows][D]      scale : f32 [rows][D/128]      ssum : f32 [rows][D/32], sum of x / scale
 struct HAct {
     _Float16 *hi = nullptr;
@@ -114,20 +116,29 @@ struct HAct {
     float *ssum = nullptr;
 };
 
-// Store 128 consecutive activations held four per lane in an aligned 32-lane group (lane i holds
-// elements 4i..4i+3; an inactive group holds zeros).  elem0: this lane's first element in the row.
-__device__ inline void hact_store128(float4 v, bool active, const HAct &q, size_t row, int d, int elem0) {
-    float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    m = fmaxf(m, dpp_move<0xB1>(m));
-    m = fmaxf(m, dpp_move<0x4E>(m));
-    m = fmaxf(m, dpp_move<0x141>(m));
-    m = fmaxf(m, dpp_move<0x140>(m));
-    m = fmaxf(m, __shfl_xor(m, 16, 64));
-    // m = f * 2^ex with f in [0.5, 1): x / scale = x * 2^(10 - ex)
+// The scale for a largest magnitude m = f * 2^ex, f in [0.5, 1): x / scale = x * 2^(10 - ex).
+__device__ inline void hact_scale_of(float m, float &inv, float &scale) {
     int ex = (int)((__float_as_uint(m) >> 23) & 255u) - 126;
     ex = ex < -116 ? -116 : ex;
-    const float inv = __uint_as_float((uint32_t)(137 - ex) << 23);
-    const float scale = __uint_as_float((uint32_t)(117 + ex) << 23);
+    inv = __uint_as_float((uint32_t)(137 - ex) << 23);
+    scale = __uint_as_float((uint32_t)(117 + ex) << 23);
+}
+
+// Store 128 consecutive activations held four per lane in an aligned 32-lane group (lane i holds
+// elements 4i..4i+3; an inactive group holds zeros).  elem0: this lane's first element in the row.
+// row_max < 0: the scale comes from these 128 elements; else from row_max, the largest magnitude of the row.
+__device__ inline void hact_store128(float4 v, bool active, const HAct &q, size_t row, int d, int elem0, float row_max = -1.0f) {
+    float m = row_max;
+    if (row_max < 0.0f) {
+        m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = fmaxf(m, dpp_move<0xB1>(m));
+        m = fmaxf(m, dpp_move<0x4E>(m));
+        m = fmaxf(m, dpp_move<0x141>(m));
+        m = fmaxf(m, dpp_move<0x140>(m));
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+    }
+    float inv, scale;
+    hact_scale_of(m, inv, scale);
     const float f[4] = {__fmul_rn(v.x, inv), __fmul_rn(v.y, inv), __fmul_rn(v.z, inv), __fmul_rn(v.w, inv)};
     _Float16 hi[4], lo[4];
     float sum = 0.0f;
