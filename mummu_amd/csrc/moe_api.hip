@@ -793,8 +793,10 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
 
     mummu_moe *h = new mummu_moe();
     h->cfg = *cfg;
-    // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
+    // MUMMU_GEMM_Q4K_F16=0: Q4_K banks of the batched path stay on the int8 units (the form every other block-quantized
+    // type takes) instead of the f16 units
     if (const char *e = getenv("MUMMU_GEMM_Q4K_F16")) h->gemm_q4k_f16 = atoi(e) != 0;
+    // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
     if (const char *e = getenv("MUMMU_GEMM_MIN_TOKENS")) {
         const int v = atoi(e);
         if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = h->gemm_min_f32 = v;
