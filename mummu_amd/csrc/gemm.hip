@@ -77,17 +77,17 @@ __device__ inline bool xcd_tile(const int32_t *__restrict__ n_tiles, int slabs, 
 // F16 banks
 // ---------------------------------------------------------------------------------------
 
-// GATE_UP: A = x (f32, gathered by token through `sorted`), two weight matrices, epilogue
-//          act16[pos, n] = f16(silu(g) * u).
+// GATE_UP: A = x rounded to f16 (one small launch before this one: every output slab of a tile gathers the
+//          tile's rows again, and as halfs that is half the traffic), rows gathered by token through `sorted`;
+//          two weight matrices, epilogue act16[pos, n] = f16(silu(g) * u).
 // else   : A = act16 (f16, rows already in sorted order), one matrix, y[pos, n] = f32 sum.
 // BF16: the banks hold bf16; every weight becomes a half on its way into LDS (exact from 2^-14 up:
 // a bf16 has 8 significant bits; smaller weights keep an absolute error below 2^-25).
 template <bool GATE_UP, int MT, bool BF16>
 __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
-    const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const float *__restrict__ x,
-    const _Float16 *__restrict__ act_in, const int32_t *__restrict__ sorted, int k_slots,
-    const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles, int in_dim, int out_dim,
-    _Float16 *__restrict__ act_out, float *__restrict__ y_out) {
+    const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const _Float16 *__restrict__ act_in,
+    const int32_t *__restrict__ sorted, int k_slots, const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles,
+    int in_dim, int out_dim, _Float16 *__restrict__ act_out, float *__restrict__ y_out) {
     constexpr int NB = GATE_UP ? 2 : 1;
     constexpr int BM = 32 * MT;
     __shared__ __attribute__((aligned(16))) _Float16 s_a[BM][kLds];
@@ -112,26 +112,18 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
         if (GATE_UP) b_ptr[NB - 1][i] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_chunk * 16;
     }
 
-    // activation tile: f32 source -> 16 threads per row, 4 elements each (2*MT passes of 16 rows);
-    // f16 source -> 8 threads per row, 8 elements each (MT passes of 32 rows)
-    constexpr int A_PASSES = GATE_UP ? 2 * MT : MT;
-    const int a_col = GATE_UP ? (tid & 15) * 4 : (tid & 7) * 8;
+    // activation tile: 8 threads per row, 8 halfs each (MT passes of 32 rows)
+    constexpr int A_PASSES = MT;
+    const int a_col = (tid & 7) * 8;
     // rows past the tile's end read the tile's last row: their products are never stored
-    const float *a_src32[A_PASSES];
     const _Float16 *a_src16[A_PASSES];
     int a_row[A_PASSES];
 #pragma unroll
     for (int p = 0; p < A_PASSES; p++) {
-        a_row[p] = GATE_UP ? p * 16 + (tid >> 4) : p * 32 + (tid >> 3);
+        a_row[p] = p * 32 + (tid >> 3);
         const int r = a_row[p] < rows ? a_row[p] : rows - 1;
-        if (GATE_UP) {
-            const int a = sorted[p0 + r];
-            a_src32[p] = x + (size_t)(a / k_slots) * (size_t)in_dim + a_col;
-            a_src16[p] = nullptr;
-        } else {
-            a_src16[p] = act_in + (size_t)(p0 + r) * (size_t)in_dim + a_col;
-            a_src32[p] = nullptr;
-        }
+        const int src = GATE_UP ? sorted[p0 + r] / k_slots : p0 + r;
+        a_src16[p] = act_in + (size_t)src * (size_t)in_dim + a_col;
     }
 
     float16v acc[NB][MT];
@@ -143,7 +135,6 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
             for (int r = 0; r < 16; r++) acc[b][m][r] = 0.0f;
 
     u32x4 rb[NB][4];
-    f32x4 ra32[A_PASSES];
     u32x4 ra16[A_PASSES];
     auto fetch = [&](int k0) {
 #pragma unroll
@@ -151,10 +142,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
 #pragma unroll
             for (int i = 0; i < 4; i++) rb[b][i] = *(const u32x4 *)(b_ptr[b][i] + (size_t)k0 * 2);
 #pragma unroll
-        for (int p = 0; p < A_PASSES; p++) {
-            if (GATE_UP) ra32[p] = *(const f32x4 *)(a_src32[p] + k0);
-            else ra16[p] = *(const u32x4 *)(a_src16[p] + k0);
-        }
+        for (int p = 0; p < A_PASSES; p++) ra16[p] = *(const u32x4 *)(a_src16[p] + k0);
     };
     // The K loop starts at a slab-dependent step and wraps.  An f16 row of 2048 elements is 4096
     // bytes - the period of the memory channel interleave - so one K step of ALL rows lives in one
@@ -184,14 +172,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
                 *(u32x4 *)&s_b[b][(tid >> 3) + 32 * i][b_chunk * 8] = v;
             }
 #pragma unroll
-        for (int p = 0; p < A_PASSES; p++) {
-            if (GATE_UP) {
-                uint2 v = make_uint2(pack_half2(ra32[p].x, ra32[p].y), pack_half2(ra32[p].z, ra32[p].w));
-                *(uint2 *)&s_a[a_row[p]][a_col] = v;
-            } else {
-                *(u32x4 *)&s_a[a_row[p]][a_col] = ra16[p];
-            }
-        }
+        for (int p = 0; p < A_PASSES; p++) *(u32x4 *)&s_a[a_row[p]][a_col] = ra16[p];
         MUMMU_TIMER_MARK(1);
         __syncthreads();
         MUMMU_TIMER_MARK(2);
@@ -1237,6 +1218,22 @@ __global__ __launch_bounds__(256) void quantize_rows_h_kernel(const float *__res
     }
 }
 
+// x [n, d] f32 -> f16, round to nearest.
+__global__ __launch_bounds__(256) void convert_rows_f16_kernel(const float *__restrict__ x, size_t count, _Float16 *__restrict__ out) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= count) return;
+    const float4 v = *(const float4 *)(x + i);
+    *(uint2 *)(out + i) = make_uint2(pack_half2(v.x, v.y), pack_half2(v.z, v.w));
+}
+
+hipError_t launch_convert_rows_f16(const float *x, int n, int d, _Float16 *out, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (d % 4 != 0) return hipErrorInvalidValue;
+    const size_t count = (size_t)n * (size_t)d;
+    launch_kernel(convert_rows_f16_kernel, dim3((unsigned)((count / 4 + 255) / 256)), dim3(256), 0, s, x, count, out);
+    return hipGetLastError();
+}
+
 hipError_t launch_quantize_rows_h(const float *x, int n, int d, HAct q, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     if (d % 128 != 0) return hipErrorInvalidValue;
@@ -1357,13 +1354,13 @@ static hipError_t launch_gemm_f32(const uint8_t *w0, const uint8_t *w1, const fl
 }
 
 template <bool GATE_UP, bool BF16>
-static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const float *x, const _Float16 *act_in,
+static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const _Float16 *act_in,
                                   const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
                                   int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
                                   hipStream_t s) {
     dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
 #define MUMMU_F16(MT)                                                                                                    \
-    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT, BF16>, grid, block, 0, s, w0, w1, x, act_in, sorted, k_slots, tiles, n_tiles, \
+    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT, BF16>, grid, block, 0, s, w0, w1, act_in, sorted, k_slots, tiles, n_tiles, \
                   in_dim, out_dim, act_out, y_out)
     switch (tile_rows) {
     case 32: MUMMU_F16(1); break;
@@ -1380,7 +1377,7 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
                                float *act32, QAct64 actq, HAct acth, hipStream_t s) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
-    if (xh.hi != nullptr) {
+    if (xh.hi != nullptr && xh.lo != nullptr) {
         if (!grouped_gemm_q4k_f16(b)) return hipErrorInvalidValue;
         const bool out_h = acth.hi != nullptr;
         if (out_h && !grouped_gemm_q4k_f16_down(b)) return hipErrorInvalidValue;
@@ -1390,11 +1387,13 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     if (b.gate_type == T_F32)
         return launch_gemm_f32<true>(b.gate, b.up, x, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden, b.inter, act32,
                                      nullptr, s);
+    // (f16 and bf16 banks read x as halfs: xh.hi alone, from launch_convert_rows_f16)
+    if ((b.gate_type == T_F16 || b.gate_type == T_BF16) && xh.hi == nullptr) return hipErrorInvalidValue;
     if (b.gate_type == T_F16)
-        return launch_gemm_f16<true, false>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+        return launch_gemm_f16<true, false>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
                                             b.inter, (_Float16 *)act16, nullptr, s);
     if (b.gate_type == T_BF16)
-        return launch_gemm_f16<true, true>(b.gate, b.up, x, nullptr, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+        return launch_gemm_f16<true, true>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
                                            b.inter, (_Float16 *)act16, nullptr, s);
     switch (b.gate_type) {
 #define MUMMU_GU(T)                                                                                                          \
@@ -1427,10 +1426,10 @@ hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float
                                       nullptr, y, s);
     const bool few_rows = n_assign <= 64 * b.n_experts;  // an expert's rows fit one tile, on average
     if (b.down_type == T_F16)
-        return launch_gemm_f16<false, false>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+        return launch_gemm_f16<false, false>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
                                              tile_rows, b.inter, b.hidden, nullptr, y, s);
     if (b.down_type == T_BF16)
-        return launch_gemm_f16<false, true>(b.down, nullptr, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+        return launch_gemm_f16<false, true>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
                                             tile_rows, b.inter, b.hidden, nullptr, y, s);
     switch (b.down_type) {
 #define MUMMU_DN(T)                                                                                                      \

@@ -162,6 +162,8 @@ bool grouped_gemm_q4k_f16(const ExpertBanks &b);
 bool grouped_gemm_q4k_f16_down(const ExpertBanks &b);
 // x [n, d] f32 -> HAct (d % 128 == 0).
 hipError_t launch_quantize_rows_h(const float *x, int n, int d, HAct q, hipStream_t s);
+// x [n, d] f32 -> halfs (d % 4 == 0): what the gate/up launch of f16 and bf16 banks reads (as xh.hi, nothing else set).
+hipError_t launch_convert_rows_f16(const float *x, int n, int d, _Float16 *out, hipStream_t s);
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, HAct xh, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
                                float *act32, QAct64 actq, HAct acth, hipStream_t s);

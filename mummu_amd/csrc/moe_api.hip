@@ -450,9 +450,13 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         // Q4_K banks on the f16 units: x as pairs of halfs in the (not yet written) buffer of the down product's
         // output, the activations between the two products in the f16 and f32 activation buffers
         const bool hf = h->gemm_q4k_f16 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
-        const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum} : HAct();
+        // (f16 / bf16 banks: x as halfs in the same buffer)
+        const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
+        const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum}
+                           : (half_banks ? HAct{(_Float16 *)h->y, nullptr, nullptr, nullptr} : HAct());
         const HAct acth = hf_down ? HAct{(_Float16 *)h->act16, (_Float16 *)h->act, h->actq.scale, (float *)h->actq.sum} : HAct();
         if (hf) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows_h(x, (int)n, b.hidden, xh, s));
+        else if (half_banks) LAUNCH(h, K_QUANTIZE, s, launch_convert_rows_f16(x, (int)n, b.hidden, xh.hi, s));
         else if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
         LAUNCH(h, K_DISPATCH, s,
                launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch,
@@ -643,9 +647,12 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
         // (the routed path may have left the 16-bit activations in the decode layout, or not made them)
         // (Q4_K on the f16 units as in the routed path; the routed products are done with their output buffer)
         const bool hf = h->gemm_q4k_f16 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
-        const HAct xh = hf ? HAct{(_Float16 *)h->sh_y, (_Float16 *)h->sh_y + (size_t)n * H, h->xq.scale, (float *)h->xq.sum} : HAct();
+        const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
+        const HAct xh = hf ? HAct{(_Float16 *)h->sh_y, (_Float16 *)h->sh_y + (size_t)n * H, h->xq.scale, (float *)h->xq.sum}
+                           : (half_banks ? HAct{(_Float16 *)h->sh_y, nullptr, nullptr, nullptr} : HAct());
         const HAct acth = hf_down ? HAct{(_Float16 *)h->sh_act16, (_Float16 *)h->sh_act, h->sh_actq.scale, (float *)h->sh_actq.sum} : HAct();
         if (hf) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows_h(x, (int)n, H, xh, s));
+        else if (half_banks) LAUNCH(h, K_QUANTIZE, s, launch_convert_rows_f16(x, (int)n, H, xh.hi, s));
         else if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, H, xq64, s));
         LAUNCH(h, K_SHARED, s,
                launch_gemm_gate_up(b, x, xq64, xh, h->sh_sorted, 1, h->sh_tiles, h->sh_ntiles, h->sh_max_tiles, tile_rows, h->sh_act16,
