@@ -202,7 +202,14 @@ MUMMU_API int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, in
  * block's maximum keeps 5 bits.  This shows in one corner: a token whose SwiGLU hidden row is all but zero except
  * for one or two elements (every gate pre-activation far below zero) has outputs orders of magnitude below the
  * batch's, and relative to THAT magnitude single elements come out up to 4e-3 off (2e-8 of the batch's typical
- * output).  F32 / F16 / BF16 banks do not take this path (f32 or f16 products). */
+ * output).  F32 / F16 / BF16 banks do not take this path (f32 or f16 products).
+ * One exception on the batched path: Q4_K gate/up (and down) banks.  A Q4_K weight is d * (sc * q) - dmin * m
+ * with sc * q < 1024 an exact half, so their grouped GEMM runs on the f16 matrix units against activations held
+ * as PAIRS of halfs, x = 2^e * (hi + lo), hi = f16(x / 2^e), lo = f16(x / 2^e - hi), 2^e one power of two per row
+ * (per 128 elements between the two products): 22 significant bits per element, every element of a row down to
+ * 2^-24 of the row's largest.  That form measures 2e-6 by the reference's measure and has no such corner; it is
+ * also the faster one.  The environment variable MUMMU_GEMM_Q4K_F16=0, read by mummu_moe_create, keeps Q4_K on the
+ * integer form above. */
 
 /* ---- device-pointer entry points (no host copies, no synchronisation) ------------------
  * stream is a hipStream_t (NULL = the null stream).  Safe to capture into a HIP graph:
