@@ -1309,7 +1309,9 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
 }
 
 bool grouped_gemm_q4k_f16(const ExpertBanks &b) {
-    return b.gate_type == T_Q4_K && b.up_type == T_Q4_K && b.hidden % 256 == 0 && b.inter % 128 == 0;
+    // (one expert's matrix is addressed with 32-bit byte offsets)
+    return b.gate_type == T_Q4_K && b.up_type == T_Q4_K && b.hidden % 256 == 0 && b.inter % 128 == 0 &&
+           (size_t)b.hidden * (size_t)b.inter < (1ull << 32);
 }
 
 bool grouped_gemm_q4k_f16_down(const ExpertBanks &b) {

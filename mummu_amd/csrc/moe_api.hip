@@ -449,7 +449,9 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
         // Q4_K banks on the f16 units: x as pairs of halfs in the (not yet written) buffer of the down product's
         // output, the activations between the two products in the f16 and f32 activation buffers
-        const bool hf = h->gemm_q4k_f16 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
+        // (its kernels address the activation planes with 32-bit byte offsets)
+        const bool small32 = (size_t)na * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
+        const bool hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
         // (f16 / bf16 banks: x as halfs in the same buffer)
         const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
         const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum}
@@ -646,7 +648,8 @@ int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int 
         LAUNCH(h, K_SHARED, s, launch_identity_tiles((int)n, tile_rows, h->sh_sorted, h->sh_tiles, h->sh_ntiles, s));
         // (the routed path may have left the 16-bit activations in the decode layout, or not made them)
         // (Q4_K on the f16 units as in the routed path; the routed products are done with their output buffer)
-        const bool hf = h->gemm_q4k_f16 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
+        const bool small32 = (size_t)n * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
+        const bool hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
         const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
         const HAct xh = hf ? HAct{(_Float16 *)h->sh_y, (_Float16 *)h->sh_y + (size_t)n * H, h->xq.scale, (float *)h->xq.sum}
                            : (half_banks ? HAct{(_Float16 *)h->sh_y, nullptr, nullptr, nullptr} : HAct());
