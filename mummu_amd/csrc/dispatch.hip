@@ -8,18 +8,18 @@
 // every expert's segment lists its assignments in ascending a = token*k + slot, which is that
 // order.
 //
-// Three small launches over chunks of 1024 assignments (one fused launch of one workgroup when
-// there is a single chunk, where the launches themselves are most of the time):
+// Two small launches over chunks of 1024 assignments (one fused launch of one workgroup when there is a single
+// chunk, where the launches themselves are most of the time):
 //   count   per chunk: every assignment's rank among the chunk's assignments to the same expert
 //           (wave ballots, then a prefix over the workgroup's 16 waves in LDS) and the chunk's
 //           per-expert counts
-//   scan    one workgroup: per expert the running count over chunks and the total (also added to
-//           the layer's hit counters when asked: 8 atomics per token from the router would all
-//           land on the same few cache lines), the exclusive
-//           scan over experts (offsets), and the grouped GEMM's work list of
-//           (expert, first sorted position, rows <= tile_rows) triples - every expert writes its
-//           own tiles at the position an exclusive scan of the tile counts gives it
-//   place   per chunk: position = offsets[e] + chunk_base[chunk][e] + rank
+//   scan + place   per chunk: per expert the count over the chunks before this one and the total, the
+//           exclusive scan of the totals over experts (offsets), then
+//           position = offsets[e] + rows of e in earlier chunks + rank.  Workgroup 0 also adds the totals to
+//           the layer's hit counters when asked (8 atomics per token from the router would all land on the same
+//           few cache lines) and writes the grouped GEMM's work list of (expert, first sorted position,
+//           rows <= tile_rows) triples - every expert writes its own tiles at the position an exclusive scan of
+//           the tile counts gives it
 //
 // Outputs (device):
 //   offsets[E+1]      expert e owns sorted positions [offsets[e], offsets[e+1])
@@ -77,26 +77,28 @@ __global__ __launch_bounds__(kDispatchThreads) void dispatch_count_kernel(const 
     }
 }
 
-// counts[chunk][e] -> exclusive running count over chunks (in place); offsets; tiles.
-__global__ __launch_bounds__(kDispatchMaxExperts) void dispatch_scan_kernel(int32_t *__restrict__ counts, int n_chunks,
-                                                                            int n_experts, int tile_rows,
-                                                                            int32_t *__restrict__ offsets,
-                                                                            int32_t *__restrict__ tiles,
-                                                                            int32_t *__restrict__ n_tiles,
-                                                                            unsigned long long *__restrict__ hits) {
+// scan + place: every chunk's workgroup scans the (chunks x experts) counts for itself - a few thousand integers out
+// of L2 - instead of waiting for a launch of one workgroup to do it once (a third launch costs 4-5 us, the repeated
+// scan a fraction of that even at 64k tokens); workgroup 0 also writes offsets, the tile list and the hit counters.
+__global__ __launch_bounds__(kDispatchThreads) void dispatch_scan_place_kernel(
+    const int32_t *__restrict__ ids, int n_assign, int n_experts, int n_chunks, int tile_rows,
+    const int32_t *__restrict__ rank_in, const int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
+    int32_t *__restrict__ sorted, int32_t *__restrict__ inv, int32_t *__restrict__ tiles, int32_t *__restrict__ n_tiles,
+    unsigned long long *__restrict__ hits) {
     __shared__ int s_carry[kDispatchMaxExperts / 64][2];
-    const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
-    int total = 0;
+    __shared__ int s_pos[kDispatchMaxExperts];   // offsets[e] + rows of e in the chunks before this one
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int chunk = blockIdx.x;
+    const int e = tid;
+    int total = 0, before = 0;
     if (e < n_experts) {
         for (int c = 0; c < n_chunks; c++) {
             const int v = counts[(size_t)c * n_experts + e];
-            counts[(size_t)c * n_experts + e] = total;
+            before += c < chunk ? v : 0;
             total += v;
         }
     }
     const int my_tiles = (total + tile_rows - 1) / tile_rows;
-    // exclusive scans over experts of the totals and of the tile counts: inside each wave, then
-    // over the (at most 8) wave sums
     int incl = total, incl_t = my_tiles;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -106,54 +108,48 @@ __global__ __launch_bounds__(kDispatchMaxExperts) void dispatch_scan_kernel(int3
             incl_t += up_t;
         }
     }
-    if (lane == 63) {
+    if (lane == 63 && wave < kDispatchMaxExperts / 64) {
         s_carry[wave][0] = incl;
         s_carry[wave][1] = incl_t;
     }
     __syncthreads();
-    int base = 0, base_t = 0;
-    for (int w = 0; w < wave; w++) {
-        base += s_carry[w][0];
-        base_t += s_carry[w][1];
-    }
-    const int begin = base + incl - total;
     if (e < n_experts) {
-        if (hits) hits[e] += (unsigned long long)total;  // rows served per expert (nn/moe.rs:1562-1564)
-        offsets[e] = begin;
-        if (e == n_experts - 1) offsets[n_experts] = begin + total;
-        if (tiles != nullptr) {
-            int nt = base_t + incl_t - my_tiles;
-            for (int r = 0; r < total; r += tile_rows, nt++) {
-                tiles[3 * nt] = e;
-                tiles[3 * nt + 1] = begin + r;
-                tiles[3 * nt + 2] = (total - r) < tile_rows ? (total - r) : tile_rows;
+        int base = 0, base_t = 0;
+        for (int w = 0; w < wave; w++) {
+            base += s_carry[w][0];
+            base_t += s_carry[w][1];
+        }
+        const int begin = base + incl - total;
+        s_pos[e] = begin + before;
+        if (chunk == 0) {
+            if (hits) hits[e] += (unsigned long long)total;  // rows served per expert (nn/moe.rs:1562-1564)
+            offsets[e] = begin;
+            if (e == n_experts - 1) offsets[n_experts] = begin + total;
+            if (tiles != nullptr) {
+                int nt = base_t + incl_t - my_tiles;
+                for (int r = 0; r < total; r += tile_rows, nt++) {
+                    tiles[3 * nt] = e;
+                    tiles[3 * nt + 1] = begin + r;
+                    tiles[3 * nt + 2] = (total - r) < tile_rows ? (total - r) : tile_rows;
+                }
+                if (e == n_experts - 1) *n_tiles = base_t + incl_t;
             }
-            if (e == n_experts - 1) *n_tiles = base_t + incl_t;
         }
     }
-}
-
-__global__ __launch_bounds__(kDispatchThreads) void dispatch_place_kernel(const int32_t *__restrict__ ids, int n_assign,
-                                                                          int n_experts,
-                                                                          const int32_t *__restrict__ rank_in,
-                                                                          const int32_t *__restrict__ chunk_base,
-                                                                          const int32_t *__restrict__ offsets,
-                                                                          int32_t *__restrict__ sorted,
-                                                                          int32_t *__restrict__ inv) {
-    const int a = blockIdx.x * kDispatchThreads + threadIdx.x;
+    __syncthreads();
+    const int a = chunk * kDispatchThreads + tid;
     if (a >= n_assign) return;
-    const int e = ids[a];
-    if ((unsigned)e >= (unsigned)n_experts) return;
-    const int pos = offsets[e] + chunk_base[(size_t)blockIdx.x * n_experts + e] + rank_in[a];
+    const int ea = ids[a];
+    if ((unsigned)ea >= (unsigned)n_experts) return;
+    const int pos = s_pos[ea] + rank_in[a];
     sorted[pos] = a;
     inv[a] = pos;
 }
 
-
 // The three steps above in one launch of one workgroup, for batches of at most kFusedChunks
 // chunks: the per-chunk counts never leave LDS and every thread keeps its assignments' experts and
 // ranks in registers between the steps.  Same outputs, element for element.  One workgroup takes
-// about 7 us per chunk against 15 us for the three launches whatever the size, so this form only
+// about 7 us per chunk against 10 us for the two launches whatever the size, so this form only
 // serves a single chunk (up to 1024 assignments).
 constexpr int kFusedChunks = 1;
 
@@ -303,17 +299,15 @@ hipError_t launch_dispatch(const int32_t *ids, int n_assign, int n_experts, int 
         return hipGetLastError();
     }
     int32_t *rank = scratch, *counts = scratch + n_assign;
-    // per-kernel timing brackets the three launches as one: start from the first, stop from the last
+    // per-kernel timing brackets the two launches as one: start from the first, stop from the last
     const LaunchTiming timing = g_launch_timing;
     g_launch_timing.stop = nullptr;
     launch_kernel(dispatch_count_kernel, dim3(chunks), dim3(kDispatchThreads), 0, s, ids, n_assign, n_experts, rank, counts,
                   flags);
     g_launch_timing.start = nullptr;
-    launch_kernel(dispatch_scan_kernel, dim3(1), dim3(kDispatchMaxExperts), 0, s, counts, chunks, n_experts, tile_rows,
-                  offsets, tiles, n_tiles, hits);
     g_launch_timing.stop = timing.stop;
-    launch_kernel(dispatch_place_kernel, dim3(chunks), dim3(kDispatchThreads), 0, s, ids, n_assign, n_experts,
-                  (const int32_t *)rank, (const int32_t *)counts, (const int32_t *)offsets, sorted, inv);
+    launch_kernel(dispatch_scan_place_kernel, dim3(chunks), dim3(kDispatchThreads), 0, s, ids, n_assign, n_experts, chunks,
+                  tile_rows, (const int32_t *)rank, (const int32_t *)counts, offsets, sorted, inv, tiles, n_tiles, hits);
     g_launch_timing = timing;
     return hipGetLastError();
 }
