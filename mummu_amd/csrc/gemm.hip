@@ -20,6 +20,7 @@
 //                    integer sums are exact, C = 256*C_hi + C_lo, and the f32 accumulator takes
 //                    s * sum_blocks(d_block * C).  Q4_K's offset term -dmin*m*sum(x) is one
 //                    v_mfma_f32_32x32x2_f32 per K step over the per-block activation sums.
+#include <cmath>
 #include <type_traits>
 
 #include "device_utils.h"
@@ -1048,14 +1049,18 @@ __global__ __launch_bounds__(256 * WM, GATE_UP ? 2 : 3) void grouped_gemm_q4k_f1
                 f[3] = __builtin_elementwise_fma(biased_pair(w_b & mask, true), mul, add);
                 __builtin_memcpy(&bfrag[b], f, 16);
             }
+            // (the hi products of every block first, then the lo products: instructions that accumulate into the same
+            // registers are NB * MW apart)
 #pragma unroll
-            for (int m = 0; m < MW; m++) {
+            for (int m = 0; m < MW; m++)
 #pragma unroll
-                for (int b = 0; b < NB; b++) {
+                for (int b = 0; b < NB; b++)
                     c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[kk & 1][m], bfrag[b], (first && kk == 0) ? zero : c1[b][m], 0, 0, 0);
+#pragma unroll
+            for (int m = 0; m < MW; m++)
+#pragma unroll
+                for (int b = 0; b < NB; b++)
                     c1[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[kk & 1][m], bfrag[b], c1[b][m], 0, 0, 0);
-                }
-            }
         }
     };
     // what has been summed into c1 -> acc.  part: which 128-element run of the super-block (the whole of it with
@@ -1273,6 +1278,27 @@ bool grouped_gemm_supported(const ExpertBanks &b) {
 // that streams its whole weight slab again, so the tile is sized to hold the average expert load
 // plus its spread (binomial: about +-sqrt(avg) per expert, 3.5 sigma here) when that fits; the f16
 // kernel goes up to 128 rows, the int8 kernel (more registers per row) to 64.
+// Tile rows for the f16-unit Q4_K kernels, which come in 32- and 64-row forms: the one with the smaller expected
+// cost when an expert's rows are spread like a binomial around the average (normal approximation, variance =
+// mean).  A 32-row workgroup costs 0.55 of a 64-row one (measured at 4096 tokens, where both forms run full
+// tiles): the expansion of the weights, the loads and the barriers do not shrink with the rows.  At an average
+// of 64 rows half the experts need a second, almost empty 64-row tile and 32-row tiles win; at 48 one 64-row
+// tile holds nearly every expert and wins; from a few hundred rows on the 64-row form wins by its 9 %.
+int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts) {
+    const double avg = (double)n_assign / (double)(n_experts > 0 ? n_experts : 1);
+    const double sigma = __builtin_sqrt(avg > 1.0 ? avg : 1.0);
+    auto expected_tiles = [&](double rows) {
+        double t = 0.0;
+        for (int j = 0; j < 1024; j++) {
+            const double p = 0.5 * erfc(((double)j * rows + 0.5 - avg) / (sigma * 1.4142135623730951));
+            t += p;
+            if (p < 1e-6) break;
+        }
+        return t;
+    };
+    return 0.55 * expected_tiles(32.0) < expected_tiles(64.0) ? 32 : 64;
+}
+
 int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts) {
     const int max_rows = (grouped_gemm_quantized(b) || b.gate_type == T_F32) ? 64 : 128;
     const double avg = (double)n_assign / (double)n_experts;

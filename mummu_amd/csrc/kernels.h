@@ -152,6 +152,7 @@ hipError_t launch_identity_tiles(int n, int tile_rows, int32_t *sorted, int32_t 
 bool grouped_gemm_supported(const ExpertBanks &b);
 bool grouped_gemm_quantized(const ExpertBanks &b);
 int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts);
+int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts);   // (the f16-unit Q4_K kernels: 32 or 64)
 // x [n, d] f32 -> QAct64 (d % 64 == 0).
 hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s);
 // Q4_K banks can take the f16 units instead, against activations held as pairs of halfs (HAct: xh tokens x

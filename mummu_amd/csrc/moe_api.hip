@@ -443,7 +443,6 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
     const int na = (int)(n * k);
     if (n >= batched_from(h, L)) {
         // batched: sort the assignments by expert, then one grouped GEMM per projection
-        const int tile_rows = grouped_gemm_tile_rows(b, na, b.n_experts);
         // the 16-bit activation buffers, viewed in the batched path's 64-element-block layout
         const QAct64 xq64{h->xq.hi, h->xq.lo, h->xq.scale, (float *)h->xq.sum};
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
@@ -452,6 +451,7 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         // (its kernels address the activation planes with 32-bit byte offsets)
         const bool small32 = (size_t)na * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
         const bool hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
+        const int tile_rows = hf_down ? grouped_gemm_tile_rows_q4k_f16(na, b.n_experts) : grouped_gemm_tile_rows(b, na, b.n_experts);
         // (f16 / bf16 banks: x as halfs in the same buffer)
         const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
         const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum}
