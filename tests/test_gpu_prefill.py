@@ -35,6 +35,7 @@ CASES = [
     ("F16", 512, 256, 8, 2, 200),     # 50 per expert -> 96-row tiles
     ("F16", 512, 256, 8, 4, 130),     # 65 per expert -> 96/128-row tiles
     ("F16", 1024, 512, 16, 4, 1027),  # 257 per expert -> several 64-row tiles, 5 dispatch chunks, odd token count
+    ("F16", 256, 256, 128, 8, 1500),  # 12 dispatch chunks over 128 experts: every chunk's workgroup scans the counts itself
     ("BF16", 512, 256, 8, 2, 130),    # bf16 weights become halfs on the way into LDS
     ("BF16", 1024, 512, 16, 4, 515),
     ("F32", 512, 256, 8, 2, 77),      # f32 matrix cores, everything f32: held to 1e-5
