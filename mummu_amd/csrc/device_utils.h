@@ -33,21 +33,24 @@ constexpr int kWave = 64;
 
 // Phase marks for kernel timing studies.  A normal build compiles them away; with
 // -DMUMMU_TRACE every wave stores the constant 100 MHz wall clock at each mark into a caller-provided buffer
-// (16 slots per wave), set per translation unit through mummu_trace_set_<unit>().
+// (16 slots per wave), set per translation unit through mummu_trace_set_<unit>(buffer, waves it holds).
 #ifdef MUMMU_TRACE
 static __device__ long long *g_trace_buf = nullptr;
+static __device__ long long g_trace_waves = 0;  // waves the buffer has room for; a wave past it records nothing
 #ifndef MUMMU_TRACE_MASK
 #define MUMMU_TRACE_MASK 0xFFFF  // which of the 16 marks are compiled in (every mark costs a clock read and a store)
 #endif
+#define MUMMU_TRACE_WAVE ((long long)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6))
 #define MUMMU_PHASE(ph)                                                                                           \
     do {                                                                                                          \
-        if (((MUMMU_TRACE_MASK >> (ph)) & 1) && g_trace_buf && (threadIdx.x & 63) == 0)                           \
-            g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16 + \
-                        (ph)] = wall_clock64();                                                                       \
+        if (((MUMMU_TRACE_MASK >> (ph)) & 1) && g_trace_buf && (threadIdx.x & 63) == 0 &&                         \
+            MUMMU_TRACE_WAVE < g_trace_waves)                                                                     \
+            g_trace_buf[MUMMU_TRACE_WAVE * 16 + (ph)] = wall_clock64();                                           \
     } while (0)
-#define MUMMU_TRACE_UNIT(name)                                                                      \
-    extern "C" __attribute__((visibility("default"))) int mummu_trace_set_##name(void *p) {         \
-        return (int)hipMemcpyToSymbol(HIP_SYMBOL(mummu::g_trace_buf), &p, sizeof(p));                \
+#define MUMMU_TRACE_UNIT(name)                                                                        \
+    extern "C" __attribute__((visibility("default"))) int mummu_trace_set_##name(void *p, long long waves) { \
+        if (hipMemcpyToSymbol(HIP_SYMBOL(mummu::g_trace_waves), &waves, sizeof(waves)) != hipSuccess) return 1; \
+        return (int)hipMemcpyToSymbol(HIP_SYMBOL(mummu::g_trace_buf), &p, sizeof(p));                  \
     }
 // Loop timers: MARK(i) adds the time since the previous mark to slot i; STORE writes the slot sums
 // (slot 6 = first mark's clock, slot 7 = last) to the wave's 8 trace words.
@@ -61,9 +64,8 @@ static __device__ long long *g_trace_buf = nullptr;
 #define MUMMU_TIMER_STORE                                                                                         \
     do {                                                                                                          \
         tm_acc_[7] = tm_last_;                                                                                    \
-        if (g_trace_buf && (threadIdx.x & 63) == 0)                                                               \
-            for (int i_ = 0; i_ < 8; i_++)                                                                        \
-                g_trace_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16 + i_] = tm_acc_[i_]; \
+        if (g_trace_buf && (threadIdx.x & 63) == 0 && MUMMU_TRACE_WAVE < g_trace_waves)                           \
+            for (int i_ = 0; i_ < 8; i_++) g_trace_buf[MUMMU_TRACE_WAVE * 16 + i_] = tm_acc_[i_];                 \
     } while (0)
 #else
 #define MUMMU_PHASE(ph) do { } while (0)

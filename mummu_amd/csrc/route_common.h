@@ -246,13 +246,20 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         // one expert per lane: the rounds run on the bit patterns (a probability is a non-negative finite float, so it
         // orders like its bits; -1 marks a lane that is out of the running), and every lane remembers the slot it won
         // instead of lane 0 writing each round's winner
+        // The renormaliser (the selected probabilities summed in slot order) builds up inside the rounds, where every
+        // lane holds each round's maximum, so the winners write their own slot and nothing goes through LDS.
         int cand = lane < n_experts ? __float_as_int(p[0]) : -1;
         int my_slot = -1;
+        float sum32 = 0.0f;
+        double sum64 = 0.0;
         auto round = [&](int s) {
             const int best = wave_max_i32(cand);
             const int win = (int)__builtin_ctzll(__ballot(cand == best));  // lowest expert id holding the maximum
             my_slot = lane == win ? s : my_slot;
             cand = lane == win ? -1 : cand;
+            const float bf = __int_as_float(best);
+            sum32 = __fadd_rn(sum32, bf);
+            sum64 = __dadd_rn(sum64, (double)bf);
         };
         if (k == 8) {  // the usual top-8 as straight-line code (a taken branch costs as much as half a round)
 #pragma unroll
@@ -260,10 +267,23 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
         } else {
             for (int s = 0; s < k; s++) round(s);
         }
-        if (my_slot >= 0) {
-            sc.w[my_slot] = p[0];
-            sc.id[my_slot] = lane;
+        MUMMU_PHASE(13);
+        float denom = 1.0f;
+        if (flavour == 0) {
+            if (norm) denom = sum32;
+        } else {
+            const float fs = (float)sum64;
+            const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
+            denom = fs > floor_v ? fs : floor_v;
         }
+        if (my_slot >= 0) {
+            float wv = p[0];
+            if (flavour != 0 || norm) wv = __fdiv_rn(wv, denom);
+            ids[orow * k + my_slot] = lane;
+            weights[orow * k + my_slot] = wv;
+            if (hits) atomicAdd(&hits[lane], 1ULL);
+        }
+        return;
     } else if (!ANY_K || k <= 16) {
         // k rounds of "largest remaining probability, lowest id on a tie": the wave maximum,
         // then the first lane (and, within a lane, the first expert) that holds it
