@@ -944,12 +944,16 @@ __global__ __launch_bounds__(256 * WM, GATE_UP ? 2 : 3) void grouped_gemm_q4k_f1
     // during this one's last step
     u32x4 raw[2][NB], rh_next[NB];
     uint32_t dd[NB], sc4[NB][2], mn4[NB][2];
+    // (the header of the NEXT super-block comes with the weights of this one's last step and is unpacked at the end
+    // of that step, a whole step after its load: a value loaded in the loop's last step and first read in the next
+    // iteration is copied between registers at the loop's end, behind a wait for every load in flight)
     auto load_b = [&](int k0, int st, u32x4 (&dst)[NB]) {
         const uint32_t o = b_off + (uint32_t)(k0 >> 8) * 144u;
+        const uint32_t oh = b_off - 16u * (uint32_t)g + (k0 + 256 < in_dim ? (uint32_t)(k0 >> 8) * 144u + 144u : 0u);
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             dst[b] = *(const u32x4 *)(b_base[b] + (o + 16u + (uint32_t)st * 32u));
-            if (st == 0) rh_next[b] = *(const u32x4 *)(b_base[b] + (o - 16u * (uint32_t)g));
+            if (st == 3) rh_next[b] = *(const u32x4 *)(b_base[b] + oh);
         }
     };
     // ggml get_scale_min_k4 for all eight sub-blocks at once
@@ -1110,7 +1114,10 @@ __global__ __launch_bounds__(256 * WM, GATE_UP ? 2 : 3) void grouped_gemm_q4k_f1
         }
     };
 
-    // prologue: step 0 into tile 0
+    // prologue: the first header, step 0 into tile 0
+#pragma unroll
+    for (int b = 0; b < NB; b++) rh_next[b] = *(const u32x4 *)(b_base[b] + (b_off - 16u * (uint32_t)g));
+    unpack_header();
     load_b(0, 0, raw[0]);
     load_a(0, 0);
     store_a(0, 0, 0);
@@ -1127,15 +1134,17 @@ __global__ __launch_bounds__(256 * WM, GATE_UP ? 2 : 3) void grouped_gemm_q4k_f1
         const int sum_buf = ROW ? sb_par : (st >> 1) & 1;
         const int sum_buf_next = ROW ? (st == 3 ? sb_par ^ 1 : sb_par) : (((st + 1) & 3) >> 1) & 1;
         MUMMU_TIMER_MARK(0);
-        if (st == 0) unpack_header();
-        // the next step: weights into the other set of registers, activations into registers
-        load_b(k_next, (st + 1) & 3, raw[(st + 1) & 1]);
+        // the next step: activations into registers, weights into the other set of registers.  (Loads come back in
+        // the order issued: the activations are wanted at the end of this step, the weights a step later, so the
+        // wait before store_a must not have the weight loads in front of it.)
         load_a(k_next, (st + 1) & 3);
+        load_b(k_next, (st + 1) & 3, raw[(st + 1) & 1]);
         MUMMU_CODE_FENCE();  // (the loads stay here, a whole step ahead of their first use)
         MUMMU_TIMER_MARK(1);
         multiply(st, st & 1, raw[st & 1]);
         MUMMU_TIMER_MARK(2);
         if (ROW ? st == 3 : (st & 1) == 1) fold(st >> 1, sum_buf);
+        if (st == 3) unpack_header();
         MUMMU_TIMER_MARK(3);
         MUMMU_CODE_FENCE();
         // ... and into the tile that the step before this one was read from
