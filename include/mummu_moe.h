@@ -209,7 +209,8 @@ MUMMU_API int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, in
  * (per 128 elements between the two products): 22 significant bits per element, every element of a row down to
  * 2^-24 of the row's largest.  That form measures 2e-6 by the reference's measure and has no such corner; it is
  * also the faster one.  The environment variable MUMMU_GEMM_Q4K_F16=0, read by mummu_moe_create, keeps Q4_K on the
- * integer form above. */
+ * integer form above; MUMMU_GEMM_TILE_ROWS=16, 32 or 64 fixes the rows per tile of these kernels (by default the
+ * library picks the form with the smallest expected cost for the batch: same results, different speed). */
 
 /* ---- device-pointer entry points (no host copies, no synchronisation) ------------------
  * stream is a hipStream_t (NULL = the null stream).  Safe to capture into a HIP graph:

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <climits>
 #include <cstdlib>
 #include <cmath>
@@ -92,6 +93,7 @@ struct mummu_moe {
     // the 16-bit float decode kernels lose from 7 tokens on, the f32 ones from 10, the integer ones from 19)
     int gemm_min_f16 = 7, gemm_min_quant = 19, gemm_min_f32 = 10;
     int gemm_q4k_f16 = 1;        // Q4_K banks of the batched path on the f16 units (0: the int8 form)
+    int gemm_tile_rows = 0;          // 0: chosen per batch; else forced (f16-unit Q4_K kernels)
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
     int sh_inter_max = 0;
     int64_t sh_ws_tokens = 0;
@@ -247,7 +249,7 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     HIPCHK(h, hipMalloc(&h->actq.lo, ae));
     HIPCHK(h, hipMalloc(&h->actq.scale, sizeof(float) * (ae / 16)));
     HIPCHK(h, hipMalloc(&h->actq.sum, sizeof(int32_t) * (ae / 16)));
-    h->max_tiles = n_experts + (int)((na + 31) / 32) + 1;
+    h->max_tiles = n_experts + (int)((na + 15) / 16) + 1;   // (the smallest tiles have 16 rows)
     HIPCHK(h, hipMalloc(&h->offsets, sizeof(int32_t) * (size_t)(n_experts + 1)));
     HIPCHK(h, hipMalloc(&h->sorted, sizeof(int32_t) * (size_t)na));
     HIPCHK(h, hipMalloc(&h->inv, sizeof(int32_t) * (size_t)na));
@@ -451,7 +453,10 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         // (its kernels address the activation planes with 32-bit byte offsets)
         const bool small32 = (size_t)na * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
         const bool hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
-        const int tile_rows = hf_down ? grouped_gemm_tile_rows_q4k_f16(na, b.n_experts) : grouped_gemm_tile_rows(b, na, b.n_experts);
+        int tile_rows = hf_down ? grouped_gemm_tile_rows_q4k_f16(na, b.n_experts) : grouped_gemm_tile_rows(b, na, b.n_experts);
+        if (hf_down && h->gemm_tile_rows != 0) tile_rows = h->gemm_tile_rows;
+        // (the launches' grids cover the most tiles this batch can have, not the most the workspace holds)
+        const int tiles_bound = std::min(h->max_tiles, b.n_experts + (na + tile_rows - 1) / tile_rows + 1);
         // (f16 / bf16 banks: x as halfs in the same buffer)
         const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
         const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum}
@@ -464,10 +469,10 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
                launch_dispatch(h->ids, na, b.n_experts, tile_rows, h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->disp_scratch,
                                count_hits ? L.hits : nullptr, h->flags, s));
         LAUNCH(h, K_GEMM_GATE_UP, s,
-               launch_gemm_gate_up(b, x, xq64, xh, h->sorted, k, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->act16, h->act, actq64,
+               launch_gemm_gate_up(b, x, xq64, xh, h->sorted, k, h->tiles, h->n_tiles, tiles_bound, tile_rows, h->act16, h->act, actq64,
                                    acth, s));
         LAUNCH(h, K_GEMM_DOWN, s,
-               launch_gemm_down(b, h->act16, h->act, actq64, acth, na, h->tiles, h->n_tiles, h->max_tiles, tile_rows, h->y, s));
+               launch_gemm_down(b, h->act16, h->act, actq64, acth, na, h->tiles, h->n_tiles, tiles_bound, tile_rows, h->y, s));
         LAUNCH(h, K_COMBINE, s, launch_combine(h->y, h->ids, h->weights, h->inv, (int)n, k, b.hidden, residual, out, s));
         return MUMMU_OK;
     }
@@ -806,6 +811,11 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     // MUMMU_GEMM_Q4K_F16=0: Q4_K banks of the batched path stay on the int8 units (the form every other block-quantized
     // type takes) instead of the f16 units
     if (const char *e = getenv("MUMMU_GEMM_Q4K_F16")) h->gemm_q4k_f16 = atoi(e) != 0;
+    // MUMMU_GEMM_TILE_ROWS=16 | 32 | 64: rows per tile of the f16-unit Q4_K kernels (default: by expected cost)
+    if (const char *e = getenv("MUMMU_GEMM_TILE_ROWS")) {
+        const int v = atoi(e);
+        if (v == 16 || v == 32 || v == 64) h->gemm_tile_rows = v;
+    }
     // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
     if (const char *e = getenv("MUMMU_GEMM_MIN_TOKENS")) {
         const int v = atoi(e);

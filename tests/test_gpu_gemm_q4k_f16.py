@@ -60,6 +60,17 @@ def test_f16_units_match_the_f64_reference_at_f32_accuracy(monkeypatch, H, I, E,
     assert not np.array_equal(got, got8), "the switch did not change the arithmetic: is the f16-unit form running?"
 
 
+@pytest.mark.parametrize("tile_rows", [16, 32, 64])
+@pytest.mark.parametrize("H,I,E,k,n", [(1024, 512, 8, 2, 300), (2048, 1024, 64, 8, 40), (256, 256, 4, 2, 97)])
+def test_every_tile_form_on_the_same_batch(monkeypatch, tile_rows, H, I, E, k, n):
+    # MUMMU_GEMM_TILE_ROWS forces the 16-, 32- or 64-row form, whatever the cost model would pick: full tiles, ragged
+    # last tiles and experts with a row or two (or none) under each of them
+    monkeypatch.setenv("MUMMU_GEMM_TILE_ROWS", str(tile_rows))
+    x = normal((n, H), 70 + n)
+    _, err = run(monkeypatch, True, H, I, E, k, x, seed=60 + n)
+    assert err.max() <= 3e-5, f"{tile_rows}-row tiles: max relative error {err.max():.3e}"
+
+
 @pytest.mark.parametrize("down_type", [M.Q6_K, M.Q8_0])
 def test_q4k_gate_up_feeding_a_down_bank_of_another_type(monkeypatch, down_type):
     # the gate/up launch takes the f16 units and writes the 16-bit byte planes the int8 down product reads
