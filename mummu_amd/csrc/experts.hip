@@ -29,6 +29,8 @@
 #include "gemv_common.h"
 #include "route_common.h"
 
+#include <algorithm>
+#include <cstdint>
 #include <type_traits>
 
 MUMMU_TRACE_UNIT(experts)
@@ -1139,6 +1141,8 @@ hipError_t launch_down_combine(const ExpertBanks &b, QAct actq, const int32_t *i
 // ------------------------------------------------------------------------------------------
 constexpr int kCombineMaxK = 512;
 
+// VEC4: hidden % 4 == 0, a thread takes four neighbouring columns (one 16-byte load per slot).
+template <bool VEC4>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ ids,
                                                       const float *__restrict__ weights,
                                                       const int32_t *__restrict__ inv, int k, int hidden,
@@ -1163,13 +1167,35 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         s_row[s] = inv ? inv[a] : a;
     }
     __syncthreads();
-    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < hidden; c += gridDim.y * blockDim.x) {
-        float sum = 0.0f;
-        for (int r = 0; r < k; r++) {
-            const float v = y[(size_t)s_row[r] * (size_t)hidden + c];
-            sum = __fadd_rn(sum, __fmul_rn(s_w[r], v));
+    if constexpr (VEC4) {
+        for (int c = 4 * (blockIdx.y * blockDim.x + threadIdx.x); c < hidden; c += 4 * gridDim.y * blockDim.x) {
+            float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            for (int r = 0; r < k; r++) {
+                const float4 v = *(const float4 *)(y + (size_t)s_row[r] * (size_t)hidden + c);
+                const float w = s_w[r];
+                sum.x = __fadd_rn(sum.x, __fmul_rn(w, v.x));
+                sum.y = __fadd_rn(sum.y, __fmul_rn(w, v.y));
+                sum.z = __fadd_rn(sum.z, __fmul_rn(w, v.z));
+                sum.w = __fadd_rn(sum.w, __fmul_rn(w, v.w));
+            }
+            if (residual) {
+                const float4 q = *(const float4 *)(residual + (size_t)t * hidden + c);
+                sum.x = __fadd_rn(q.x, sum.x);
+                sum.y = __fadd_rn(q.y, sum.y);
+                sum.z = __fadd_rn(q.z, sum.z);
+                sum.w = __fadd_rn(q.w, sum.w);
+            }
+            *(float4 *)(out + (size_t)t * hidden + c) = sum;
         }
-        out[(size_t)t * hidden + c] = residual ? __fadd_rn(residual[(size_t)t * hidden + c], sum) : sum;
+    } else {
+        for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < hidden; c += gridDim.y * blockDim.x) {
+            float sum = 0.0f;
+            for (int r = 0; r < k; r++) {
+                const float v = y[(size_t)s_row[r] * (size_t)hidden + c];
+                sum = __fadd_rn(sum, __fmul_rn(s_w[r], v));
+            }
+            out[(size_t)t * hidden + c] = residual ? __fadd_rn(residual[(size_t)t * hidden + c], sum) : sum;
+        }
     }
 }
 
@@ -1177,10 +1203,14 @@ hipError_t launch_combine(const float *y, const int32_t *ids, const float *weigh
                           int hidden, const float *residual, float *out, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     if (k > kCombineMaxK) return hipErrorInvalidValue;
-    int ysplit = (hidden + 255) / 256;
-    if (n >= 64) ysplit = 1;  // plenty of workgroups already
+    // a token's row is split over enough workgroups to have about four on every CU
+    const bool vec4 = hidden % 4 == 0 && (((uintptr_t)y | (uintptr_t)out | (uintptr_t)residual) & 15) == 0;
+    const int per_wg = vec4 ? 1024 : 256;   // columns a workgroup covers per pass
+    int ysplit = (1024 + n - 1) / n;
+    ysplit = std::max(1, std::min(ysplit, (hidden + per_wg - 1) / per_wg));
     dim3 block(256), grid(n, ysplit);
-    launch_kernel(combine_kernel, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out);
+    if (vec4) launch_kernel(combine_kernel<true>, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out);
+    else launch_kernel(combine_kernel<false>, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out);
     return hipGetLastError();
 }
 
