@@ -1456,22 +1456,7 @@ __global__ __launch_bounds__(512, 4) void grouped_gemm_q4k_f16_m16_kernel(
 // stores the row 1024 elements at a time.
 __global__ __launch_bounds__(256) void quantize_rows_h_kernel(const float *__restrict__ x, int d, HAct q) {
     __shared__ float s_max[4];
-    const int row = blockIdx.x, tid = threadIdx.x;
-    const float *xr = x + (size_t)row * (size_t)d;
-    float m = 0.0f;
-    for (int e0 = tid * 4; e0 < d; e0 += 1024) {
-        const float4 v = *(const float4 *)(xr + e0);
-        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-    }
-    m = wave_max(m);
-    if ((tid & 63) == 0) s_max[tid >> 6] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
-    for (int e0 = tid * 4; e0 - tid * 4 < d; e0 += 1024) {   // (whole 32-lane groups run together: d is a multiple of 128)
-        const bool active = e0 < d;
-        const float4 v = active ? *(const float4 *)(xr + e0) : make_float4(0.f, 0.f, 0.f, 0.f);
-        hact_store128(v, active, q, (size_t)row, d, e0, m);
-    }
+    hact_quantize_row<256>(x, d, q, (int)blockIdx.x, s_max);
 }
 
 // x [n, d] f32 -> f16, round to nearest.

@@ -36,7 +36,9 @@ hipError_t launch_route_topk(const float *logits, int n, int n_experts, int k, i
 bool router_fused_supported(int n_experts);
 hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, int hidden, int n_experts, int k,
                                int flavour, int norm, float *logits, int32_t *ids, float *weights,
-                               unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s);
+                               unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s, HAct xh = HAct());
+// xh set: the launch also writes x as pairs of halfs (only where router_converts_x holds, and never together with xq)
+bool router_converts_x(int n, int hidden, const float *x, const void *w);
 // x [n, D] f32 -> QAct (D % 16 == 0).
 hipError_t launch_quantize_rows(const float *x, int n, int d, QAct q, hipStream_t s);
 // x * rsqrt(mean(x^2) + eps) * gamma, one wave per token.

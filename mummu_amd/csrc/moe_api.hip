@@ -439,8 +439,26 @@ int batched_from(const mummu_moe *h, const Layer &L) {
     return grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16;
 }
 
+// Q4_K banks on the f16 units (batched path): whether gate/up (hf) and down (hf_down) take that form for this batch,
+// and where x goes as pairs of halfs: the (not yet written) buffer of the down product's output.
+struct HalfPlan {
+    bool hf = false, hf_down = false;
+    HAct xh;
+};
+
+HalfPlan half_plan(const mummu_moe *h, const ExpertBanks &b, int64_t n, int k) {
+    HalfPlan p;
+    const size_t na = (size_t)(n * k);
+    // (its kernels address the activation planes with 32-bit byte offsets)
+    const bool small32 = na * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
+    p.hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b);
+    p.hf_down = p.hf && grouped_gemm_q4k_f16_down(b);
+    if (p.hf) p.xh = HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum};
+    return p;
+}
+
 int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, int64_t n, int k, const float *residual,
-                float *out, hipStream_t s, bool count_hits = false) {
+                float *out, hipStream_t s, bool count_hits = false, bool xh_done = false) {
     ExpertBanks b = banks_of(h, L);
     const int na = (int)(n * k);
     if (n >= batched_from(h, L)) {
@@ -450,19 +468,18 @@ int run_experts(mummu_moe *h, const Layer &L, const float *x, bool x_quantized, 
         const QAct64 actq64{h->actq.hi, h->actq.lo, h->actq.scale, (float *)h->actq.sum};
         // Q4_K banks on the f16 units: x as pairs of halfs in the (not yet written) buffer of the down product's
         // output, the activations between the two products in the f16 and f32 activation buffers
-        // (its kernels address the activation planes with 32-bit byte offsets)
-        const bool small32 = (size_t)na * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
-        const bool hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b), hf_down = hf && grouped_gemm_q4k_f16_down(b);
+        const HalfPlan hp = half_plan(h, b, n, k);
+        const bool hf = hp.hf, hf_down = hp.hf_down;
         int tile_rows = hf_down ? grouped_gemm_tile_rows_q4k_f16(na, b.n_experts) : grouped_gemm_tile_rows(b, na, b.n_experts);
         if (hf_down && h->gemm_tile_rows != 0) tile_rows = h->gemm_tile_rows;
         // (the launches' grids cover the most tiles this batch can have, not the most the workspace holds)
         const int tiles_bound = std::min(h->max_tiles, b.n_experts + (na + tile_rows - 1) / tile_rows + 1);
         // (f16 / bf16 banks: x as halfs in the same buffer)
         const bool half_banks = b.gate_type == T_F16 || b.gate_type == T_BF16;
-        const HAct xh = hf ? HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum}
-                           : (half_banks ? HAct{(_Float16 *)h->y, nullptr, nullptr, nullptr} : HAct());
+        const HAct xh = hf ? hp.xh : (half_banks ? HAct{(_Float16 *)h->y, nullptr, nullptr, nullptr} : HAct());
         const HAct acth = hf_down ? HAct{(_Float16 *)h->act16, (_Float16 *)h->act, h->actq.scale, (float *)h->actq.sum} : HAct();
-        if (hf) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows_h(x, (int)n, b.hidden, xh, s));
+        if (hf && !xh_done) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows_h(x, (int)n, b.hidden, xh, s));
+        else if (hf) {}   // (the router launch wrote them)
         else if (half_banks) LAUNCH(h, K_QUANTIZE, s, launch_convert_rows_f16(x, (int)n, b.hidden, xh.hi, s));
         else if (grouped_gemm_quantized(b)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows64(x, (int)n, b.hidden, xq64, s));
         LAUNCH(h, K_DISPATCH, s,
@@ -576,10 +593,13 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
     if (n > 8 && router_fused_supported(E)) {
         // many tokens: one workgroup per token tile does logits, routing and quantization
         // on the batched path the dispatch adds the per-expert row counts to the hit counters
+        // ... and on the batched path with Q4_K banks on the f16 units it writes x as pairs of halfs beside the routing
+        HAct xh;
+        if (batched && !want_xq && router_converts_x((int)n, H, x, L.router)) xh = half_plan(h, banks_of(h, L), n, k).xh;
         LAUNCH(h, K_ROUTER, s,
                launch_router_fused(x, L.router, L.router_type, (int)n, H, E, k, h->cfg.router_flavour, norm, h->logits,
-                                   h->ids, h->weights, batched ? nullptr : L.hits, h->flags, xq, s));
-        return run_experts(h, L, x, want_xq, n, k, residual, out, s, batched);
+                                   h->ids, h->weights, batched ? nullptr : L.hits, h->flags, xq, s, xh));
+        return run_experts(h, L, x, want_xq, n, k, residual, out, s, batched, xh.hi != nullptr);
     } else {
         if (want_xq) {
             const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, h->xslots, h->xstate};

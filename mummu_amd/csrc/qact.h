@@ -163,4 +163,28 @@ __device__ inline void hact_store128(float4 v, bool active, const HAct &q, size_
     }
 }
 
+// One workgroup of NT threads turns row `row` of x [n, d] into HAct with one scale for the whole row (d % 128 == 0):
+// the row's largest magnitude first, then the row NT * 4 elements at a time.  s_max: NT / 64 floats of LDS.
+template <int NT>
+__device__ inline void hact_quantize_row(const float *__restrict__ x, int d, const HAct &q, int row, float *s_max) {
+    const int tid = threadIdx.x;
+    const float *xr = x + (size_t)row * (size_t)d;
+    float m = 0.0f;
+    for (int e0 = tid * 4; e0 < d; e0 += NT * 4) {
+        const float4 v = *(const float4 *)(xr + e0);
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+    m = wave_max(m);
+    if ((tid & 63) == 0) s_max[tid >> 6] = m;
+    __syncthreads();
+    m = s_max[0];
+#pragma unroll
+    for (int w = 1; w < NT / 64; w++) m = fmaxf(m, s_max[w]);
+    for (int e0 = tid * 4; e0 - tid * 4 < d; e0 += NT * 4) {   // (whole 32-lane groups run together: d is a multiple of 128)
+        const bool active = e0 < d;
+        const float4 v = active ? *(const float4 *)(xr + e0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        hact_store128(v, active, q, (size_t)row, d, e0, m);
+    }
+}
+
 }  // namespace mummu

@@ -362,10 +362,19 @@ template <int WT, int TT, int JN, int CHUNKS, int SPLIT = 1>
 __global__ __launch_bounds__(64 * (SPLIT > 1 ? SPLIT : kStreamWaves)) void router_stream_kernel(
     const float *__restrict__ x, const void *__restrict__ w, int n, int hidden, int n_experts, int k, int flavour,
     int norm, float *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ weights,
-    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags) {
+    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags, HAct xh) {
     static_assert(SPLIT == 1 || TT == 1, "a split token is one token");
     __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[SPLIT > 1 ? 1 : kStreamWaves];
     __shared__ float s_logit[SPLIT > 1 ? 64 * JN : 1];
+    if constexpr (SPLIT > 1) {
+        // workgroups past the tokens (launched when xh is set): each turns one row of x into the pairs of halfs the
+        // f16-unit GEMM reads, beside the routing instead of in a launch of its own
+        if ((int)blockIdx.x >= n) {
+            __shared__ float s_max[SPLIT];
+            hact_quantize_row<64 * SPLIT>(x, hidden, xh, (int)blockIdx.x - n, s_max);
+            return;
+        }
+    }
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int t0 = SPLIT > 1 ? (int)blockIdx.x : (blockIdx.x * kStreamWaves + wave) * TT;
@@ -497,10 +506,20 @@ static hipError_t launch_router_block_t(const float *x, const void *w, int n, in
 
 bool router_fused_supported(int n_experts) { return n_experts <= 128; }
 
+// Which batches the router launch also converts x for: the streaming form with a workgroup per token, while those
+// workgroups leave the chip room (up to 256 tokens the extra workgroups save the 4 us launch of their own: 32 / 128 /
+// 256 tokens 110.6 / 119.5 / 157.0 -> 107.1 / 115.8 / 155.3 us per layer; from 512 on the router launch grows by what
+// the conversion took).
+bool router_converts_x(int n, int hidden, const float *x, const void *w) {
+    const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
+    return n > 8 && n <= 256 && vec && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks;
+}
+
 hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, int hidden, int n_experts, int k,
                                int flavour, int norm, float *logits, int32_t *ids, float *weights,
-                               unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s) {
+                               unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s, HAct xh) {
     if (n <= 0) return hipSuccess;
+    if (xh.hi != nullptr && (xq.hi != nullptr || !router_converts_x(n, hidden, x, w))) return hipErrorInvalidValue;
     if (n_experts > 128 || k > n_experts || k < 1) return hipErrorInvalidValue;
     if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
@@ -511,24 +530,25 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
         // wave per SIMD a token gets a whole workgroup
         const int tt = n > 2048 ? 2 : 1;
         const int split = n <= 512 ? 8 : (n <= 1024 ? 4 : (n <= 2048 ? 2 : 1));
+        const int extra = xh.hi != nullptr ? n : 0;   // (split > 1 wherever router_converts_x holds)
         dim3 block(64 * kStreamWaves), grid((n + tt * kStreamWaves - 1) / (tt * kStreamWaves));
 #define MUMMU_RT3(WT, JN, CH)                                                                                            \
     do {                                                                                                                 \
         if (split == 8)                                                                                                  \
-            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 8>, dim3(n), dim3(512), 0, s, x, w, n, hidden, n_experts, k, flavour, \
-                          norm, logits, ids, weights, hits, flags);                                                      \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 8>, dim3(n + extra), dim3(512), 0, s, x, w, n, hidden, n_experts, k, flavour, \
+                          norm, logits, ids, weights, hits, flags, xh);                                                  \
         else if (split == 4)                                                                                             \
-            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 4>, dim3(n), dim3(256), 0, s, x, w, n, hidden, n_experts, k, flavour, \
-                          norm, logits, ids, weights, hits, flags);                                                      \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 4>, dim3(n + extra), dim3(256), 0, s, x, w, n, hidden, n_experts, k, flavour, \
+                          norm, logits, ids, weights, hits, flags, xh);                                                  \
         else if (split == 2)                                                                                             \
-            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 2>, dim3(n), dim3(128), 0, s, x, w, n, hidden, n_experts, k, flavour, \
-                          norm, logits, ids, weights, hits, flags);                                                      \
+            launch_kernel(router_stream_kernel<WT, 1, JN, CH, 2>, dim3(n + extra), dim3(128), 0, s, x, w, n, hidden, n_experts, k, flavour, \
+                          norm, logits, ids, weights, hits, flags, xh);                                                  \
         else if (tt == 2)                                                                                                \
             launch_kernel(router_stream_kernel<WT, 2, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
-                          logits, ids, weights, hits, flags);                                                            \
+                          logits, ids, weights, hits, flags, HAct());                                                    \
         else                                                                                                             \
             launch_kernel(router_stream_kernel<WT, 1, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
-                          logits, ids, weights, hits, flags);                                                            \
+                          logits, ids, weights, hits, flags, HAct());                                                    \
     } while (0)
 #define MUMMU_RT2(WT, JN)                                                                                                \
     do {                                                                                                                 \
