@@ -79,6 +79,36 @@ WORKLOADS = {
 BANK_TYPES = {"Q4_K": 12, "Q8_0": 8, "F16": 1, "F32": 0, "Q6_K": 14, "Q5_1": 7, "Q5_K": 13, "BF16": 30}
 
 
+def probe_read(M) -> int:
+    """Times the library's read-only stream (mummu_probe_read) over a gate + up bank of the OLMoE Q4_K shape
+    (64 experts x 1024 rows x 1152 bytes, twice: 151 MB), rotating over three such banks so that no launch finds its
+    bytes in the 256 MB Infinity Cache: front to back, and 128 / 64 / 32 bytes of each of a workgroup's 128 rows per
+    step (32 is what a 64-element K step of the grouped GEMM asks of a Q4_K row)."""
+    row_bytes, rows = 1152, 2 * 64 * 1024
+    bank = rows * row_bytes
+    banks, reps = 3, 30
+    buf = M.DeviceBuffer(banks * bank)
+    buf.upload(np.zeros(banks * bank // 8, dtype=np.int64))
+    out = {"metric": "read-only stream over a 151 MB bank (no compute)", "unit": "TB/s", "bytes_per_launch": bank,
+           "row_bytes": row_bytes, "rows_per_workgroup": 128, "launches_timed": reps, "patterns": {}}
+    with M.SparseMoe(M.SparseMoeConfig(64, 64, 2, 1), max_tokens=1) as moe:
+        for piece in (0, 128, 64, 32):
+            for i in range(banks):
+                M.probe_read(buf, bank, row_bytes, piece, moe.stream, offset=i * bank)
+            moe.timer_start()
+            for i in range(reps):
+                M.probe_read(buf, bank, row_bytes, piece, moe.stream, offset=(i % banks) * bank)
+            ms = moe.timer_stop()
+            us = ms * 1e3 / reps
+            out["patterns"]["front_to_back" if piece == 0 else f"{piece}_bytes_per_row_and_step"] = {
+                "us_per_launch": round(us, 2), "tb_per_s": round(bank / (us * 1e-6) / 1e12, 3)}
+    best = max(v["tb_per_s"] for v in out["patterns"].values())
+    out["value"] = best
+    out["of_8_tb_per_s"] = round(best / 8.0, 3)
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -99,6 +129,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--probe-read", action="store_true",
+                    help="instead of the workload: what a read-only kernel streams on this GPU (a ceiling for the roofline's "
+                         "achieved figure), one JSON line")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -111,6 +144,9 @@ def main() -> int:
     if _lib.device_count() < 1:
         print("bench.py: no HIP device", file=sys.stderr)
         return 3
+
+    if args.probe_read:
+        return probe_read(M)
 
     w = WORKLOADS[args.workload]
     H, I, E, k, norm = w["hidden"], w["inter"], w["experts"], w["top_k"], w["norm"]

@@ -430,6 +430,12 @@ MUMMU_API int mummu_timer_stop(mummu_moe *h, float *ms);
  * calibrated against.  No counterpart in the reference. */
 MUMMU_API int mummu_probe_copy(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
 
+/* A read-only stream over `bytes` bytes seen as rows of row_bytes bytes (a multiple of 128): one workgroup per slab
+ * of 128 rows, which it reads piece_bytes (32, 64 or 128) of every row at a time, the way the grouped GEMMs walk
+ * a weight slab, or front to back (piece_bytes = 0).  What is read is dropped: the launch measures what the memory
+ * system delivers to a kernel that does nothing else (bench.py --probe-read).  No counterpart in the reference. */
+MUMMU_API int mummu_probe_read(const void *src_dev, size_t bytes, int row_bytes, int piece_bytes, void *stream);
+
 /* Per-kernel timing: when enabled, every kernel launched by the *_device entry points on
  * the handle's stream is bracketed by HIP events.  mummu_moe_kernel_times() synchronises and
  * returns, per kernel slot, the summed milliseconds and the launch count since the last

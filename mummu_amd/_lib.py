@@ -109,6 +109,7 @@ SIGNATURES = {
     "mummu_timer_start": (_I, [_P]),
     "mummu_timer_stop": (_I, [_P, C.POINTER(C.c_float)]),
     "mummu_probe_copy": (_I, [_P, _P, _SZ, _P]),
+    "mummu_probe_read": (_I, [_P, _SZ, _I, _I, _P]),
     "mummu_gguf_last_error": (C.c_char_p, []),
     "mummu_gguf_open": (_I, [C.c_char_p, C.POINTER(_P)]),
     "mummu_gguf_close": (None, [_P]),

@@ -1614,6 +1614,58 @@ int mummu_probe_copy(void *dst_dev, const void *src_dev, size_t bytes, void *str
     return MUMMU_OK;
 }
 
+extern "C++" {
+namespace {
+typedef unsigned int probe_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kProbeRows = 128;   // rows a workgroup walks in the strided forms: the output slab of the grouped GEMMs
+
+// PIECE bytes of each of the slab's rows per step, one step's loads issued and waited for before the next
+// (PIECE = 0: the slab front to back, 4 KB per step).  What is read goes nowhere.
+template <int PIECE>
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint8_t *__restrict__ src, int row_bytes) {
+    const int tid = threadIdx.x;
+    const uint8_t *slab = src + (size_t)blockIdx.x * kProbeRows * (size_t)row_bytes;
+    probe_u32x4 acc = {0u, 0u, 0u, 0u};
+    if constexpr (PIECE == 0) {
+        const int steps = kProbeRows * row_bytes / 4096;
+        for (int i = 0; i < steps; i++) acc ^= *(const probe_u32x4 *)(slab + (size_t)i * 4096 + tid * 16);
+    } else {
+        constexpr int LPR = PIECE / 16, RPP = 256 / LPR, PASSES = kProbeRows / RPP;
+        const uint8_t *base = slab + (size_t)(tid / LPR) * (size_t)row_bytes + (tid % LPR) * 16;
+        const int steps = row_bytes / PIECE;
+        for (int st = 0; st < steps; st++) {
+            probe_u32x4 r[PASSES];
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) r[p] = *(const probe_u32x4 *)(base + (size_t)p * RPP * (size_t)row_bytes + (size_t)st * PIECE);
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) acc ^= r[p];
+        }
+    }
+    asm volatile("" ::"v"(acc));
+}
+}  // namespace
+}  // extern "C++"
+
+int mummu_probe_read(const void *src_dev, size_t bytes, int row_bytes, int piece_bytes, void *stream) {
+    if (!src_dev || ((uintptr_t)src_dev & 15) || row_bytes < 128 || (row_bytes & 127))
+        return fail(nullptr, MUMMU_ERR_ARG, "probe_read: null or unaligned buffer, or a row that is not a multiple of 128 bytes");
+    const size_t slab = (size_t)kProbeRows * (size_t)row_bytes;
+    const size_t slabs = bytes / slab;
+    if (slabs == 0 || slabs > 0x7fffffffull) return fail(nullptr, MUMMU_ERR_ARG, "probe_read: fewer bytes than one slab of 128 rows");
+    const dim3 grid((unsigned)slabs), block(256);
+    const uint8_t *src = (const uint8_t *)src_dev;
+    switch (piece_bytes) {
+    case 0: launch_kernel(probe_read_kernel<0>, grid, block, 0, (hipStream_t)stream, src, row_bytes); break;
+    case 32: launch_kernel(probe_read_kernel<32>, grid, block, 0, (hipStream_t)stream, src, row_bytes); break;
+    case 64: launch_kernel(probe_read_kernel<64>, grid, block, 0, (hipStream_t)stream, src, row_bytes); break;
+    case 128: launch_kernel(probe_read_kernel<128>, grid, block, 0, (hipStream_t)stream, src, row_bytes); break;
+    default: return fail(nullptr, MUMMU_ERR_ARG, "probe_read: piece_bytes is 0 (front to back), 32, 64 or 128");
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(nullptr, MUMMU_ERR_DEVICE, std::string("probe_read: ") + hipGetErrorString(e));
+    return MUMMU_OK;
+}
+
 int mummu_moe_kernel_timing(mummu_moe *h, int enable) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     h->timing = enable != 0;

@@ -408,6 +408,16 @@ def probe_copy(dst: "DeviceBuffer", src: "DeviceBuffer", nbytes: int, stream=Non
         raise MoeError(rc, lib.mummu_moe_last_error(None).decode())
 
 
+def probe_read(src: "DeviceBuffer", nbytes: int, row_bytes: int, piece_bytes: int, stream=None, offset: int = 0):
+    """Launch the library's read-only stream over nbytes (from byte `offset` of src) seen as rows of row_bytes:
+    piece_bytes of each of a workgroup's 128 rows per step (the grouped GEMMs' walk of a weight slab), or front to
+    back (0)."""
+    lib = _lib.load()
+    rc = lib.mummu_probe_read(C.c_void_p(int(src.ptr) + offset), nbytes, row_bytes, piece_bytes, stream)
+    if rc:
+        raise MoeError(rc, lib.mummu_moe_last_error(None).decode())
+
+
 class PackedWeight:
     """A weight in burn's packed block-32 layout, resident in HBM, behind Q4GemvOps::q4s_gemv
     (nn/packed_gemv.rs:248-260): `words` [K, N*bits/32] u32 (element j of a word at bits j*bits), `scales`
