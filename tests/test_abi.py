@@ -75,6 +75,10 @@ def test_null_arguments_are_errors_not_crashes():
     assert lib.mummu_dequantize(_lib.Q8_0, buf, 33, out) == _lib.ERR_BLOCKS
     assert lib.mummu_dequantize(_lib.Q8_0, buf, 0, out) == _lib.ERR_BLOCKS
     assert lib.mummu_dequantize(15, buf, 33, out) == _lib.ERR_TYPE
+    # the read probe checks its arguments before it launches anything
+    assert lib.mummu_probe_read(None, 1 << 20, 1152, 32, None) == _lib.ERR_ARG
+    assert lib.mummu_probe_read(C.c_void_p(4096), 1 << 20, 100, 32, None) == _lib.ERR_ARG     # a row that is no multiple of 128 bytes
+    assert lib.mummu_probe_read(C.c_void_p(4096), 1000, 1152, 32, None) == _lib.ERR_ARG       # less than one slab of 128 rows
 
 
 def test_missing_library_fails_loudly(monkeypatch):

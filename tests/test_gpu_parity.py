@@ -447,3 +447,17 @@ def test_a_graph_is_refused_once_the_buffers_it_points_into_are_gone():
             g.launch()
         assert e.value.code == _lib.ERR_STALE
         g.close()
+
+
+def test_the_read_probe_runs_every_pattern_and_refuses_the_others():
+    # mummu_probe_read drops what it reads: all there is to check is that every pattern launches and finishes over a
+    # buffer of exactly two slabs, and that a piece size without a kernel is refused
+    row_bytes = 1152
+    buf = M.DeviceBuffer(2 * 128 * row_bytes)
+    buf.upload(np.zeros(2 * 128 * row_bytes // 4, dtype=np.int32))
+    for piece in (0, 32, 64, 128):
+        M.probe_read(buf, 2 * 128 * row_bytes, row_bytes, piece)
+    M.synchronize()
+    with pytest.raises(M.MoeError):
+        M.probe_read(buf, 2 * 128 * row_bytes, row_bytes, 48)
+
