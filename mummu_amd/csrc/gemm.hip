@@ -1319,7 +1319,8 @@ __global__ __launch_bounds__(512, 4) void grouped_gemm_q4k_f16_m16_kernel(
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             // this lane's bytes belong to sub-blocks 4 hs + 2 (kg / 2) (low nibbles) and the one after (high nibbles)
-            const uint32_t sw = sc4[b][hs] >> (16 * (kg >> 1));
+            // (hs is a constant at every call: picked with a conditional, an index would send the array to LDS)
+            const uint32_t sw = (hs ? sc4[b][1] : sc4[b][0]) >> (16 * (kg >> 1));
             const float sc_lo = (float)(sw & 0xFFu), sc_hi = (float)((sw >> 8) & 0xFFu);
             const _Float16 ml = (_Float16)sc_lo, al = (_Float16)__fmul_rn(-1024.0f, sc_lo);
             const _Float16 mh = (_Float16)__fmul_rn(0.0625f, sc_hi), ah = (_Float16)__fmul_rn(-64.0f, sc_hi);
@@ -1372,7 +1373,10 @@ __global__ __launch_bounds__(512, 4) void grouped_gemm_q4k_f16_m16_kernel(
             const float d = half_bits_to_float((uint16_t)(dd[b] & 0xFFFFu));
             const float ndmin = -half_bits_to_float((uint16_t)(dd[b] >> 16));
             // K index 4 kg + i of the fold: sub-block (4 kg + i) % 8 with ROW, else 4 hs + i (its K groups 2, 3 meet zeros)
-            const uint32_t word = ROW ? ((kg & 1) ? mn4[b][1] : mn4[b][0]) : mn4[b][hs];
+            // (with one scale per row the word depends on the lane: blended with a mask - a conditional between the two
+            // array elements becomes an indexed load and sends the array to LDS)
+            const uint32_t lane_mask = 0u - (uint32_t)(kg & 1);
+            const uint32_t word = ROW ? (mn4[b][0] ^ ((mn4[b][0] ^ mn4[b][1]) & lane_mask)) : (hs ? mn4[b][1] : mn4[b][0]);
             half4v bm;
 #pragma unroll
             for (int i = 0; i < 4; i++) bm[i] = (_Float16)(float)((word >> (8 * i)) & 0xFFu);
@@ -1520,8 +1524,11 @@ bool grouped_gemm_supported(const ExpertBanks &b) {
 // full tiles): the expansion of the weights, the loads and the barriers do not shrink with the rows.  At an
 // average of 64 rows half the experts need a second, almost empty 64-row tile and 32-row tiles win; at 48 one
 // 64-row tile holds nearly every expert and wins; from a few hundred rows on the 64-row form wins by its 9 %.
-// A launch of 16-row tiles costs 0.96 of one with as many 32-row tiles (32 tokens over 64 experts: gate/up 57.5
-// against 56.0 us, down 24.9 against 30.0 us), so it is taken while next to no expert has more than 16 rows.
+// A launch of 16-row tiles costs 0.83-0.89 of one with as many 32-row tiles (32 / 64 tokens over 64 experts: gate/up
+// 46.1 / 50.2 against 56.0 / 55.8 us, down 25.1 / 26.7 against 30.0 / 30.8 us), but every expert that needs a second
+// tile streams its weights again: with 10 % more tiles (96 tokens) the 16-row launches already take 65.9 + 33.9 us
+// against 56.5 + 31.8 us.  So the 16-row form is taken only while next to no expert has more than 16 rows (its
+// expected tiles within 4 % of the 32-row form's).
 int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts) {
     const double avg = (double)n_assign / (double)(n_experts > 0 ? n_experts : 1);
     const double sigma = __builtin_sqrt(avg > 1.0 ? avg : 1.0);
