@@ -362,16 +362,23 @@ template <int WT, int TT, int JN, int CHUNKS, int SPLIT = 1>
 __global__ __launch_bounds__(64 * (SPLIT > 1 ? SPLIT : kStreamWaves)) void router_stream_kernel(
     const float *__restrict__ x, const void *__restrict__ w, int n, int hidden, int n_experts, int k, int flavour,
     int norm, float *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ weights,
-    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags, HAct xh) {
+    unsigned long long *__restrict__ hits, int32_t *__restrict__ flags, HAct xh, QAct xq) {
     static_assert(SPLIT == 1 || TT == 1, "a split token is one token");
     __shared__ __attribute__((aligned(16))) RouteScratch<JN> sc[SPLIT > 1 ? 1 : kStreamWaves];
     __shared__ float s_logit[SPLIT > 1 ? 64 * JN : 1];
     if constexpr (SPLIT > 1) {
-        // workgroups past the tokens (launched when xh is set): each turns one row of x into the pairs of halfs the
+        // workgroups past the tokens (launched when xh or xq is set): each turns one row of x into the pairs of halfs the
         // f16-unit GEMM reads, beside the routing instead of in a launch of its own
         if ((int)blockIdx.x >= n) {
             __shared__ float s_max[SPLIT];
-            hact_quantize_row<64 * SPLIT>(x, hidden, xh, (int)blockIdx.x - n, s_max);
+            const int row = (int)blockIdx.x - n;
+            if (xh.hi != nullptr) {
+                hact_quantize_row<64 * SPLIT>(x, hidden, xh, row, s_max);
+            } else {
+                // ... or into the 16-bit blocks of 16 the decode kernels read (hidden % 16 == 0: whole 16-lane rows)
+                for (int e0 = threadIdx.x; e0 < hidden; e0 += 64 * SPLIT)
+                    quantize_store16(x[(size_t)row * (size_t)hidden + e0], true, xq, (size_t)row, hidden, e0);
+            }
             return;
         }
     }
@@ -520,35 +527,38 @@ hipError_t launch_router_fused(const float *x, const void *w, int wtype, int n, 
                                unsigned long long *hits, int32_t *flags, QAct xq, hipStream_t s, HAct xh) {
     if (n <= 0) return hipSuccess;
     if (xh.hi != nullptr && (xq.hi != nullptr || !router_converts_x(n, hidden, x, w))) return hipErrorInvalidValue;
+    // (x quantized for the decode kernels: beside the streaming router as well where it converts x, else inside the
+    // block form below)
+    const bool xq_beside = xq.hi != nullptr && router_converts_x(n, hidden, x, w);
     if (n_experts > 128 || k > n_experts || k < 1) return hipErrorInvalidValue;
     if (xq.hi != nullptr && hidden % 64 != 0) return hipErrorInvalidValue;
     const bool vec = (hidden % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)w & 15) == 0);
     // enough tokens to fill the chip with independent waves: activations in registers, weight
     // rows streamed (on this path the caller quantizes x separately)
-    if (n > 8 && vec && xq.hi == nullptr && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks) {
+    if (n > 8 && vec && (xq.hi == nullptr || xq_beside) && hidden % 512 == 0 && hidden <= 512 * kRouterMaxChunks) {
         // two tokens per wave once there are enough waves to keep every SIMD busy, else one; below a
         // wave per SIMD a token gets a whole workgroup
         const int tt = n > 2048 ? 2 : 1;
         const int split = n <= 512 ? 8 : (n <= 1024 ? 4 : (n <= 2048 ? 2 : 1));
-        const int extra = xh.hi != nullptr ? n : 0;   // (split > 1 wherever router_converts_x holds)
+        const int extra = (xh.hi != nullptr || xq_beside) ? n : 0;   // (split > 1 wherever router_converts_x holds)
         dim3 block(64 * kStreamWaves), grid((n + tt * kStreamWaves - 1) / (tt * kStreamWaves));
 #define MUMMU_RT3(WT, JN, CH)                                                                                            \
     do {                                                                                                                 \
         if (split == 8)                                                                                                  \
             launch_kernel(router_stream_kernel<WT, 1, JN, CH, 8>, dim3(n + extra), dim3(512), 0, s, x, w, n, hidden, n_experts, k, flavour, \
-                          norm, logits, ids, weights, hits, flags, xh);                                                  \
+                          norm, logits, ids, weights, hits, flags, xh, xq);                                                  \
         else if (split == 4)                                                                                             \
             launch_kernel(router_stream_kernel<WT, 1, JN, CH, 4>, dim3(n + extra), dim3(256), 0, s, x, w, n, hidden, n_experts, k, flavour, \
-                          norm, logits, ids, weights, hits, flags, xh);                                                  \
+                          norm, logits, ids, weights, hits, flags, xh, xq);                                                  \
         else if (split == 2)                                                                                             \
             launch_kernel(router_stream_kernel<WT, 1, JN, CH, 2>, dim3(n + extra), dim3(128), 0, s, x, w, n, hidden, n_experts, k, flavour, \
-                          norm, logits, ids, weights, hits, flags, xh);                                                  \
+                          norm, logits, ids, weights, hits, flags, xh, xq);                                                  \
         else if (tt == 2)                                                                                                \
             launch_kernel(router_stream_kernel<WT, 2, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
-                          logits, ids, weights, hits, flags, HAct());                                                    \
+                          logits, ids, weights, hits, flags, HAct(), QAct());                                                    \
         else                                                                                                             \
             launch_kernel(router_stream_kernel<WT, 1, JN, CH>, grid, block, 0, s, x, w, n, hidden, n_experts, k, flavour, norm, \
-                          logits, ids, weights, hits, flags, HAct());                                                    \
+                          logits, ids, weights, hits, flags, HAct(), QAct());                                                    \
     } while (0)
 #define MUMMU_RT2(WT, JN)                                                                                                \
     do {                                                                                                                 \
