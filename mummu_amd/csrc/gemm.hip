@@ -1233,7 +1233,8 @@ __global__ __launch_bounds__(512, 4) void grouped_gemm_q4k_f16_m16_kernel(
     __shared__ __attribute__((aligned(16))) float s_as[2][BM];
     // block sums of one fold.  ROW: the super-block's eight hi halfs, then its eight lo halfs; else the stage's four
     // hi halfs, four lo halfs and eight zeros (the fold is one K = 16 instruction either way)
-    __shared__ __attribute__((aligned(16))) _Float16 s_sum[2][BM][16];
+    // (rows of 20 halfs: with 16 the rows four apart share their banks)
+    __shared__ __attribute__((aligned(16))) _Float16 s_sum[2][BM][20];
 
     int tile, slab;
     if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
@@ -1307,10 +1308,12 @@ __global__ __launch_bounds__(512, 4) void grouped_gemm_q4k_f16_m16_kernel(
     // buf: the tile of the stage; sum_buf / slot: where its block sums go
     auto store_a = [&](int buf, int sum_buf, int slot) {
         *(u32x4 *)(s_raw + (size_t)buf * kBuf + a_lds) = ra;
-        const _Float16 h = (_Float16)rsum;
-        s_sum[sum_buf][m_row][slot + m_blk] = h;
-        s_sum[sum_buf][m_row][slot + (ROW ? 8 : 4) + m_blk] = (_Float16)__fsub_rn(rsum, (float)h);
-        if (!ROW) s_as[sum_buf][m_row] = rscale;
+        if (wave == 0) {   // (every wave holds the same sums: one stores them)
+            const _Float16 h = (_Float16)rsum;
+            s_sum[sum_buf][m_row][slot + m_blk] = h;
+            s_sum[sum_buf][m_row][slot + (ROW ? 8 : 4) + m_blk] = (_Float16)__fsub_rn(rsum, (float)h);
+            if (!ROW) s_as[sum_buf][m_row] = rscale;
+        }
     };
 
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
