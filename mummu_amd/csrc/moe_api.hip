@@ -92,6 +92,7 @@ struct mummu_moe {
     // batches at least this large take dispatch + grouped GEMM (measured crossovers on the OLMoE shape:
     // the 16-bit float decode kernels lose from 7 tokens on, the f32 ones from 10, the integer ones from 19)
     int gemm_min_f16 = 7, gemm_min_quant = 19, gemm_min_f32 = 10;
+    int gemm_min_q4k = 18;   // Q4_K banks on the f16 units (17 tokens: 88.8 us either way; 18: 89.1 against 92.6 us)
     int gemm_q4k_f16 = 1;        // Q4_K banks of the batched path on the f16 units (0: the int8 form)
     int gemm_tile_rows = 0;          // 0: chosen per batch; else forced (f16-unit Q4_K kernels)
     // shared-expert workspace: tokens x widest shared inter, tokens x hidden, tokens
@@ -436,6 +437,7 @@ int batched_from(const mummu_moe *h, const Layer &L) {
     const ExpertBanks b = banks_of(h, L);
     if (!grouped_gemm_supported(b)) return 0x7fffffff;
     if (b.gate_type == T_F32) return h->gemm_min_f32;
+    if (h->gemm_q4k_f16 && grouped_gemm_q4k_f16_down(b)) return h->gemm_min_q4k;
     return grouped_gemm_quantized(b) ? h->gemm_min_quant : h->gemm_min_f16;
 }
 
@@ -839,7 +841,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
     // MUMMU_GEMM_MIN_TOKENS: smallest batch that takes dispatch + grouped GEMM instead of the decode kernels
     if (const char *e = getenv("MUMMU_GEMM_MIN_TOKENS")) {
         const int v = atoi(e);
-        if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = h->gemm_min_f32 = v;
+        if (v >= 1) h->gemm_min_f16 = h->gemm_min_quant = h->gemm_min_f32 = h->gemm_min_q4k = v;
     }
     h->layers.resize((size_t)cfg->num_layers);
     auto bail = [&](int rc) {
