@@ -19,6 +19,9 @@ Prints ONE JSON line (the contract the round driver reads), including
                 measured live with HIP events on the library's stream,
   cpu_baseline  the CPU oracle (a C restatement of the reference's routed CPU path) timed on
                 this host on a bounded sample of the same workload.
+
+Two other modes print a JSON line of their own instead: --probe-read (what a read-only kernel streams on
+this GPU) and --packed-gemv K,N,BITS,ROWS (the packed-GEMV op, microseconds per call).
 """
 from __future__ import annotations
 
@@ -109,6 +112,45 @@ def probe_read(M) -> int:
     return 0
 
 
+def packed_gemv(M, lib, synth, spec: str) -> int:
+    """Times the packed-GEMV op (Q4GemvOps::q4s_gemv, nn/packed_gemv.rs) with device-resident inputs:
+    `--packed-gemv K,N,BITS,ROWS[,REPS]` (5120,17408,4,1 is the Q4S weight the reference quotes).  Several copies of the
+    weight are used in rotation so that no call finds its weight in the 256 MB cache.  Prints one JSON line:
+    wall-clock microseconds per call (two launches: the product and the sum over the K split) and the packed bytes
+    (values + scales) per second."""
+    parts = [int(v) for v in spec.split(",")]
+    if len(parts) not in (4, 5) or parts[2] not in (4, 8):
+        print("bench.py: --packed-gemv takes K,N,BITS,ROWS[,REPS] with BITS 4 or 8", file=sys.stderr)
+        return 2
+    k, n, bits, rows = parts[:4]
+    reps = parts[4] if len(parts) == 5 else 50
+    g = np.random.Generator(np.random.PCG64(1))
+    lim = 1 << (bits - 1)
+    codes = g.integers(-lim, lim, (k, n), dtype=np.int8)
+    scales = g.uniform(0.001, 0.01, (k, n // 32)).astype(np.float32)
+    words = synth.pack_words(codes, bits)
+    copies = max(1, min(8, int(600e6 // (words.nbytes + scales.nbytes))))
+    weights = [M.PackedWeight(words, scales, k, n, bits) for _ in range(copies)]
+    x = g.standard_normal((rows, k)).astype(np.float32)
+    xd, yd = M.DeviceBuffer.from_array(x), M.DeviceBuffer(4 * rows * n)
+    for w in weights:
+        w.gemv_device(xd, rows, yd)
+    lib.mummu_device_synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        for w in weights:
+            w.gemv_device(xd, rows, yd)
+    lib.mummu_device_synchronize()
+    dt = (time.perf_counter() - t0) / (reps * copies)
+    nbytes = weights[0].resident_bytes()
+    print(json.dumps({"op": "q4s_gemv", "k": k, "n": n, "value_bits": bits, "rows": rows,
+                      "us_per_call": round(dt * 1e6, 2), "packed_bytes": nbytes, "gb_per_s": round(nbytes / dt / 1e9, 1),
+                      "weight_copies": copies, "calls": reps * copies}))
+    for w in weights:
+        w.close()
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +174,9 @@ def main() -> int:
     ap.add_argument("--probe-read", action="store_true",
                     help="instead of the workload: what a read-only kernel streams on this GPU (a ceiling for the roofline's "
                          "achieved figure), one JSON line")
+    ap.add_argument("--packed-gemv", default=None, metavar="K,N,BITS,ROWS[,REPS]",
+                    help="instead of the workload: time the packed-GEMV op on a [K, N] weight of 4- or 8-bit values, "
+                         "one JSON line")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -147,6 +192,8 @@ def main() -> int:
 
     if args.probe_read:
         return probe_read(M)
+    if args.packed_gemv:
+        return packed_gemv(M, _lib.load(), synth, args.packed_gemv)
 
     w = WORKLOADS[args.workload]
     H, I, E, k, norm = w["hidden"], w["inter"], w["experts"], w["top_k"], w["norm"]
