@@ -36,6 +36,8 @@ typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int16v __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // staging registers: first-class vectors stay in VGPRs
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
 constexpr int kBN = 128;            // output rows per workgroup
 constexpr int kBK = 64;             // K step
@@ -51,6 +53,32 @@ __device__ inline uint32_t pack_half2(float a, float b) {
 
 __host__ __device__ inline size_t gemm_row_bytes(int type, int in_dim) {
     return (size_t)(in_dim / block_elems(type)) * (size_t)block_bytes(type);
+}
+
+// Two biased halfs 1024 + byte from bytes 0, 1 (or 2, 3) of t.
+__device__ inline half2v biased_pair(uint32_t t, bool upper) {
+    const uint32_t u = __builtin_amdgcn_perm(0x64646464u, t, upper ? 0x04030402u : 0x04010400u);
+    half2v h;
+    __builtin_memcpy(&h, &u, 4);
+    return h;
+}
+
+// Eight Q8_0 codes (two words of int8) times the block scale d as two halfs each, hi = rn(d * code) and
+// lo = d * code - hi (exact: a 19-bit product, subnormal halfs included, which the vector and the matrix units
+// both keep): a code b becomes the half 1024 + (b ^ 0x80) = b + 1152 by a byte permute, minus 1152 is exact.
+__device__ inline void q8_half_planes(uint32_t c0, uint32_t c1, _Float16 d, half8 &hi, half8 &lo) {
+    const half2v d2 = {d, d}, bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const uint32_t u0 = c0 ^ 0x80808080u, u1 = c1 ^ 0x80808080u;
+    const half2v q[4] = {biased_pair(u0, false) - bias, biased_pair(u0, true) - bias, biased_pair(u1, false) - bias,
+                         biased_pair(u1, true) - bias};
+    half2v h[4], l[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        h[j] = q[j] * d2;
+        l[j] = __builtin_elementwise_fma(q[j], d2, -h[j]);
+    }
+    __builtin_memcpy(&hi, h, 16);
+    __builtin_memcpy(&lo, l, 16);
 }
 
 // Epilogue shared by both families: acc register r of lane l is element
@@ -84,33 +112,46 @@ __device__ inline bool xcd_tile(const int32_t *__restrict__ n_tiles, int slabs, 
 // else   : A = act16 (f16, rows already in sorted order), one matrix, y[pos, n] = f32 sum.
 // BF16: the banks hold bf16; every weight becomes a half on its way into LDS (exact from 2^-14 up:
 // a bf16 has 8 significant bits; smaller weights keep an absolute error below 2^-25).
-template <bool GATE_UP, int MT, bool BF16>
+// WT = T_Q8_0: the banks hold Q8_0 blocks (34 bytes: f16 d, 32 int8 codes).  A thread's share of a row and K step is
+// then 8 codes and their block's d; the codes go to LDS as they are, and the wave that owns a column turns its 8
+// codes of an instruction into two operands, hi + lo = d * code exactly, and multiplies both: twice the matrix
+// work of an f16 bank at half the bytes, and the weights lose nothing (x and the activations between the two
+// products are halfs, as for every bank of this kernel).  Needs |d| * 127 inside the half range.
+template <bool GATE_UP, int MT, int WT>
 __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const _Float16 *__restrict__ act_in,
     const int32_t *__restrict__ sorted, int k_slots, const int32_t *__restrict__ tiles, const int32_t *__restrict__ n_tiles,
     int in_dim, int out_dim, _Float16 *__restrict__ act_out, float *__restrict__ y_out) {
     constexpr int NB = GATE_UP ? 2 : 1;
     constexpr int BM = 32 * MT;
+    constexpr bool BF16 = WT == T_BF16, Q8 = WT == T_Q8_0;
+    constexpr int kQRow = kBK + 8;   // a row of codes in LDS (bytes): 72 keeps the 8-byte reads of 32 columns conflict-free
     __shared__ __attribute__((aligned(16))) _Float16 s_a[BM][kLds];
-    __shared__ __attribute__((aligned(16))) _Float16 s_b[NB][kBN][kLds];
+    __shared__ __attribute__((aligned(16))) _Float16 s_b[Q8 ? 1 : NB][Q8 ? 1 : kBN][kLds];
+    __shared__ __attribute__((aligned(16))) uint8_t s_q[Q8 ? NB : 1][Q8 ? kBN : 1][kQRow];   // Q8_0: the step's codes ...
+    __shared__ _Float16 s_d[Q8 ? NB : 1][Q8 ? kBN : 1][2];                                    // ... and the d of its two blocks
 
     int tile, slab;
     if (!xcd_tile(n_tiles, (out_dim + kBN - 1) / kBN, tile, slab)) return;
     const int e = tiles[3 * tile], p0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
     const int n0 = slab * kBN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const size_t row_bytes = (size_t)in_dim * 2;
+    static_assert(WT == T_F16 || WT == T_BF16 || WT == T_Q8_0, "banks this kernel reads");
+    const size_t row_bytes = Q8 ? (size_t)(in_dim / 32) * 34 : (size_t)in_dim * 2;
 
     // weight tile: a K step of one row is 128 contiguous bytes = 8 lanes x 16 B, so one load
     // instruction of a wave covers 8 whole rows; thread -> chunk tid%8 of rows tid/8 + 32*i
+    // (Q8_0: the step is two blocks = 68 bytes; chunk c = codes 8 (c % 4) .. +7 of block c / 4, at byte
+    // 34 (c / 4) + 2 + 8 (c % 4) of the step)
     const int b_chunk = tid & 7;
+    const size_t b_chunk_at = Q8 ? (size_t)(34 * (b_chunk >> 2) + 2 + 8 * (b_chunk & 3)) : (size_t)b_chunk * 16;
     const uint8_t *b_ptr[NB][4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int r = (tid >> 3) + 32 * i;
         const int b_out = n0 + r < out_dim ? n0 + r : out_dim - 1;  // clamped; never stored
-        b_ptr[0][i] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_chunk * 16;
-        if (GATE_UP) b_ptr[NB - 1][i] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + (size_t)b_chunk * 16;
+        b_ptr[0][i] = w0 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + b_chunk_at;
+        if (GATE_UP) b_ptr[NB - 1][i] = w1 + ((size_t)e * (size_t)out_dim + (size_t)b_out) * row_bytes + b_chunk_at;
     }
 
     // activation tile: 8 threads per row, 8 halfs each (MT passes of 32 rows)
@@ -141,7 +182,20 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
 #pragma unroll
         for (int b = 0; b < NB; b++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) rb[b][i] = *(const u32x4 *)(b_ptr[b][i] + (size_t)k0 * 2);
+            for (int i = 0; i < 4; i++) {
+                if constexpr (Q8) {
+                    // 8 codes (2-byte aligned) and the d of their block, 2 + 8 (c % 4) bytes before them
+                    const uint8_t *p = b_ptr[b][i] + (size_t)(k0 >> 5) * 34;
+                    uint32_t c0, c1;
+                    uint16_t db;
+                    __builtin_memcpy(&c0, p, 4);
+                    __builtin_memcpy(&c1, p + 4, 4);
+                    __builtin_memcpy(&db, p - (2 + 8 * (b_chunk & 3)), 2);
+                    rb[b][i] = u32x4{c0, c1, (uint32_t)db, 0u};
+                } else {
+                    rb[b][i] = *(const u32x4 *)(b_ptr[b][i] + (size_t)k0 * 2);
+                }
+            }
 #pragma unroll
         for (int p = 0; p < A_PASSES; p++) ra16[p] = *(const u32x4 *)(a_src16[p] + k0);
     };
@@ -166,6 +220,14 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 u32x4 v = rb[b][i];
+                if constexpr (Q8) {
+                    *(uint2 *)&s_q[b][(tid >> 3) + 32 * i][b_chunk * 8] = make_uint2(v[0], v[1]);
+                    if ((b_chunk & 3) == 0) {
+                        const uint16_t db = (uint16_t)v[2];
+                        __builtin_memcpy(&s_d[b][(tid >> 3) + 32 * i][b_chunk >> 2], &db, 2);
+                    }
+                    continue;
+                }
                 if (BF16) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) v[q] = pack_half2(__uint_as_float(v[q] << 16), __uint_as_float(v[q] & 0xFFFF0000u));
@@ -182,14 +244,26 @@ __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
         // multiply: wave owns columns 32*wave .. +31
 #pragma unroll
         for (int kk = 0; kk < kBK / 16; kk++) {
-            half8 bfrag[NB];
+            half8 bfrag[NB], bfrag_lo[NB];
 #pragma unroll
-            for (int b = 0; b < NB; b++) bfrag[b] = *(const half8 *)&s_b[b][32 * wave + (lane & 31)][kk * 16 + (lane >> 5) * 8];
+            for (int b = 0; b < NB; b++) {
+                if constexpr (Q8) {
+                    const uint2 c = *(const uint2 *)&s_q[b][32 * wave + (lane & 31)][kk * 16 + (lane >> 5) * 8];
+                    q8_half_planes(c.x, c.y, s_d[b][32 * wave + (lane & 31)][kk >> 1], bfrag[b], bfrag_lo[b]);
+                } else {
+                    bfrag[b] = *(const half8 *)&s_b[b][32 * wave + (lane & 31)][kk * 16 + (lane >> 5) * 8];
+                }
+            }
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 const half8 afrag = *(const half8 *)&s_a[32 * m + (lane & 31)][kk * 16 + (lane >> 5) * 8];
 #pragma unroll
                 for (int b = 0; b < NB; b++) acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[b], acc[b][m], 0, 0, 0);
+                if constexpr (Q8) {
+#pragma unroll
+                    for (int b = 0; b < NB; b++)
+                        acc[b][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag_lo[b], acc[b][m], 0, 0, 0);
+                }
             }
         }
         MUMMU_TIMER_MARK(4);
@@ -833,8 +907,6 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_q_kernel(
 // same accumulator.  The offset term is one more instruction per 128 elements: the sums of the four
 // 32-element blocks (hi and lo halfs, K = 8) against the four m.  Per output element and 128 elements
 // of K that leaves three vector operations where the int8 form spends fourteen.
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
 // Only the activation tile goes through LDS.  Wave w owns output columns 32w..32w+31 for every row of the
 // tile, so the weights of those columns are its own: lane (column c, K group g) reads 16 of the 32 quant
@@ -851,14 +923,6 @@ struct HTileLds {
     static constexpr int kC = GATE_UP ? BM * kLdsC * 4 : 0;   // f32 staging of the epilogue (aliases the tiles)
     static constexpr int kBytes = 2 * kBuf > kC ? 2 * kBuf : kC;
 };
-
-// Two biased halfs 1024 + byte from bytes 0, 1 (or 2, 3) of t.
-__device__ inline half2v biased_pair(uint32_t t, bool upper) {
-    const uint32_t u = __builtin_amdgcn_perm(0x64646464u, t, upper ? 0x04030402u : 0x04010400u);
-    half2v h;
-    __builtin_memcpy(&h, &u, 4);
-    return h;
-}
 
 // GATE_UP: A = the token rows of a_in gathered through `sorted`; the epilogue writes silu(g)*u in sorted
 //          order, as HAct (OUT_H: the down banks are Q4_K too) or in the int8 kernels' QAct64.
@@ -1549,8 +1613,8 @@ int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts) {
     return 0.55 * e32 < e64 ? 32 : 64;
 }
 
-int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts) {
-    const int max_rows = (grouped_gemm_quantized(b) || b.gate_type == T_F32) ? 64 : 128;
+int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts, bool q8_half) {
+    const int max_rows = ((grouped_gemm_quantized(b) && !q8_half) || b.gate_type == T_F32) ? 64 : 128;
     const double avg = (double)n_assign / (double)n_experts;
     const int want = (int)(avg + 3.5 * __builtin_sqrt(avg) + 1.0);
     if (want > max_rows) return 64;  // several full tiles per expert whatever the size: 64 rows measured best
@@ -1582,6 +1646,33 @@ static hipError_t launch_gemm_q(const uint8_t *w0, const uint8_t *w1, QAct64 a_i
     else MUMMU_Q(1, 1);
 #undef MUMMU_Q
     return hipGetLastError();
+}
+
+// Largest |d| of a Q8_0 bank as half bits (infinities and NaNs compare above every finite value).
+__global__ __launch_bounds__(256) void q8_scale_max_kernel(const uint8_t *__restrict__ bank, size_t n_blocks, uint32_t *__restrict__ max_bits) {
+    uint32_t m = 0u;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n_blocks; i += (size_t)gridDim.x * 256) {
+        uint16_t db;
+        __builtin_memcpy(&db, bank + i * 34, 2);
+        const uint32_t a = db & 0x7FFFu;
+        m = a > m ? a : m;
+    }
+    m = (uint32_t)wave_max_i32((int)m);
+    if ((threadIdx.x & 63) == 0 && m != 0u) atomicMax(max_bits, m);
+}
+
+hipError_t launch_q8_scale_max(const uint8_t *bank, size_t n_blocks, uint32_t *max_bits, hipStream_t s) {
+    if (n_blocks == 0) return hipSuccess;
+    const size_t want = (n_blocks + 255) / 256;
+    launch_kernel(q8_scale_max_kernel, dim3((unsigned)(want < 2048 ? want : 2048)), dim3(256), 0, s, bank, n_blocks, max_bits);
+    return hipGetLastError();
+}
+
+// Q8_0 banks through the f16 kernel (every weight as two halfs): all three banks Q8_0 and, checked when the layer
+// was loaded, every |d| * 127 inside the half range
+bool grouped_gemm_q8_f16(const ExpertBanks &b) {
+    return b.q8_half_ok && b.gate_type == T_Q8_0 && b.up_type == T_Q8_0 && b.down_type == T_Q8_0 && b.hidden % 64 == 0 &&
+           b.inter % 64 == 0;
 }
 
 bool grouped_gemm_q4k_f16(const ExpertBanks &b) {
@@ -1638,14 +1729,14 @@ static hipError_t launch_gemm_f32(const uint8_t *w0, const uint8_t *w1, const fl
     return hipGetLastError();
 }
 
-template <bool GATE_UP, bool BF16>
+template <bool GATE_UP, int WT>
 static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const _Float16 *act_in,
                                   const int32_t *sorted, int k_slots, const int32_t *tiles, const int32_t *n_tiles,
                                   int max_tiles, int tile_rows, int in_dim, int out_dim, _Float16 *act_out, float *y_out,
                                   hipStream_t s) {
     dim3 block(256), grid((unsigned)((max_tiles + 7) / 8 * 8) * (unsigned)((out_dim + kBN - 1) / kBN));
 #define MUMMU_F16(MT)                                                                                                    \
-    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT, BF16>, grid, block, 0, s, w0, w1, act_in, sorted, k_slots, tiles, n_tiles, \
+    launch_kernel(grouped_gemm_f16_kernel<GATE_UP, MT, WT>, grid, block, 0, s, w0, w1, act_in, sorted, k_slots, tiles, n_tiles, \
                   in_dim, out_dim, act_out, y_out)
     switch (tile_rows) {
     case 32: MUMMU_F16(1); break;
@@ -1660,8 +1751,14 @@ static hipError_t launch_gemm_f16(const uint8_t *w0, const uint8_t *w1, const _F
 
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, HAct xh, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
-                               float *act32, QAct64 actq, HAct acth, hipStream_t s) {
+                               float *act32, QAct64 actq, HAct acth, hipStream_t s, bool q8_half) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (q8_half) {
+        // (x as halfs in xh.hi alone, as for the f16 banks)
+        if (!grouped_gemm_q8_f16(b) || xh.hi == nullptr || xh.lo != nullptr) return hipErrorInvalidValue;
+        return launch_gemm_f16<true, T_Q8_0>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+                                             b.inter, (_Float16 *)act16, nullptr, s);
+    }
     if (xh.hi != nullptr && xh.lo != nullptr) {
         if (!grouped_gemm_q4k_f16(b)) return hipErrorInvalidValue;
         const bool out_h = acth.hi != nullptr;
@@ -1675,10 +1772,10 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
     // (f16 and bf16 banks read x as halfs: xh.hi alone, from launch_convert_rows_f16)
     if ((b.gate_type == T_F16 || b.gate_type == T_BF16) && xh.hi == nullptr) return hipErrorInvalidValue;
     if (b.gate_type == T_F16)
-        return launch_gemm_f16<true, false>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+        return launch_gemm_f16<true, T_F16>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
                                             b.inter, (_Float16 *)act16, nullptr, s);
     if (b.gate_type == T_BF16)
-        return launch_gemm_f16<true, true>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
+        return launch_gemm_f16<true, T_BF16>(b.gate, b.up, xh.hi, sorted, k_slots, tiles, n_tiles, max_tiles, tile_rows, b.hidden,
                                            b.inter, (_Float16 *)act16, nullptr, s);
     switch (b.gate_type) {
 #define MUMMU_GU(T)                                                                                                          \
@@ -1699,8 +1796,14 @@ hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, 
 }
 
 hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, HAct acth, int n_assign,
-                            const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s) {
+                            const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s,
+                            bool q8_half) {
     if (!grouped_gemm_supported(b)) return hipErrorInvalidValue;
+    if (q8_half) {
+        if (!grouped_gemm_q8_f16(b) || acth.hi != nullptr) return hipErrorInvalidValue;
+        return launch_gemm_f16<false, T_Q8_0>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+                                              tile_rows, b.inter, b.hidden, nullptr, y, s);
+    }
     if (acth.hi != nullptr) {
         if (!grouped_gemm_q4k_f16_down(b)) return hipErrorInvalidValue;
         return launch_gemm_q4k_f16<false>(b.down, nullptr, acth, nullptr, 1, tiles, n_tiles, max_tiles, tile_rows, b.inter, b.hidden,
@@ -1711,10 +1814,10 @@ hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float
                                       nullptr, y, s);
     const bool few_rows = n_assign <= 64 * b.n_experts;  // an expert's rows fit one tile, on average
     if (b.down_type == T_F16)
-        return launch_gemm_f16<false, false>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+        return launch_gemm_f16<false, T_F16>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
                                              tile_rows, b.inter, b.hidden, nullptr, y, s);
     if (b.down_type == T_BF16)
-        return launch_gemm_f16<false, true>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
+        return launch_gemm_f16<false, T_BF16>(b.down, nullptr, (const _Float16 *)act16, nullptr, 1, tiles, n_tiles, max_tiles,
                                             tile_rows, b.inter, b.hidden, nullptr, y, s);
     switch (b.down_type) {
 #define MUMMU_DN(T)                                                                                                      \

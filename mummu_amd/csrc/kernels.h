@@ -49,6 +49,7 @@ struct ExpertBanks {
     const uint8_t *gate, *up, *down;  // device, GGUF order
     int gate_type, up_type, down_type;
     int hidden, inter, n_experts;
+    bool q8_half_ok = false;          // Q8_0 banks whose every |d| * 127 is inside the half range (launch_q8_scale_max)
 };
 
 
@@ -153,7 +154,7 @@ hipError_t launch_identity_tiles(int n, int tile_rows, int32_t *sorted, int32_t 
 // A x inter in sorted order; gate/up and down may differ in type).
 bool grouped_gemm_supported(const ExpertBanks &b);
 bool grouped_gemm_quantized(const ExpertBanks &b);
-int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts);
+int grouped_gemm_tile_rows(const ExpertBanks &b, int n_assign, int n_experts, bool q8_half = false);
 int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts);   // (the f16-unit Q4_K kernels: 32 or 64)
 // x [n, d] f32 -> QAct64 (d % 64 == 0).
 hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStream_t s);
@@ -163,14 +164,21 @@ hipError_t launch_quantize_rows64(const float *x, int n, int d, QAct64 q, hipStr
 // down bank of another type the gate/up launch still writes actq.
 bool grouped_gemm_q4k_f16(const ExpertBanks &b);
 bool grouped_gemm_q4k_f16_down(const ExpertBanks &b);
+// Q8_0 banks (gate, up and down) can take the f16 kernel of the f16 banks instead: x as halfs in xh.hi alone, every
+// weight as two halfs made inside the kernel, act16 between the two products.  The launchers take that form with
+// q8_half set (tile rows from grouped_gemm_tile_rows(..., true): up to 128).
+bool grouped_gemm_q8_f16(const ExpertBanks &b);
+// max over a Q8_0 bank's blocks of |d| as half bits, folded into *max_bits (atomic max; start it at 0)
+hipError_t launch_q8_scale_max(const uint8_t *bank, size_t n_blocks, uint32_t *max_bits, hipStream_t s);
 // x [n, d] f32 -> HAct (d % 128 == 0).
 hipError_t launch_quantize_rows_h(const float *x, int n, int d, HAct q, hipStream_t s);
 // x [n, d] f32 -> halfs (d % 4 == 0): what the gate/up launch of f16 and bf16 banks reads (as xh.hi, nothing else set).
 hipError_t launch_convert_rows_f16(const float *x, int n, int d, _Float16 *out, hipStream_t s);
 hipError_t launch_gemm_gate_up(const ExpertBanks &b, const float *x, QAct64 xq, HAct xh, const int32_t *sorted, int k_slots,
                                const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, void *act16,
-                               float *act32, QAct64 actq, HAct acth, hipStream_t s);
+                               float *act32, QAct64 actq, HAct acth, hipStream_t s, bool q8_half = false);
 hipError_t launch_gemm_down(const ExpertBanks &b, const void *act16, const float *act32, QAct64 actq, HAct acth, int n_assign,
-                            const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s);
+                            const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, float *y, hipStream_t s,
+                            bool q8_half = false);
 
 }  // namespace mummu
