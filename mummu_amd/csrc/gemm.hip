@@ -1595,7 +1595,9 @@ bool grouped_gemm_supported(const ExpertBanks &b) {
 // 46.1 / 50.2 against 56.0 / 55.8 us, down 25.1 / 26.7 against 30.0 / 30.8 us), but every expert that needs a second
 // tile streams its weights again: with 10 % more tiles (96 tokens) the 16-row launches already take 65.9 + 33.9 us
 // against 56.5 + 31.8 us.  So the 16-row form is taken only while next to no expert has more than 16 rows (its
-// expected tiles within 4 % of the 32-row form's).
+// expected tiles within 1 % of the 32-row form's: 64 experts x 8 slabs of 16-row tiles are exactly the 512
+// workgroups the chip holds at once, and the first second tiles start a second round - 72 / 80 tokens: 104 / 114 us
+// per layer with 16-row tiles, 105 / 106-112 us with 32-row tiles).
 int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts) {
     const double avg = (double)n_assign / (double)(n_experts > 0 ? n_experts : 1);
     const double sigma = __builtin_sqrt(avg > 1.0 ? avg : 1.0);
@@ -1609,7 +1611,7 @@ int grouped_gemm_tile_rows_q4k_f16(int n_assign, int n_experts) {
         return t;
     };
     const double e16 = expected_tiles(16.0), e32 = expected_tiles(32.0), e64 = expected_tiles(64.0);
-    if (0.96 * e16 < e32 && 0.96 * 0.55 * e16 < e64) return 16;
+    if (0.99 * e16 < e32 && 0.99 * 0.55 * e16 < e64) return 16;
     return 0.55 * e32 < e64 ? 32 : 64;
 }
 
