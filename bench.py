@@ -40,7 +40,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # kernel-timing slot -> name of the kernel in the rocprofv3 summaries
-PROFILE_KERNEL_NAMES = {"gate_up": ("gate_up_fused_kernel", "gate_up_q_kernel"), "down_combine": ("down_combine_q_kernel",)}
+PROFILE_KERNEL_NAMES = {"gate_up": ("gate_up_fused_kernel", "gate_up_q_kernel"), "down_combine": ("down_combine_q_kernel",),
+                        "decode_layer": ("decode_layer_kernel",)}
 
 
 def profiled_traffic(workload, tokens, slot):
@@ -168,6 +169,10 @@ def main() -> int:
     ap.add_argument("--no-steady", action="store_true",
                     help="leave out the event-timed replays behind `steady` (rocprofv3's kernel trace has crashed inside "
                          "hipGraphLaunch between event records; the profile commands pass this)")
+    ap.add_argument("--no-deferred-combine", action="store_true",
+                    help="decode steps that take the one-launch form: enqueue the sum over a token's eight weighted rows as a launch "
+                         "of its own after every step, instead of leaving it to the launch of the next step (see "
+                         "mummu_moe_set_deferred_combine)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--seed", type=int, default=1234)
@@ -228,6 +233,8 @@ def main() -> int:
     t_setup = time.time()
     moe = M.SparseMoe(M.SparseMoeConfig(H, I, E, k), num_layers=L, max_tokens=max(n, 8), norm_topk_prob=norm,
                       router_flavour=w.get("flavour", 0))
+    deferred = not args.no_deferred_combine and not args.stack and not args.shared_inter
+    moe.set_deferred_combine(deferred)
     routers = []
     keep_layer0 = None
     for l in range(L):
@@ -371,7 +378,8 @@ def main() -> int:
     # the dominant kernel and the bytes one launch of it has to move
     # at one token the gate/up launch is the fused one where the device allows it: it also reads the router and the f32 row
     fused = n == 1 and moe.router_exchange_state()[0]
-    kernel_bytes = {"gate_up": mean_distinct * gate_up_expert_bytes + (router_bytes + n * H * 4 if fused else n * E * 4),
+    kernel_bytes = {"decode_layer": mean_distinct * expert_bytes + router_bytes + n * H * 4,
+                    "gate_up": mean_distinct * gate_up_expert_bytes + (router_bytes + n * H * 4 if fused else n * E * 4),
                     "down_combine": mean_distinct * (expert_bytes - gate_up_expert_bytes),
                     "down": mean_distinct * (expert_bytes - gate_up_expert_bytes),
                     "gemm_gate_up": mean_distinct * gate_up_expert_bytes}
@@ -409,7 +417,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
                    "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "shared_inter": args.shared_inter,
-                   "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
+                   "deferred_combine": bool(deferred), "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
                    "graph_replays_timed": (replays + (1 if left else 0)) if graph is not None else 0,
                    "first_timed_step": first,
                    "cache_cold": bool((per_graph - 1) * layer_bytes * layers_per_step > 256e6) if graph is not None else

@@ -249,6 +249,27 @@ MUMMU_API int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const fl
  * the number of workgroups that gave up waiting. */
 MUMMU_API int mummu_moe_set_router_exchange(mummu_moe *h, int enable, unsigned spin_ticks);
 MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbacks);
+/* With top_k = 8, gate / up banks of Q4_K or Q8_0, a down bank of Q4_K, Q8_0 or Q6_K, at most 128 experts and an
+ * intermediate size of at most 1024, the step above runs its experts in ONE launch instead (followed by the small launch
+ * that adds up each token's eight weighted rows): the eight expert slots of a token land on the eight XCDs, and the
+ * workgroups of a slot pass the expert's hidden row to one another through their XCD's L2 the way the router logits
+ * travel, so the down product starts inside the launch that made its input.  No counterpart in the reference.  Same bits
+ * as the other forms; the same spin_ticks bounds its waits, and a workgroup that gives up computes the hidden blocks it
+ * misses itself (counted by _state's fallbacks).  enable = 0 keeps the two-launch form; 1 (default) uses this one
+ * wherever mummu_moe_set_router_exchange's setting allows the fused forms.  Environment: MUMMU_LAYER_FUSION=0. */
+MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
+/* The one-launch form leaves a token's eight weighted rows to be added up.  With enable = 1 (default 0) a
+ * mummu_moe_forward_device call that takes that form no longer enqueues the launch that adds them: the launch of the NEXT
+ * such call on the same stream does it on the side (waves that would otherwise wait for the routing), so a sequence of
+ * decode steps costs one launch per step.  out_dev of a call is then complete once the next call's work, or
+ * mummu_moe_flush, has run on the stream; every other entry point of the handle, mummu_graph_begin / _end / _launch and
+ * mummu_moe_check enqueue a pending sum first, so a captured graph always ends with its last step's sum and a caller
+ * that reads out_dev after mummu_moe_check sees it whole.  A call whose input overlaps the pending output is preceded by
+ * that sum as well.  No counterpart in the reference.  Same bits as mummu_moe_forward_device without it.  Not taken with a
+ * shared expert on the layer or inside mummu_moe_stack_forward*.  Environment: MUMMU_DEFERRED_COMBINE=1. */
+MUMMU_API int mummu_moe_set_deferred_combine(mummu_moe *h, int enable);
+/* Enqueues the sum a deferred step left pending (nothing to do otherwise); does not synchronise. */
+MUMMU_API int mummu_moe_flush(mummu_moe *h);
 /* ExpertExec::run_tensor_resident (nn/moe.rs:360-371, DeviceExpert's at :470-501): the SwiGLU of one expert on rows
  * that are already on this device, the result left there; only enqueues on `stream`.  rows <= max_tokens. */
 MUMMU_API int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_dev, int64_t rows, int hidden,

@@ -19,7 +19,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(HERE, "lib", "libmummu_moe.so")
 
-SOURCES = ["dequant.hip", "router.hip", "experts.hip", "dispatch.hip", "gemm.hip", "moe_api.hip", "packed_gemv.hip", "gguf_reader.cpp", "safetensors_loader.cpp"]
+SOURCES = ["dequant.hip", "router.hip", "experts.hip", "decode_layer.hip", "dispatch.hip", "gemm.hip", "moe_api.hip", "packed_gemv.hip", "gguf_reader.cpp", "safetensors_loader.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]

@@ -28,6 +28,7 @@
 #include "kernels.h"
 #include "gemv_common.h"
 #include "route_common.h"
+#include "decode_parts.h"
 
 #include <algorithm>
 #include <cstdint>
@@ -58,95 +59,6 @@ static hipError_t with_bank_type(int type, F &&f) {
     default: return hipErrorInvalidValue;
     }
 #undef MUMMU_TYPE_CASE
-}
-
-// The gate/up products of one (token, expert) assignment `a` for this workgroup's tile of output rows, given the
-// lane's share `la` of the token's 16-bit activations: NIT iterations of rows_per_it rows per wave, then
-// silu(gate) * up per row, written as f32 (act) or staged in LDS (s_act, rows_per_block floats) and re-quantized to
-// 16-bit blocks for the down product (ACTQ).
-template <int WT, int UPL, int NIT, bool ACTQ>
-__device__ __forceinline__ void gate_up_tile(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, int e, int a,
-                                             const LaneAct<UPL> &la, const RowSplit &rs, int hidden, int inter,
-                                             float *__restrict__ act, const QAct &actq, float *s_act) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
-    const int rows_per_wave = NIT * rs.rows_per_it;
-    const int rows_per_block = rows_per_wave * (blockDim.x >> 6);
-    const int block_row0 = blockIdx.y * rows_per_block;
-    const int row0 = block_row0 + wave * rows_per_wave;
-    const size_t row_bytes = type_row_bytes(WT, hidden);
-    const uint8_t *ge = gate + (size_t)e * (size_t)inter * row_bytes;
-    const uint8_t *ue = up + (size_t)e * (size_t)inter * row_bytes;
-
-    // Software pipeline over the wave's NIT row iterations: the loads of iterations i+1 and i+2
-    // are in flight while iteration i is multiplied, so the integer dots run under the stream
-    // instead of after it (the scheduling barriers keep the compiler from hoisting every load
-    // to the top, where a wave would sit blocked on issue until most of its data had arrived).
-    RawRow<WT, UPL> rg[NIT], ru[NIT];
-    auto fetch = [&](int i) {
-        const int row = row0 + i * rs.rows_per_it + sub;
-        const bool ok = row < inter;
-        load_row<WT, UPL>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
-        load_row<WT, UPL>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
-    };
-    constexpr int AHEAD = NIT < 2 ? NIT : 2;
-#pragma unroll
-    for (int i = 0; i < AHEAD; i++) fetch(i);
-    MUMMU_CODE_FENCE();
-    MUMMU_PHASE(1);
-    float part[2 * NIT];
-#pragma unroll
-    for (int i = 0; i < NIT; i++) {
-        if (i + AHEAD < NIT) fetch(i + AHEAD);
-        MUMMU_CODE_FENCE();
-        part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
-        part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
-        MUMMU_CODE_FENCE();
-    }
-    MUMMU_PHASE(2);
-    dispatch_group(rs.group, [&](auto group_tag) {
-        constexpr int GROUP = decltype(group_tag)::value;
-        constexpr int count = reduced_count<2 * NIT, GROUP>();
-        if constexpr (count < 2) {
-            // whole-wave rows and fewer than four iterations: the shared reduction would leave a
-            // row's gate and up sums in different lanes, so reduce each over the wave instead
-#pragma unroll
-            for (int i = 0; i < NIT; i++) {
-                const float g = wave_sum(part[2 * i]), u = wave_sum(part[2 * i + 1]);
-                const int row = row0 + i * rs.rows_per_it + sub;
-                if (lane == 0 && row < inter) {
-                    const float v = __fmul_rn(det_silu(g), u);
-                    if (ACTQ) s_act[row - block_row0] = v;
-                    else act[(size_t)a * (size_t)inter + row] = v;
-                }
-            }
-            return;
-        }
-        const int offset = reduce_partials<2 * NIT, GROUP>(part, lane);
-        constexpr int width = GROUP < 16 ? GROUP : 16;
-        if ((lane & (width - 1)) == 0) {
-#pragma unroll
-            for (int j = 0; j < count; j += 2) {
-                const int row = row0 + ((offset + j) >> 1) * rs.rows_per_it + sub;
-                if (row < inter) {
-                    const float v = __fmul_rn(det_silu(part[j]), part[j + 1]);
-                    if (ACTQ) s_act[row - block_row0] = v;
-                    else act[(size_t)a * (size_t)inter + row] = v;
-                }
-            }
-        }
-    });
-    MUMMU_PHASE(3);
-    if (ACTQ) {
-        __syncthreads();
-        MUMMU_PHASE(4);
-        for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
-            const int row = block_row0 + r;
-            const bool on = row < inter;  // inter % 16 == 0: a 16-lane row is all on or all off
-            quantize_store16(on ? s_act[r] : 0.0f, on, actq, (size_t)a, inter, on ? row : 0);
-        }
-    }
-    MUMMU_PHASE(5);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -200,119 +112,25 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
     }
-    gate_up_tile<WT, UPL, NIT, ACTQ>(gate, up, e, a, la, rs, hidden, inter, act, actq, s_act);
+    gate_up_tile<WT, UPL, NIT, ACTQ>(gate, up, e, a, la, rs, hidden, inter, act, actq, s_act, blockIdx.y);
 }
 
 // ------------------------------------------------------------------------------------------
 // Decode, first of two launches: router logits, routing and gate/up in ONE kernel.
 //
-// The grid is the gate/up grid (slot, row tile, token).  Workgroups are dealt to the chip's 8 XCDs round-robin
-// by linear id, and the workgroups of one XCD share its L2.  Those of one token on one XCD split the token's E
-// router rows between them (a wave per row, the fixed summation order of router.hip), publish each logit as a
-// 16-byte record in a table of their XCD, and wave 0 of every workgroup collects the E records of its XCD before it
-// routes.  Producer and consumer sit behind the same L2, so a plain store followed by a device-scope load (which
-// bypasses the CU's own L1) sees the record within a fraction of a microsecond, where a round trip through memory
-// between XCDs costs about as much as a kernel launch.  The table is indexed by the XCD the workgroup actually runs
-// on (read from the hardware id register): a workgroup never looks for records on another XCD.
-//
-// A record = {logit bits, epoch low, epoch high, check word}.  The epoch is a 64-bit counter in device memory that the
-// launch after this one increments (down_combine), so records of earlier launches never match and the table needs no
-// clearing.  The wait is bounded (spin_ticks of the 100 MHz clock): a wave that does not find its records - workgroups
-// placed otherwise than assumed, or a tiny spin_ticks from a test - computes the missing logits itself, same bits.
-//
-// Every wave also loads the token's f32 row: with a gamma it is normalised first (RmsNorm, the RmsNorm kernel's bits),
-// wave c quantizes the c-th 512-element chunk to the 16-bit blocks of QAct into LDS, which feed the integer dots.
+// The grid is the gate/up grid (slot, row tile, token).  The prologue (decode_route_prologue: the workgroups of a
+// token that share an XCD split the router's rows, pass the logits to one another through that XCD's L2, route, and
+// leave the token's 16-bit row in LDS) is followed by the workgroup's tile of gate/up rows.  The epoch of the
+// exchange is incremented by the launch after this one (down_combine).
 // hidden <= 2048 and a multiple of 64; (slots * row tiles) a multiple of 8.
 // ------------------------------------------------------------------------------------------
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-__device__ inline u32x4 load_device_scope_b128(const u32x4 *p) {
-    u32x4 r;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p) : "memory");
-    return r;
-}
-
-__device__ inline unsigned xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u; }  // HW_REG_XCC_ID[3:0]
-
-__device__ inline u32x4 exchange_record(float logit, unsigned long long epoch, unsigned what) {
-    u32x4 r;
-    r.x = __float_as_uint(logit);
-    r.y = (unsigned)epoch;
-    r.z = (unsigned)(epoch >> 32);
-    r.w = r.x ^ r.y ^ r.z ^ what ^ 0x5A5A5A5Au;
-    return r;
-}
-
-// 8 consecutive activations of one lane (half a 16-element block; the partner lane holds the other half) -> their hi / lo
-// bytes, the block's scale and integer sum: the arithmetic of quantize16, bit for bit.
-__device__ inline void quantize_half_block(const float (&v)[8], uint2 &hi, uint2 &lo, float &scale, int &sum) {
-    float m = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
-    m = fmaxf(m, dpp_move<0xB1>(m));  // the partner lane
-    const float inv = m > 0.0f ? __fdiv_rn(32512.0f, m) : 0.0f;
-    uint32_t hw[2] = {0u, 0u}, lw[2] = {0u, 0u};
-    sum = 0;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        int xq = (int)__builtin_rintf(__fmul_rn(v[i], inv));
-        xq = xq > 32512 ? 32512 : (xq < -32512 ? -32512 : xq);
-        const int l = ((xq + 128) & 255) - 128;
-        const int h = (xq - l) >> 8;
-        hw[i >> 2] |= (uint32_t)(h & 255) << (8 * (i & 3));
-        lw[i >> 2] |= (uint32_t)(l & 255) << (8 * (i & 3));
-        sum += xq;
-    }
-    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, false);
-    hi = make_uint2(hw[0], hw[1]);
-    lo = make_uint2(lw[0], lw[1]);
-    scale = m > 0.0f ? __fdiv_rn(m, 32512.0f) : 0.0f;
-}
-
-// load_lane_act from the workgroup's LDS copy of one token's 16-bit row (UPL = 1: hidden <= 2048).
-template <int WT>
-__device__ inline void load_lane_act_lds(const int8_t *s_hi, const int8_t *s_lo, const float *s_scale, const int *s_sum, int unit0,
-                                         int units, LaneAct<1> &a) {
-    const bool on = unit0 < units;
-    int e0, e1;
-    unit_halves<WT>(on ? unit0 : 0, e0, e1);
-    const int4 h0 = *(const int4 *)(s_hi + e0), h1 = *(const int4 *)(s_hi + e1);
-    const int4 l0 = *(const int4 *)(s_lo + e0), l1 = *(const int4 *)(s_lo + e1);
-    a.xh[0][0] = h0.x; a.xh[0][1] = h0.y; a.xh[0][2] = h0.z; a.xh[0][3] = h0.w;
-    a.xh[0][4] = h1.x; a.xh[0][5] = h1.y; a.xh[0][6] = h1.z; a.xh[0][7] = h1.w;
-    a.xl[0][0] = l0.x; a.xl[0][1] = l0.y; a.xl[0][2] = l0.z; a.xl[0][3] = l0.w;
-    a.xl[0][4] = l1.x; a.xl[0][5] = l1.y; a.xl[0][6] = l1.z; a.xl[0][7] = l1.w;
-    a.s[0][0] = on ? s_scale[e0 >> 4] : 0.0f;
-    a.s[0][1] = on ? s_scale[e1 >> 4] : 0.0f;
-    a.sx[0][0] = on ? s_sum[e0 >> 4] : 0;
-    a.sx[0][1] = on ? s_sum[e1 >> 4] : 0;
-    a.fsx[0][0] = __fmul_rn(a.s[0][0], (float)a.sx[0][0]);
-    a.fsx[0][1] = __fmul_rn(a.s[0][1], (float)a.sx[0][1]);
-}
-
-template <int RT>
-__device__ __forceinline__ float router_logit_of(const void *__restrict__ w, int e, const WaveRow &x, int hidden, int lane) {
-    WaveRouterRow wr;
-    wave_router_row_load<RT>(w, (size_t)e * (size_t)hidden, hidden, lane, wr);
-    return wave_router_dot(x, wr, hidden, lane);
-}
-
-__device__ __forceinline__ float router_logit_any(const void *__restrict__ w, int wtype, int e, const WaveRow &x, int hidden, int lane) {
-    if (wtype == T_F16) return router_logit_of<T_F16>(w, e, x, hidden, lane);
-    if (wtype == T_BF16) return router_logit_of<T_BF16>(w, e, x, hidden, lane);
-    return router_logit_of<T_F32>(w, e, x, hidden, lane);
-}
-
 template <int WT, int NIT, int RJN>
 __global__ __launch_bounds__(256) void gate_up_fused_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, int k,
                                                             int hidden, int inter, int n_experts, QAct actq,
                                                             int32_t *__restrict__ flags, RouteInline route, RouterExchange rx) {
-    constexpr int JN = RJN;
     extern __shared__ float s_dyn[];  // [rows_per_block] gate/up results, then the token's 16-bit row
-    __shared__ __attribute__((aligned(16))) RouteScratch<JN> s_route;
-    __shared__ int s_ids[64];
-    __shared__ float s_w[64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) DecodeShared<RJN> sh;
+    const int lane = threadIdx.x & 63;
     const int t = blockIdx.z;  // grid = (slot, row tile, token)
     const int a = t * gridDim.x + blockIdx.x;
     const RowSplit rs = row_split(hidden);
@@ -324,175 +142,16 @@ __global__ __launch_bounds__(256) void gate_up_fused_kernel(const uint8_t *__res
     float *s_xscale = (float *)(s_xlo + hidden);
     int *s_xsum = (int *)(s_xscale + hidden / 16);
     MUMMU_PHASE(0);
-
-    // which router rows this workgroup computes: the workgroups of token t on one XCD are those with the same linear id
-    // modulo 8; `mine` counts them in linear order
-    const int per_token = gridDim.x * gridDim.y;             // a multiple of 8
-    const int per_xcd = per_token >> 3;
-    const int mine = (blockIdx.y * gridDim.x + blockIdx.x) >> 3;
-    const int rows_each = (n_experts + per_xcd - 1) / per_xcd;
-    const int row_begin = mine * rows_each;
-    const int row_end = row_begin + rows_each < n_experts ? row_begin + rows_each : n_experts;
-
-    // every load that does not depend on anything goes out first: the epoch, the token's row, this wave's router row.
-    // A wave with a router row (or with a gamma: the sum of squares runs over the whole row) and wave 0 take the whole row,
-    // the others only the 512-element chunk they quantize (chunk = wave: four waves, at most four chunks).
-    const unsigned long long epoch = *rx.epoch;
-    const float *xr = rx.x + (size_t)t * (size_t)hidden;
-    const int my_row = row_begin + wave, my_end = row_end;
-    const bool whole_row = rx.gamma != nullptr || my_row < my_end || wave == 0;  // (wave 0: it may have to compute missing logits)
-    const int qbase = lane * 8 + 512 * wave;
-    const bool qon = qbase < hidden;  // hidden % 64 == 0: the two lanes of a 16-element block are on or off together
-    WaveRow xrow;
-    f32x4 qa, qb;
-    if (whole_row) {
-        wave_row_load(xr, hidden, lane, xrow);
-    } else {
-        qa = ((const f32x4 *)(xr + (qon ? qbase : 0)))[0];
-        qb = ((const f32x4 *)(xr + (qon ? qbase : 0)))[1];
-    }
-    WaveRouterRow wrow;
-    if (my_row < my_end) {
-        const size_t at = (size_t)my_row * (size_t)hidden;
-        if (rx.wtype == T_F16) wave_router_row_load<T_F16>(rx.w, at, hidden, lane, wrow);
-        else if (rx.wtype == T_BF16) wave_router_row_load<T_BF16>(rx.w, at, hidden, lane, wrow);
-        else wave_router_row_load<T_F32>(rx.w, at, hidden, lane, wrow);
-    }
-    if (rx.gamma != nullptr) {
-        const float r = wave_row_rms_scale(xrow, hidden, lane, rx.eps);
-        wave_row_normalise(xrow, r, rx.gamma, hidden, lane);
-        if (rx.xnorm_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
-            float *xo = rx.xnorm_out + (size_t)t * (size_t)hidden;
-#pragma unroll
-            for (int c = 0; c < kWaveRowChunks; c++) {
-                const int base = lane * 8 + 512 * c;
-                if (base >= hidden) continue;
-                ((f32x4 *)(xo + base))[0] = xrow.a[c];
-                ((f32x4 *)(xo + base))[1] = xrow.b[c];
-            }
-        }
-    }
-    u32x4 *table = (u32x4 *)rx.slots + ((size_t)xcc_id() * kExchangeTokens + (size_t)t) * (size_t)n_experts;
-    // this wave's router row (more rows than waves: the remaining ones in further rounds, each with its own loads)
-    if (my_row < my_end) {
-        const float logit = wave_router_dot(xrow, wrow, hidden, lane);
-        if (lane == 0) table[my_row] = exchange_record(logit, epoch, (unsigned)(t * n_experts + my_row));
-    }
-    for (int row = row_begin + wave + (blockDim.x >> 6); row < row_end; row += blockDim.x >> 6) {
-        const float logit = router_logit_any(rx.w, rx.wtype, row, xrow, hidden, lane);
-        if (lane == 0) table[row] = exchange_record(logit, epoch, (unsigned)(t * n_experts + row));
-    }
-    MUMMU_PHASE(8);
-    // this wave's chunk of the row into LDS as 16-bit blocks (lane pairs hold the 16-element blocks)
-    if (whole_row) {
-        qa = xrow.a[0];
-        qb = xrow.b[0];
-#pragma unroll
-        for (int cc = 1; cc < kWaveRowChunks; cc++) {
-            qa = wave == cc ? xrow.a[cc] : qa;
-            qb = wave == cc ? xrow.b[cc] : qb;
-        }
-    }
-    if (512 * wave < hidden) {
-        const float v[8] = {qon ? qa.x : 0.0f, qon ? qa.y : 0.0f, qon ? qa.z : 0.0f, qon ? qa.w : 0.0f,
-                            qon ? qb.x : 0.0f, qon ? qb.y : 0.0f, qon ? qb.z : 0.0f, qon ? qb.w : 0.0f};
-        uint2 hi, lo;
-        float scale;
-        int sum;
-        quantize_half_block(v, hi, lo, scale, sum);
-        if (qon) {
-            *(uint2 *)(s_xhi + qbase) = hi;
-            *(uint2 *)(s_xlo + qbase) = lo;
-            if ((lane & 1) == 0) {
-                s_xscale[qbase >> 4] = scale;
-                s_xsum[qbase >> 4] = sum;
-            }
-            if (rx.xq_out.hi != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
-                // one workgroup per token also leaves the row in global memory (the shared expert's launches read it)
-                *(uint2 *)(rx.xq_out.hi + (size_t)t * (size_t)hidden + qbase) = hi;
-                *(uint2 *)(rx.xq_out.lo + (size_t)t * (size_t)hidden + qbase) = lo;
-                if ((lane & 1) == 0) {
-                    rx.xq_out.scale[(size_t)t * (size_t)(hidden / 16) + (qbase >> 4)] = scale;
-                    rx.xq_out.sum[(size_t)t * (size_t)(hidden / 16) + (qbase >> 4)] = sum;
-                }
-            }
-        }
-    }
-    MUMMU_PHASE(9);
-    if (wave == 0) {
-        // collect the E logits of token t from this XCD's table
-        float l[JN];
-        bool have[JN];
-#pragma unroll
-        for (int j = 0; j < JN; j++) {
-            l[j] = 0.0f;
-            have[j] = lane + 64 * j >= n_experts;
-        }
-        const unsigned long long t_begin = wall_clock64();
-        bool complete = false;
-        while (rx.spin_ticks != 0u) {  // (a bound of 0: do not look at the table at all)
-            bool all = true;
-#pragma unroll
-            for (int j = 0; j < JN; j++) {
-                if (have[j]) continue;
-                const int e = lane + 64 * j;
-                const u32x4 r = load_device_scope_b128(table + e);
-                const u32x4 want = exchange_record(__uint_as_float(r.x), epoch, (unsigned)(t * n_experts + e));
-                if (r.y == want.y && r.z == want.z && r.w == want.w) {
-                    l[j] = __uint_as_float(r.x);
-                    have[j] = true;
-                } else {
-                    all = false;
-                }
-            }
-            if (__all(all)) {
-                complete = true;
-                break;
-            }
-            if (wall_clock64() - t_begin >= (unsigned long long)rx.spin_ticks) break;
-            __builtin_amdgcn_s_sleep(1);
-        }
-        MUMMU_PHASE(10);
-        if (!complete) {
-            // records that never came: compute those logits here (the same function of the same row: the same bits)
-            if (lane == 0 && rx.fallbacks != nullptr) atomicAdd(rx.fallbacks, 1ULL);
-#pragma unroll
-            for (int j = 0; j < JN; j++) {
-                unsigned long long missing = __ballot(!have[j]);
-                while (missing != 0ull) {
-                    const int src = (int)__builtin_ctzll(missing);
-                    missing &= missing - 1ull;
-                    const float v = router_logit_any(rx.w, rx.wtype, src + 64 * j, xrow, hidden, lane);
-                    if (lane == src) l[j] = v;
-                }
-            }
-        }
-        if (rx.logits_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
-#pragma unroll
-            for (int j = 0; j < JN; j++)
-                if (lane + 64 * j < n_experts) rx.logits_out[(size_t)t * n_experts + lane + 64 * j] = l[j];
-        }
-        route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
-        wave_lds_sync();
-        if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
-            const int id = s_ids[lane];
-            route.ids[(size_t)t * k + lane] = id;
-            route.weights[(size_t)t * k + lane] = s_w[lane];
-            if (route.hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&route.hits[id], 1ULL);
-        }
-        MUMMU_PHASE(11);
-    }
-    __syncthreads();
-    MUMMU_PHASE(7);
+    decode_route_prologue<RJN>(k, hidden, n_experts, flags, route, rx, sh, s_xhi, s_xlo, s_xscale, s_xsum);
     LaneAct<1> la;
     load_lane_act_lds<WT>(s_xhi, s_xlo, s_xscale, s_xsum, unit0, rs.units, la);
     MUMMU_PHASE(14);
-    const int e = s_ids[blockIdx.x];
+    const int e = sh.ids[blockIdx.x];
     if ((unsigned)e >= (unsigned)n_experts) {
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
     }
-    gate_up_tile<WT, 1, NIT, true>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act);
+    gate_up_tile<WT, 1, NIT, true>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act, blockIdx.y);
 }
 
 // gate/up, float banks.  RJN > 0: the kernel routes by itself (see RouteInline), RJN experts per lane
@@ -1146,7 +805,10 @@ template <bool VEC4>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ ids,
                                                       const float *__restrict__ weights,
                                                       const int32_t *__restrict__ inv, int k, int hidden,
-                                                      const float *__restrict__ residual, float *__restrict__ out) {
+                                                      const float *__restrict__ residual, float *__restrict__ out,
+                                                      unsigned long long *epoch_bump) {
+    // the launch before this one (decode_layer_kernel) has finished with the epoch: move it on for the next
+    if (epoch_bump != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *epoch_bump = *epoch_bump + 1ULL;
     __shared__ int s_order[kCombineMaxK];
     __shared__ int s_row[kCombineMaxK];
     __shared__ float s_w[kCombineMaxK];
@@ -1200,7 +862,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 }
 
 hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, const int32_t *inv, int n, int k,
-                          int hidden, const float *residual, float *out, hipStream_t s) {
+                          int hidden, const float *residual, float *out, hipStream_t s, unsigned long long *epoch_bump) {
     if (n <= 0) return hipSuccess;
     if (k > kCombineMaxK) return hipErrorInvalidValue;
     // a token's row is split over enough workgroups to have about four on every CU
@@ -1209,8 +871,8 @@ hipError_t launch_combine(const float *y, const int32_t *ids, const float *weigh
     int ysplit = (1024 + n - 1) / n;
     ysplit = std::max(1, std::min(ysplit, (hidden + per_wg - 1) / per_wg));
     dim3 block(256), grid(n, ysplit);
-    if (vec4) launch_kernel(combine_kernel<true>, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out);
-    else launch_kernel(combine_kernel<false>, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out);
+    if (vec4) launch_kernel(combine_kernel<true>, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out, epoch_bump);
+    else launch_kernel(combine_kernel<false>, grid, block, 0, s, y, ids, weights, inv, k, hidden, residual, out, epoch_bump);
     return hipGetLastError();
 }
 

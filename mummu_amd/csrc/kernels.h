@@ -92,12 +92,37 @@ struct RouterExchange {
     float *logits_out = nullptr;                // nullable [n, E]
     QAct xq_out;                                // nullable (hi == nullptr): the token rows as 16-bit blocks, for a later launch
     unsigned spin_ticks = 5000;                 // bound of the wait for the other workgroups' records, 10 ns units
+    unsigned salt = 0;                          // tells launches apart that read the same epoch (a host-side launch counter)
     unsigned long long *fallbacks = nullptr;    // nullable: += 1 per workgroup that gave up waiting and computed the logits itself
 };
 inline size_t router_exchange_bytes(int n_experts) { return (size_t)kExchangeXcds * kExchangeTokens * (size_t)n_experts * 16; }
 bool gate_up_fused_supported(const ExpertBanks &b, int k, int n_tokens, const RouterExchange &rx);
 hipError_t launch_gate_up_fused(const ExpertBanks &b, const RouterExchange &rx, const RouteInline &route, int n_tokens, int k,
                                 QAct actq, int32_t *flags, hipStream_t s);
+// The whole expert side of a decode step in ONE launch (top_k = 8, gate/up Q4_K or Q8_0, down Q4_K / Q8_0 / Q6_K,
+// inter <= 1024): the prologue of launch_gate_up_fused, gate/up, and the down product of every slot, whose hidden
+// row passes between the workgroups of the XCD that owns the slot through a table in that XCD's L2 (see
+// decode_layer_kernel).  Leaves y [n * k, hidden], the per-slot down sums launch_combine adds up.
+constexpr int kActBlocksMax = 64;  // 16-element blocks of a hidden row the table holds (inter <= 1024)
+struct LayerExchange {
+    void *act_slots = nullptr;               // layer_exchange_bytes() bytes, 256-byte aligned
+    float *y = nullptr;                      // [n * k, hidden] out
+    unsigned long long *fallbacks = nullptr; // nullable: += 1 per workgroup that computed blocks of other workgroups itself
+};
+// A weighted sum over the eight slots of an earlier launch's tokens that this launch performs on the side (waves that
+// would otherwise wait for the routing): out = (residual +) the sum in ascending expert id, as launch_combine.
+struct PendingSum {
+    const float *y = nullptr;         // [n * 8, hidden]
+    const int32_t *ids = nullptr;     // [n, 8]
+    const float *weights = nullptr;   // [n, 8]
+    const float *residual = nullptr;  // nullable [n, hidden]
+    float *out = nullptr;             // [n, hidden]
+    int n = 0;                        // 0: nothing pending
+};
+inline size_t layer_exchange_bytes() { return (size_t)kExchangeXcds * kExchangeTokens * 8 * (size_t)kActBlocksMax * 64; }
+bool decode_layer_supported(const ExpertBanks &b, int k, int n_tokens, const RouterExchange &rx, const LayerExchange &lx);
+hipError_t launch_decode_layer(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
+                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &pending = PendingSum());
 // The same pair for float banks (F32 / F16 / BF16 gate/up and down, at most 512 experts, top_k <= 16):
 // gate/up with the routing inside writes act [n*k, inter] f32, then down + combine in one launch.
 bool float_decode_fused(const ExpertBanks &b, int k);
@@ -111,8 +136,9 @@ hipError_t launch_down(const ExpertBanks &b, const float *act, QAct actq, const 
 // out[t, c] = sum over the token's k slots in ASCENDING EXPERT ID of (w * y), two roundings.
 // residual (nullable): out = residual + that sum.
 // inv (nullable): y row of assignment a is inv[a] instead of a (dispatch-sorted layout).
+// epoch_bump (nullable): the 64-bit counter of the router exchange, incremented once by this launch.
 hipError_t launch_combine(const float *y, const int32_t *ids, const float *weights, const int32_t *inv, int n, int k,
-                          int hidden, const float *residual, float *out, hipStream_t s);
+                          int hidden, const float *residual, float *out, hipStream_t s, unsigned long long *epoch_bump = nullptr);
 // down + combine in one launch (no y round trip): quantized down bank and top_k <= 16.
 bool down_combine_supported(const ExpertBanks &b, int k);
 // epoch_bump (nullable): the 64-bit counter of the router exchange, incremented once by this launch.

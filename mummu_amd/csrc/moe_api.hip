@@ -24,9 +24,10 @@ namespace {
 thread_local std::string g_error;  // failures of calls that have no handle
 
 enum KernelSlot { K_ROUTER, K_ROUTER_LOGITS, K_ROUTE_TOPK, K_QUANTIZE, K_GATE_UP, K_DOWN_COMBINE, K_DOWN, K_COMBINE, K_RMSNORM,
-                  K_DISPATCH, K_GEMM_GATE_UP, K_GEMM_DOWN, K_SHARED, K_SLOTS };
+                  K_DISPATCH, K_GEMM_GATE_UP, K_GEMM_DOWN, K_SHARED, K_DECODE_LAYER, K_SLOTS };
 const char *const kSlotNames[K_SLOTS] = {"router", "router_logits", "route_topk", "quantize", "gate_up", "down_combine",
-                                         "down", "combine", "rmsnorm", "dispatch", "gemm_gate_up", "gemm_down", "shared_expert"};
+                                         "down", "combine", "rmsnorm", "dispatch", "gemm_gate_up", "gemm_down", "shared_expert",
+                                         "decode_layer"};
 
 struct Layer {
     void *router = nullptr;
@@ -114,6 +115,28 @@ struct mummu_moe {
     bool xcd_round_robin = false;
     int router_exchange = 1;
     unsigned spin_ticks = 5000;
+    // the one-launch decode form (decode_layer_kernel): the table its workgroups pass the experts' hidden rows through,
+    // and a counter that tells launches apart which read the same epoch (the nodes of one captured graph)
+    void *aslots = nullptr;
+    int layer_fusion = 1;
+    unsigned launch_salt = 0;
+    // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
+    // off by default), whose otherwise idle waves do it: the one-launch form then costs one launch per step.  The per-slot
+    // rows and the routing of consecutive steps alternate between two sets of buffers ([0] = y, ids, weights above);
+    // `pending` is the step whose sum has not been enqueued yet.
+    int deferred_combine = 0;
+    float *y_alt = nullptr, *weights_alt = nullptr;
+    int32_t *ids_alt = nullptr;
+    int decode_buf = 0;    // the set the next deferred step writes
+    int routing_buf = 0;   // the set that holds the last call's routing
+    struct {
+        bool active = false;
+        int buf = 0, k = 0;
+        int64_t n = 0;
+        const float *residual = nullptr;
+        float *out = nullptr;
+        hipStream_t stream = nullptr;
+    } pending;
     // bumped whenever a device buffer a captured graph may point into is freed (workspace regrown, a layer's or
     // a shared expert's weights replaced); a graph remembers the value it was captured under
     uint64_t generation = 0;
@@ -138,6 +161,16 @@ int fail(mummu_moe *h, int code, const std::string &msg) {
         if (e_ != hipSuccess)                                                                              \
             return fail(h, MUMMU_ERR_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_));            \
     } while (0)
+
+int flush_pending(mummu_moe *h);
+
+// Takes the handle's lock and, first of all, enqueues the weighted sum a deferred decode step may have left pending
+// (see mummu_moe_set_deferred_combine): every entry point but the one that continues such a chain starts with this.
+struct Entry {
+    std::lock_guard<std::mutex> lock;
+    int rc;
+    explicit Entry(mummu_moe *h) : lock(h->mu), rc(flush_pending(h)) {}
+};
 
 // The device address of `scratch` on the current device, looked up once per device.
 constexpr int kMaxDevices = 64;
@@ -167,11 +200,14 @@ void free_ws(mummu_moe *h) {
     h->generation++;
     void *ptrs[] = {h->logits, h->weights, h->act, h->y, h->ids, h->xin, h->xout, h->h2, h->resid[0], h->resid[1],
                     h->xq.hi, h->xq.lo, h->xq.scale, h->xq.sum, h->actq.hi, h->actq.lo, h->actq.scale, h->actq.sum,
-                    h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->act16, h->disp_scratch};
+                    h->offsets, h->sorted, h->inv, h->tiles, h->n_tiles, h->act16, h->disp_scratch, h->y_alt, h->weights_alt, h->ids_alt};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     h->logits = h->weights = h->act = h->y = h->xin = h->xout = h->h2 = h->resid[0] = h->resid[1] = nullptr;
     h->ids = nullptr;
+    h->y_alt = h->weights_alt = nullptr;
+    h->ids_alt = nullptr;
+    h->decode_buf = h->routing_buf = 0;
     h->xq = QAct();
     h->actq = QAct();
     h->offsets = h->sorted = h->inv = h->tiles = h->n_tiles = h->disp_scratch = nullptr;
@@ -225,6 +261,10 @@ int ensure_shared_ws(mummu_moe *h) {
 int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     if (n_experts < h->cfg.num_experts) n_experts = h->cfg.num_experts;
     if (n <= h->ws_tokens && n_assign <= h->ws_assign && n_experts <= h->ws_experts) return MUMMU_OK;
+    {
+        const int rc = flush_pending(h);
+        if (rc) return rc;
+    }
     HIPCHK(h, hipDeviceSynchronize());
     int64_t nt = n > h->ws_tokens ? n : h->ws_tokens;
     int64_t na = n_assign > h->ws_assign ? n_assign : h->ws_assign;
@@ -260,6 +300,13 @@ int ensure_ws(mummu_moe *h, int64_t n, int64_t n_assign, int n_experts) {
     HIPCHK(h, hipMalloc(&h->n_tiles, sizeof(int32_t)));
     HIPCHK(h, hipMalloc(&h->disp_scratch, sizeof(int32_t) * dispatch_scratch_ints((int)na, n_experts)));
     HIPCHK(h, hipMalloc(&h->act16, 2 * (size_t)na * I));
+    {
+        // the second set of the deferred sums' buffers: decode steps only (at most kExchangeTokens tokens)
+        const size_t na8 = (size_t)std::min<int64_t>(na, (int64_t)kExchangeTokens * 8);
+        HIPCHK(h, hipMalloc(&h->y_alt, sizeof(float) * na8 * H));
+        HIPCHK(h, hipMalloc(&h->ids_alt, sizeof(int32_t) * na8));
+        HIPCHK(h, hipMalloc(&h->weights_alt, sizeof(float) * na8));
+    }
     h->ws_tokens = nt;
     h->ws_assign = na;
     h->ws_experts = n_experts;
@@ -531,6 +578,8 @@ struct DecodeScratch {
     QAct xq, actq;    // [n, H] and [n*k, I rounded up to 16]
     void *xslots = nullptr;                  // router exchange table (router_exchange_bytes(E)), or null: three launches
     unsigned long long *xstate = nullptr;    // [0] its epoch, [1] its fallback counter
+    void *aslots = nullptr;                  // hidden-row exchange table (layer_exchange_bytes()), or null: no one-launch form
+    float *y = nullptr;                      // [n*k, H]: per-slot down sums of the one-launch form
 };
 
 // The two launches after the router's: gate/up with the routing inside, then down + combine.
@@ -549,17 +598,32 @@ int decode_tail(mummu_moe *h, const Layer &L, const DecodeScratch &ws, int n, in
     return MUMMU_OK;
 }
 
-// The decode step in two launches where the device and the shapes allow it: router + routing + gate/up in one kernel
-// (the workgroups exchange the logits inside it), then down + combine.  *done = false: not taken, nothing launched.
-int decode_two_launches(mummu_moe *h, const Layer &L, const DecodeScratch &ws, const float *x, int n, int k, int norm,
-                        const float *residual, float *out, hipStream_t s, const float *norm_gamma, float *xnorm_out, bool *done) {
-    *done = false;
-    if (!h->router_exchange || !h->xcd_round_robin || ws.xslots == nullptr || ws.xstate == nullptr) return MUMMU_OK;
-    // measured on the OLMoE shape (Q4_K): one token 18.1 us against 18.4 in three launches, but 23.6 / 40.2 / 69.5 us
-    // against 22.8 / 36.6 / 57.2 at 2 / 4 / 8 tokens - every workgroup repeats the router wait, and the fused kernel
-    // keeps fewer waves per CU.  So one token only, unless a caller asks for it at every size (tests do).
-    if (n > 1 && h->router_exchange < 2) return MUMMU_OK;
-    const ExpertBanks b = banks_of(h, L);
+// The two sets of buffers consecutive deferred steps alternate between.
+struct DecodeBuffers {
+    float *y;
+    int32_t *ids;
+    float *weights;
+};
+
+DecodeBuffers decode_buffers(const mummu_moe *h, int buf) {
+    return buf == 0 ? DecodeBuffers{h->y, h->ids, h->weights} : DecodeBuffers{h->y_alt, h->ids_alt, h->weights_alt};
+}
+
+// Enqueues the weighted sum a deferred step left pending (on the stream that step ran on) and moves the exchange's epoch on.
+int flush_pending(mummu_moe *h) {
+    if (!h->pending.active) return MUMMU_OK;
+    h->pending.active = false;
+    const DecodeBuffers pb = decode_buffers(h, h->pending.buf);
+    hipStream_t s = h->pending.stream;
+    LAUNCH(h, K_COMBINE, s,
+           launch_combine(pb.y, pb.ids, pb.weights, nullptr, (int)h->pending.n, h->pending.k, h->cfg.hidden_size, h->pending.residual,
+                          h->pending.out, s, h->xstate));
+    return MUMMU_OK;
+}
+
+// What the fused decode launches are told about the router and the exchange.
+RouterExchange router_exchange_of(mummu_moe *h, const Layer &L, const DecodeScratch &ws, const float *x, const float *norm_gamma,
+                                  float *xnorm_out) {
     RouterExchange rx;
     rx.x = x;
     rx.w = L.router;
@@ -572,7 +636,96 @@ int decode_two_launches(mummu_moe *h, const Layer &L, const DecodeScratch &ws, c
     rx.logits_out = ws.logits;
     rx.spin_ticks = h->spin_ticks;
     rx.fallbacks = ws.xstate + 1;
+    rx.salt = ++h->launch_salt;
     if (L.sh_loaded) rx.xq_out = ws.xq;  // the shared expert's kernels multiply the same 16-bit rows
+    return rx;
+}
+
+// The decode step as one expert launch (router + routing + gate/up + down, see decode_layer_kernel) followed by the
+// weighted sum over each token's slots.  *done = false: not taken, nothing launched.
+int decode_one_launch(mummu_moe *h, const Layer &L, const DecodeScratch &ws, const float *x, int n, int k, int norm,
+                      const float *residual, float *out, hipStream_t s, const float *norm_gamma, float *xnorm_out, bool may_defer,
+                      bool *done) {
+    *done = false;
+    if (!h->layer_fusion || !h->router_exchange || !h->xcd_round_robin || ws.xslots == nullptr || ws.xstate == nullptr ||
+        ws.aslots == nullptr || ws.y == nullptr)
+        return MUMMU_OK;
+    if (n > 1 && h->router_exchange < 2) return MUMMU_OK;  // (like the two-launch form: every workgroup of every token repeats the waits)
+    const ExpertBanks b = banks_of(h, L);
+    LayerExchange lx;
+    lx.act_slots = ws.aslots;
+    lx.y = ws.y;
+    lx.fallbacks = ws.xstate + 1;
+    RouterExchange rx = router_exchange_of(h, L, ws, x, norm_gamma, xnorm_out);
+    if (!decode_layer_supported(b, k, n, rx, lx)) return MUMMU_OK;
+    RouteInline route;
+    route.flavour = h->cfg.router_flavour;
+    route.norm = norm;
+    route.ids = ws.ids;
+    route.weights = ws.weights;
+    route.hits = L.hits;
+    // A step of the chain of deferred sums: this launch adds up what the step before left, and leaves its own rows to the
+    // next one.  It writes the set of buffers the pending step does not occupy.
+    const float *xe = x + (size_t)n * (size_t)b.hidden;
+    const bool chain = may_defer && h->deferred_combine && b.hidden % 256 == 0 && residual == nullptr && norm_gamma == nullptr;
+    PendingSum ps;
+    if (h->pending.active) {
+        const float *po = h->pending.out, *pe = po + (size_t)h->pending.n * (size_t)b.hidden;
+        const bool x_is_pending = x < pe && po < xe;   // this step reads what the pending sum has yet to write
+        if (!chain || h->pending.stream != s || x_is_pending) {
+            const int rc = flush_pending(h);
+            if (rc) return rc;
+        } else {
+            const DecodeBuffers pb = decode_buffers(h, h->pending.buf);
+            ps.y = pb.y;
+            ps.ids = pb.ids;
+            ps.weights = pb.weights;
+            ps.residual = h->pending.residual;
+            ps.out = h->pending.out;
+            ps.n = (int)h->pending.n;
+        }
+    }
+    const int buf = chain ? h->decode_buf : 0;
+    const DecodeBuffers db = decode_buffers(h, buf);
+    lx.y = db.y;
+    route.ids = db.ids;
+    route.weights = db.weights;
+    LAUNCH(h, K_DECODE_LAYER, s, launch_decode_layer(b, rx, lx, route, n, k, h->flags, s, ps));
+    h->pending.active = false;
+    h->routing_buf = buf;
+    if (chain) {
+        h->pending.active = true;
+        h->pending.buf = buf;
+        h->pending.k = k;
+        h->pending.n = n;
+        h->pending.residual = residual;
+        h->pending.out = out;
+        h->pending.stream = s;
+        h->decode_buf = 1 - buf;
+        // (the epoch of the exchange moves on with the next flush; until then the launches differ in their salt)
+        if ((h->launch_salt & 0x3FFFFFFFu) == 0u) {
+            const int rc = flush_pending(h);
+            if (rc) return rc;
+        }
+    } else {
+        LAUNCH(h, K_COMBINE, s, launch_combine(db.y, db.ids, db.weights, nullptr, n, k, b.hidden, residual, out, s, ws.xstate));
+    }
+    *done = true;
+    return MUMMU_OK;
+}
+
+// The decode step in two launches where the device and the shapes allow it: router + routing + gate/up in one kernel
+// (the workgroups exchange the logits inside it), then down + combine.  *done = false: not taken, nothing launched.
+int decode_two_launches(mummu_moe *h, const Layer &L, const DecodeScratch &ws, const float *x, int n, int k, int norm,
+                        const float *residual, float *out, hipStream_t s, const float *norm_gamma, float *xnorm_out, bool *done) {
+    *done = false;
+    if (!h->router_exchange || !h->xcd_round_robin || ws.xslots == nullptr || ws.xstate == nullptr) return MUMMU_OK;
+    // measured on the OLMoE shape (Q4_K): one token 18.1 us against 18.4 in three launches, but 23.6 / 40.2 / 69.5 us
+    // against 22.8 / 36.6 / 57.2 at 2 / 4 / 8 tokens - every workgroup repeats the router wait, and the fused kernel
+    // keeps fewer waves per CU.  So one token only, unless a caller asks for it at every size (tests do).
+    if (n > 1 && h->router_exchange < 2) return MUMMU_OK;
+    const ExpertBanks b = banks_of(h, L);
+    RouterExchange rx = router_exchange_of(h, L, ws, x, norm_gamma, xnorm_out);
     if (!gate_up_fused_supported(b, k, n, rx)) return MUMMU_OK;
     RouteInline route;
     route.flavour = h->cfg.router_flavour;
@@ -589,9 +742,14 @@ int decode_two_launches(mummu_moe *h, const Layer &L, const DecodeScratch &ws, c
 // norm_gamma != nullptr (only where decode_three_launches holds): x is the raw residual stream and the
 // first launch applies the layer's RmsNorm itself.
 int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
-                hipStream_t s, const float *norm_gamma = nullptr, float *xnorm_out = nullptr) {
+                hipStream_t s, const float *norm_gamma = nullptr, float *xnorm_out = nullptr, bool may_defer = false) {
     const Layer &L = h->layers[layer];
     const int E = h->cfg.num_experts, H = h->cfg.hidden_size;
+    h->routing_buf = 0;
+    if (!(may_defer && h->deferred_combine && n <= kExchangeTokens)) {  // (else the one-launch form decides: it may take the pending sum along)
+        const int rc = flush_pending(h);
+        if (rc) return rc;
+    }
     // the fused router also quantizes x when the gate/up banks want it (whole 64-element slices)
     const bool batched = n >= batched_from(h, L);
     const bool want_xq = is_quant_type(L.gate_type) && H % 64 == 0 && !batched;
@@ -609,10 +767,17 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
         return run_experts(h, L, x, want_xq, n, k, residual, out, s, batched, xh.hi != nullptr);
     } else {
         if (want_xq) {
-            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, h->xslots, h->xstate};
+            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, h->xslots, h->xstate, h->aslots, h->y};
             bool done = false;
-            const int rc = decode_two_launches(h, L, ws, x, (int)n, k, norm, residual, out, s, norm_gamma, xnorm_out, &done);
+            int rc = decode_one_launch(h, L, ws, x, (int)n, k, norm, residual, out, s, norm_gamma, xnorm_out, may_defer, &done);
             if (rc || done) return rc;
+            if ((rc = flush_pending(h))) return rc;
+            rc = decode_two_launches(h, L, ws, x, (int)n, k, norm, residual, out, s, norm_gamma, xnorm_out, &done);
+            if (rc || done) return rc;
+        }
+        {
+            const int rc = flush_pending(h);
+            if (rc) return rc;
         }
         // few tokens: the router rows are spread over as many CUs as there are experts
         LAUNCH(h, K_ROUTER_LOGITS, s,
@@ -620,7 +785,7 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
         const ExpertBanks b = banks_of(h, L);
         if (want_xq && gate_up_routes_inline(b, k) && down_combine_supported(b, k)) {
             // ... and the gate/up kernel routes by itself: one launch less on the decode path
-            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, nullptr, nullptr};
+            const DecodeScratch ws{h->logits, h->ids, h->weights, h->xq, h->actq, nullptr, nullptr, nullptr, nullptr};
             return decode_tail(h, L, ws, (int)n, k, norm, residual, out, s);
         }
         if (!batched && float_decode_fused(b, k)) {
@@ -647,9 +812,9 @@ int routed_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int n
 //     out = [residual +] (routed + shared_ffn(x) * sigmoid(<gate_vec, x>))
 // with the product and the two sums rounded separately, in that grouping.
 int forward_impl(mummu_moe *h, int layer, const float *x, int64_t n, int k, int norm, const float *residual, float *out,
-                 hipStream_t s, const float *norm_gamma = nullptr) {
+                 hipStream_t s, const float *norm_gamma = nullptr, bool may_defer = false) {
     const Layer &L = h->layers[layer];
-    if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s, norm_gamma);
+    if (!L.sh_loaded) return routed_impl(h, layer, x, n, k, norm, residual, out, s, norm_gamma, nullptr, may_defer);
     // with the RmsNorm inside the router launch the shared expert reads the normalised rows that launch leaves in h2
     const float *x_raw = x;
     if (norm_gamma) x = h->h2;
@@ -752,6 +917,10 @@ int probe_xcd_round_robin(mummu_moe *h) {
 
 int stack_impl(mummu_moe *h, const float *x, int64_t n, int k, int norm, float *out, hipStream_t s, int32_t *ids_host) {
     const int nl = (int)h->layers.size(), H = h->cfg.hidden_size;
+    {
+        const int rc = flush_pending(h);
+        if (rc) return rc;
+    }
     for (int l = 0; l < nl; l++) {
         int rc = check_layer(h, l);
         if (rc) return rc;
@@ -772,7 +941,8 @@ int stack_impl(mummu_moe *h, const float *x, int64_t n, int k, int norm, float *
         if (rc) return rc;
         if (ids_host) {
             HIPCHK(h, hipStreamSynchronize(s));
-            HIPCHK(h, hipMemcpy(ids_host + (size_t)l * n * k, h->ids, sizeof(int32_t) * (size_t)(n * k), hipMemcpyDeviceToHost));
+            HIPCHK(h, hipMemcpy(ids_host + (size_t)l * n * k, decode_buffers(h, h->routing_buf).ids, sizeof(int32_t) * (size_t)(n * k),
+                                hipMemcpyDeviceToHost));
         }
     }
     return MUMMU_OK;
@@ -876,8 +1046,12 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
             return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(router exchange) failed"));
         if (hipMemset(h->xslots, 0, xb) != hipSuccess || hipMemset(h->xstate, 0, 256) != hipSuccess)
             return bail(fail(h, MUMMU_ERR_DEVICE, "hipMemset(router exchange) failed"));
+        if (hipMalloc(&h->aslots, layer_exchange_bytes()) != hipSuccess || hipMemset(h->aslots, 0, layer_exchange_bytes()) != hipSuccess)
+            return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(hidden-row exchange) failed"));
         if ((rc = probe_xcd_round_robin(h))) return bail(rc);
         if (const char *e = getenv("MUMMU_ROUTER_EXCHANGE")) h->router_exchange = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
+        if (const char *e = getenv("MUMMU_LAYER_FUSION")) h->layer_fusion = atoi(e) != 0;
+        if (const char *e = getenv("MUMMU_DEFERRED_COMBINE")) h->deferred_combine = atoi(e) != 0;
     }
     {
         // resolve the static scratch's address on this device now, outside any stream capture
@@ -892,6 +1066,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
 
 void mummu_moe_destroy(mummu_moe *h) {
     if (!h) return;
+    (void)flush_pending(h);
     (void)hipDeviceSynchronize();
     for (Layer &L : h->layers) {
         void *ptrs[] = {L.router, L.gate, L.up, L.down, L.gamma, L.hits, L.sh_gate, L.sh_up, L.sh_down, L.sh_gatevec};
@@ -901,6 +1076,7 @@ void mummu_moe_destroy(mummu_moe *h) {
     free_ws(h);
     if (h->xslots) (void)hipFree(h->xslots);
     if (h->xstate) (void)hipFree(h->xstate);
+    if (h->aslots) (void)hipFree(h->aslots);
     if (h->flags) (void)hipFree(h->flags);
     for (auto &t : h->timed) {
         (void)hipEventDestroy(t.start);
@@ -917,7 +1093,8 @@ void mummu_moe_destroy(mummu_moe *h) {
 int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router_type, const void *gate, int gate_type,
                          const void *up, int up_type, const void *down, int down_type, const float *rms_gamma) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     if (layer < 0 || layer >= (int)h->layers.size())
         return fail(h, MUMMU_ERR_RANGE, "layer " + std::to_string(layer) + " out of range (" + std::to_string(h->layers.size()) + ")");
     if (!router || !gate || !up || !down) return fail(h, MUMMU_ERR_ARG, "null weight pointer");
@@ -987,7 +1164,8 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
 int mummu_moe_load_shared_expert(mummu_moe *h, int layer, int inter, const void *gate, int gate_type, const void *up, int up_type,
                                  const void *down, int down_type, const void *gate_vec, int gate_vec_type) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);  // the routed part of the layer comes first
     if (rc) return rc;
     if (!gate || !up || !down) return fail(h, MUMMU_ERR_ARG, "null weight pointer");
@@ -1061,7 +1239,8 @@ uint64_t mummu_moe_resident_bytes(const mummu_moe *h) {
 
 int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n, int top_k, int norm, float *out) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
@@ -1078,7 +1257,8 @@ int mummu_moe_forward(mummu_moe *h, int layer, const float *x, int64_t n, int to
 int mummu_moe_forward_typed(mummu_moe *h, int layer, const void *x, int x_type, int64_t n, int top_k, int norm, void *out) {
     if (x_type == MUMMU_F32) return mummu_moe_forward(h, layer, (const float *)x, n, top_k, norm, (float *)out);
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     if (x_type != MUMMU_F16 && x_type != MUMMU_BF16)
         return fail(h, MUMMU_ERR_TYPE, "forward: activations are F32, F16 or BF16 (got type " + std::to_string(x_type) + ")");
     int rc = check_layer(h, layer);
@@ -1107,7 +1287,8 @@ int mummu_moe_forward_typed(mummu_moe *h, int layer, const void *x, int x_type, 
 int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_k, int norm, int32_t *ids, float *weights,
                     float *logits) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
@@ -1128,7 +1309,8 @@ int mummu_moe_route(mummu_moe *h, int layer, const float *x, int64_t n, int top_
 int mummu_route_logits(mummu_moe *h, const float *logits, int64_t n, int n_experts, int top_k, int flavour, int norm,
                        int32_t *ids, float *weights) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     // experts.rs:542-544
     if (n_experts <= 0 || top_k <= 0 || top_k > n_experts)
         return fail(h, MUMMU_ERR_TOPK, "top-" + std::to_string(top_k) + " of " + std::to_string(n_experts) + " experts is not a routing");
@@ -1160,7 +1342,8 @@ int mummu_route_logits(mummu_moe *h, const float *logits, int64_t n, int n_exper
 int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const float *weights, const float *xs, int64_t n,
                             int top_k, float *out) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
@@ -1193,7 +1376,8 @@ int mummu_moe_apply_routing(mummu_moe *h, int layer, const int32_t *ids, const f
 
 int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const float *xs, int64_t n, int top_k, float *out) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if (n <= 0) return n < 0 ? fail(h, MUMMU_ERR_SHAPE, "negative token count") : MUMMU_OK;
@@ -1232,7 +1416,8 @@ int mummu_moe_routed(mummu_moe *h, int layer, const float *router_logits, const 
 
 int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden, float *out) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if (expert < 0 || expert >= h->cfg.num_experts)
@@ -1255,7 +1440,8 @@ int mummu_expert_run(mummu_moe *h, int layer, int expert, const float *x, int64_
 
 int mummu_expert_gate_energy(mummu_moe *h, int layer, int expert, const float *x, int64_t rows, int hidden, float *energy) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if (expert < 0 || expert >= h->cfg.num_experts)
@@ -1290,7 +1476,8 @@ int mummu_expert_gate_energy(mummu_moe *h, int layer, int expert, const float *x
 
 int mummu_moe_take_hits(mummu_moe *h, int layer, uint64_t *hits) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if (!hits) return fail(h, MUMMU_ERR_ARG, "null buffer");
@@ -1303,7 +1490,8 @@ int mummu_moe_take_hits(mummu_moe *h, int layer, uint64_t *hits) {
 
 int mummu_moe_stack_forward(mummu_moe *h, const float *x, int64_t n, int top_k, int norm, float *out, int32_t *ids) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_topk(h, top_k, h->cfg.num_experts);
     if (rc) return rc;
     if (n < 0) return fail(h, MUMMU_ERR_SHAPE, "negative token count");
@@ -1344,7 +1532,8 @@ int mummu_dequantize(int type, const void *bytes, size_t nbytes, float *out) {
 
 int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, int expert, float *out) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if (expert < 0 || expert >= h->cfg.num_experts) return fail(h, MUMMU_ERR_RANGE, "expert out of range");
@@ -1374,13 +1563,14 @@ int mummu_moe_forward_device(mummu_moe *h, int layer, const float *x_dev, int64_
     if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
     if ((rc = check_device_call(h, n, top_k, x_dev, out_dev))) return rc;
     if (n == 0) return MUMMU_OK;
-    return forward_impl(h, layer, x_dev, n, top_k, norm, nullptr, out_dev, (hipStream_t)stream);
+    return forward_impl(h, layer, x_dev, n, top_k, norm, nullptr, out_dev, (hipStream_t)stream, nullptr, /*may_defer=*/true);
 }
 
 int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const float *x_dev, int64_t n, int top_k, int norm, float *out_dev,
                                      void *stream) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = check_layer(h, layer);
     if (rc) return rc;
     if ((rc = check_topk(h, top_k, h->cfg.num_experts))) return rc;
@@ -1443,6 +1633,7 @@ int mummu_expert_run_device(mummu_moe *h, int layer, int expert, const float *x_
     if ((rc = check_device_call(h, rows, 1, x_dev, out_dev))) return rc;
     if (rows == 0) return MUMMU_OK;
     hipStream_t s = (hipStream_t)stream;
+    if ((rc = flush_pending(h))) return rc;
     ExpertBanks b = banks_of(h, h->layers[layer]);
     if (is_quant_type(b.gate_type)) LAUNCH(h, K_QUANTIZE, s, launch_quantize_rows(x_dev, (int)rows, hidden, h->xq, s));
     LAUNCH(h, K_GATE_UP, s, launch_gate_up(b, x_dev, h->xq, nullptr, (int)rows, 1, expert, h->act, h->actq, h->flags, s));
@@ -1461,15 +1652,20 @@ int mummu_moe_stack_forward_device(mummu_moe *h, const float *x_dev, int64_t n, 
 
 int mummu_moe_check(mummu_moe *h, void *stream) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    const int rc = flush_pending(h);
+    if (rc) return rc;
     return check_flags(h, (hipStream_t)stream);
 }
 
 int mummu_moe_last_routing(mummu_moe *h, int64_t n, int top_k, int32_t *ids, float *weights) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     if (n * top_k > h->ws_assign || n < 0 || top_k < 1) return fail(h, MUMMU_ERR_SHAPE, "routing larger than the workspace");
+    const int rc = flush_pending(h);
+    if (rc) return rc;
     HIPCHK(h, hipDeviceSynchronize());
-    if (ids) HIPCHK(h, hipMemcpy(ids, h->ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
-    if (weights) HIPCHK(h, hipMemcpy(weights, h->weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    const DecodeBuffers rb = decode_buffers(h, h->routing_buf);
+    if (ids) HIPCHK(h, hipMemcpy(ids, rb.ids, sizeof(int32_t) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
+    if (weights) HIPCHK(h, hipMemcpy(weights, rb.weights, sizeof(float) * (size_t)(n * top_k), hipMemcpyDeviceToHost));
     return MUMMU_OK;
 }
 
@@ -1514,15 +1710,39 @@ void *mummu_moe_stream(mummu_moe *h) { return h ? (void *)h->stream : nullptr; }
 
 int mummu_moe_set_router_exchange(mummu_moe *h, int enable, unsigned spin_ticks) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     h->router_exchange = enable < 0 ? 0 : (enable > 2 ? 2 : enable);
     h->spin_ticks = spin_ticks;
     return MUMMU_OK;
 }
 
+int mummu_moe_set_layer_fusion(mummu_moe *h, int enable) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
+    h->layer_fusion = enable != 0;
+    return MUMMU_OK;
+}
+
+int mummu_moe_set_deferred_combine(mummu_moe *h, int enable) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
+    h->deferred_combine = enable != 0;
+    return MUMMU_OK;
+}
+
+int mummu_moe_flush(mummu_moe *h) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    Entry entry(h);
+    return entry.rc;
+}
+
 int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbacks) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     if (usable) *usable = h->router_exchange && h->xcd_round_robin;
     if (fallbacks) {
         HIPCHK(h, hipDeviceSynchronize());
@@ -1537,6 +1757,10 @@ int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbac
 int mummu_graph_begin(mummu_moe *h) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     if (h->timing) return fail(h, MUMMU_ERR_ARG, "kernel timing records events; disable it before capturing a graph");
+    {
+        Entry entry(h);  // (a sum pending from eager calls is enqueued ahead of the graph, not inside it)
+        if (entry.rc) return entry.rc;
+    }
     HIPCHK(h, hipStreamBeginCapture(h->stream, hipStreamCaptureModeThreadLocal));
     return MUMMU_OK;
 }
@@ -1544,12 +1768,18 @@ int mummu_graph_begin(mummu_moe *h) {
 int mummu_graph_end(mummu_moe *h, void **graph_exec) {
     if (!h || !graph_exec) return fail(h, MUMMU_ERR_ARG, "null argument");
     hipGraph_t g = nullptr;
-    HIPCHK(h, hipStreamEndCapture(h->stream, &g));
+    std::lock_guard<std::mutex> lock(h->mu);
+    const int frc = flush_pending(h);  // the last captured step's sum becomes the graph's last node
+    hipError_t ce = hipStreamEndCapture(h->stream, &g);
+    if (frc) {
+        if (g) (void)hipGraphDestroy(g);
+        return frc;
+    }
+    if (ce != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("hipStreamEndCapture: ") + hipGetErrorString(ce));
     hipGraphExec_t ex = nullptr;
     hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
     (void)hipGraphDestroy(g);
     if (e != hipSuccess) return fail(h, MUMMU_ERR_DEVICE, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
-    std::lock_guard<std::mutex> lock(h->mu);
     *graph_exec = (void *)new CapturedGraph{ex, h->generation};
     return MUMMU_OK;
 }
@@ -1566,7 +1796,8 @@ static int graph_usable(mummu_moe *h, const CapturedGraph *g) {
 int mummu_graph_launch(mummu_moe *h, void *graph_exec) {
     if (!h || !graph_exec) return fail(h, MUMMU_ERR_ARG, "null argument");
     const CapturedGraph *g = (const CapturedGraph *)graph_exec;
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = graph_usable(h, g);
     if (rc) return rc;
     HIPCHK(h, hipGraphLaunch(g->exec, h->stream));
@@ -1577,7 +1808,8 @@ int mummu_graph_launch_timed(mummu_moe *h, void *graph_exec, int reps, float *ms
     if (!h || !graph_exec || !ms) return fail(h, MUMMU_ERR_ARG, "null argument");
     if (reps < 1 || reps > 65536) return fail(h, MUMMU_ERR_ARG, "reps must be in 1..=65536");
     const CapturedGraph *g = (const CapturedGraph *)graph_exec;
-    std::lock_guard<std::mutex> lock(h->mu);
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
     int rc = graph_usable(h, g);
     if (rc) return rc;
     std::vector<hipEvent_t> ev((size_t)reps + 1, nullptr);

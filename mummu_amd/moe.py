@@ -309,6 +309,20 @@ class SparseMoe:
         bound (10 ns units) of a workgroup's wait for the others' logits."""
         self._check(self._lib.mummu_moe_set_router_exchange(self._h, int(enable), spin_ticks))
 
+    def set_layer_fusion(self, enable):
+        """Whether a decode step on block-quantized banks with top-8 routing runs its experts in ONE launch (router,
+        routing, gate/up and the down product; on by default), else in the two-launch form."""
+        self._check(self._lib.mummu_moe_set_layer_fusion(self._h, int(bool(enable))))
+
+    def set_deferred_combine(self, enable):
+        """With the one-launch decode form: leave the sum over a token's eight weighted rows to the launch of the next
+        forward_device call (off by default).  out of a call is complete after the next call, flush() or check()."""
+        self._check(self._lib.mummu_moe_set_deferred_combine(self._h, int(bool(enable))))
+
+    def flush(self):
+        """Enqueues the sum a deferred decode step left pending; does not synchronise."""
+        self._check(self._lib.mummu_moe_flush(self._h))
+
     def router_exchange_state(self):
         """(two-launch form in use on this device, workgroups that gave up waiting since the last call)."""
         usable, fb = C.c_int(0), C.c_uint64(0)
