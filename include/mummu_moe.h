@@ -208,14 +208,14 @@ MUMMU_API int mummu_moe_dequantize_expert(mummu_moe *h, int layer, int which, in
  * as PAIRS of halfs, x = 2^e * (hi + lo), hi = f16(x / 2^e), lo = f16(x / 2^e - hi), 2^e one power of two per row
  * (per 128 elements between the two products): 22 significant bits per element, every element of a row down to
  * 2^-24 of the row's largest.  That form measures 2e-6 by the reference's measure and has no such corner; it is
- * also the faster one.  The environment variable MUMMU_GEMM_Q4K_F16=0, read by mummu_moe_create, keeps Q4_K on the
+ * also the faster one.  (A row that holds an infinity comes out NaN in that form, where f32 products give an infinity.)  The environment variable MUMMU_GEMM_Q4K_F16=0, read by mummu_moe_create, keeps Q4_K on the
  * integer form above; MUMMU_GEMM_TILE_ROWS=16, 32 or 64 fixes the rows per tile of these kernels (by default the
  * library picks the form with the smallest expected cost for the batch: same results, different speed).
  * Q8_0 banks have an optional second form on the batched path, MUMMU_GEMM_Q8_F16=1 (read by mummu_moe_create):
  * the grouped GEMM of the F16 banks with every weight d * code held exactly as two halfs, x and the activations
  * between the two products rounded to halfs as for F16 / BF16 banks (values beyond 65504 overflow there).  It is
  * 1.1 to 1.5 times faster and measures 1.3e-3 to 1.6e-3 by the reference's measure where the integer form measures
- * 2e-4, which is why it is not the default; a layer with a block whose |d| * 127 is no finite half keeps the
+ * 2e-4, which is why it is not the default; a layer with a block whose |d| * 128 is no finite half keeps the
  * integer form. */
 
 /* ---- device-pointer entry points (no host copies, no synchronisation) ------------------
@@ -246,27 +246,32 @@ MUMMU_API int mummu_moe_forward_device_noalloc(mummu_moe *h, int layer, const fl
  * 10 ns units (default 5000), before it computes them itself - the result has the same bits either way, and with
  * spin_ticks = 0 no workgroup looks for the others' logits at all.  _state reports whether the two-launch form is in
  * use on this device (it is not when workgroups with equal ids modulo 8 do not share an XCD) and returns-and-clears
- * the number of workgroups that gave up waiting. */
+ * the number of workgroups that gave up waiting.  A workgroup that gives up has sat out spin_ticks first - several
+ * steps' worth of time - which happens when the workgroups of a launch are not all resident at once (a device shared
+ * with other work): with the default setting (1) mummu_moe_check switches the handle to three launches for good once it
+ * finds 64 more of them than at its last look. */
 MUMMU_API int mummu_moe_set_router_exchange(mummu_moe *h, int enable, unsigned spin_ticks);
 MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbacks);
 /* With top_k = 8, gate / up banks of Q4_K or Q8_0, a down bank of Q4_K, Q8_0 or Q6_K, at most 128 experts and an
- * intermediate size of at most 1024, the step above runs its experts in ONE launch instead (followed by the small launch
- * that adds up each token's eight weighted rows): the eight expert slots of a token land on the eight XCDs, and the
- * workgroups of a slot pass the expert's hidden row to one another through their XCD's L2 the way the router logits
- * travel, so the down product starts inside the launch that made its input.  No counterpart in the reference.  Same bits
- * as the other forms; the same spin_ticks bounds its waits, and a workgroup that gives up computes the hidden blocks it
- * misses itself (counted by _state's fallbacks).  enable = 0 keeps the two-launch form; 1 (default) uses this one
- * wherever mummu_moe_set_router_exchange's setting allows the fused forms.  Environment: MUMMU_LAYER_FUSION=0. */
+ * intermediate size of at most 1024, the step above can run its experts in ONE launch: the eight expert slots of a token
+ * land on the eight XCDs, and the workgroups of a slot pass the expert's hidden row to one another through their XCD's L2
+ * the way the router logits travel, so the down product starts inside the launch that made its input.  What is left is
+ * the sum over a token's eight weighted rows, which crosses XCDs.  As a launch of its own that sum costs more than the
+ * form saves (19.5 against 17.3 us per layer on the OLMoE shape), so the form pays where a later launch can take the sum
+ * along: mummu_moe_set_deferred_combine.  No counterpart in the reference.  Same bits as the other forms; the same
+ * spin_ticks bounds its waits, and a workgroup that gives up computes the hidden blocks it misses itself (counted by
+ * _state's fallbacks).  enable = 0: never; 1 (default): in chains of deferred sums only; 2: wherever the kernel serves
+ * (every decode call of up to 8 tokens when mummu_moe_set_router_exchange says 2).  Environment: MUMMU_LAYER_FUSION. */
 MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
-/* The one-launch form leaves a token's eight weighted rows to be added up.  With enable = 1 (default 0) a
- * mummu_moe_forward_device call that takes that form no longer enqueues the launch that adds them: the launch of the NEXT
- * such call on the same stream does it on the side (waves that would otherwise wait for the routing), so a sequence of
- * decode steps costs one launch per step.  out_dev of a call is then complete once the next call's work, or
- * mummu_moe_flush, has run on the stream; every other entry point of the handle, mummu_graph_begin / _end / _launch and
- * mummu_moe_check enqueue a pending sum first, so a captured graph always ends with its last step's sum and a caller
- * that reads out_dev after mummu_moe_check sees it whole.  A call whose input overlaps the pending output is preceded by
- * that sum as well.  No counterpart in the reference.  Same bits as mummu_moe_forward_device without it.  Not taken with a
- * shared expert on the layer or inside mummu_moe_stack_forward*.  Environment: MUMMU_DEFERRED_COMBINE=1. */
+/* enable = 1 (default 0): a mummu_moe_forward_device call that can take the one-launch form no longer enqueues the sum over
+ * each token's eight weighted rows; the launch of the NEXT such call on the same stream does it on the side (a wave per
+ * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (14.9 us
+ * per layer on the OLMoE shape).  out_dev of a call is then complete once the next call's work, or mummu_moe_flush, has
+ * run on the stream; every other entry point of the handle, mummu_graph_begin / _end and mummu_moe_check enqueue a
+ * pending sum first, so a captured graph always ends with its last step's sum and a caller that reads out_dev after
+ * mummu_moe_check sees it whole.  A call whose input overlaps the pending output is preceded by that sum as well.
+ * No counterpart in the reference.  Same bits as mummu_moe_forward_device without it.  Not taken with a shared expert on
+ * the layer or inside mummu_moe_stack_forward*.  Environment: MUMMU_DEFERRED_COMBINE=1. */
 MUMMU_API int mummu_moe_set_deferred_combine(mummu_moe *h, int enable);
 /* Enqueues the sum a deferred step left pending (nothing to do otherwise); does not synchronise. */
 MUMMU_API int mummu_moe_flush(mummu_moe *h);

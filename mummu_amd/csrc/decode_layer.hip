@@ -77,21 +77,24 @@ __device__ __forceinline__ void quantize_tile_to_lds(const float *s_act, int row
     }
 }
 
+constexpr int kDlWaves = 4;  // waves per workgroup (eight, in half as many workgroups, measured the same: 14.9 us per layer)
+
 template <int WT, int DT, int NITD, int RJN>
-__global__ __launch_bounds__(256) void decode_layer_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
-                                                           const uint8_t *down /* not __restrict__: a code fence orders its loads */,
+// (the three banks are not __restrict__: the code fences between the row loads must order them - gate/up rows first,
+// the down rows behind them - and the compiler moves loads of restrict pointers across such a fence as it likes)
+__global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8_t *gate, const uint8_t *up, const uint8_t *down,
                                                            int k, int hidden, int inter, int n_experts, int32_t *__restrict__ flags,
                                                            RouteInline route, RouterExchange rx, LayerExchange lx, PendingSum ps) {
     constexpr int NIT = 4;
     extern __shared__ float s_dyn[];  // gate/up results of a tile | the token's 16-bit row | the slot's 16-bit hidden row
     __shared__ __attribute__((aligned(16))) DecodeShared<RJN> sh;
-    __shared__ unsigned long long s_missing[4];
+    __shared__ unsigned long long s_missing[4];   // (256 pieces at most: the first four waves look for them)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.z, slot = blockIdx.x, tile = blockIdx.y;  // grid = (slot, row tile, token)
     const int a = t * gridDim.x + slot;
     const RowSplit rs = row_split(hidden);
     const int unit0 = lane & (rs.group - 1);
-    const int rows_per_block = NIT * rs.rows_per_it * 4;
+    const int rows_per_block = NIT * rs.rows_per_it * kDlWaves;
     float *s_act = s_dyn;
     int8_t *s_xhi = (int8_t *)(s_dyn + rows_per_block);
     int8_t *s_xlo = s_xhi + hidden;
@@ -121,20 +124,25 @@ __global__ __launch_bounds__(256) void decode_layer_kernel(const uint8_t *__rest
     // row has been, so that they queue up behind them
     const RowSplit rsd = row_split(inter);
     const int subd = lane >> rsd.group_log2, unit0d = lane & (rsd.group - 1);
-    const int down_rows_wg = 4 * NITD * rsd.rows_per_it;
+    const int down_rows_wg = kDlWaves * NITD * rsd.rows_per_it;
     const int drow0 = tile * down_rows_wg + wave * NITD * rsd.rows_per_it;
     const size_t drow_bytes = type_row_bytes(DT, inter);
     const uint8_t *de = down + (size_t)e * (size_t)hidden * drow_bytes;
     RawRow<DT, 1> rd[NITD];
-    auto fetch_down = [&]() {
+    auto fetch_down = [&](float after) {
+        // (an offset of zero that the compiler cannot see through: the loads below wait for the value it is made of)
+        unsigned zero;
+        asm volatile("v_and_b32 %0, 0, %1" : "=v"(zero) : "v"(after));
 #pragma unroll
         for (int i = 0; i < NITD; i++) {
             const int row = drow0 + i * rsd.rows_per_it + subd;
             const bool ok = row < hidden;
-            load_row<DT, 1>(de + (size_t)(ok ? row : 0) * drow_bytes, unit0d, rsd.units, ok, rd[i]);
+            load_row<DT, 1>(de + (size_t)(ok ? row : 0) * drow_bytes + zero, unit0d, rsd.units, ok, rd[i]);
         }
     };
-    gate_up_tile<WT, 1, NIT, true, false>(gate, up, e, a, la, rs, hidden, inter, nullptr, QAct(), s_act, tile, fetch_down);
+    // (asked for behind the dots of iteration 0 / 1 / 2 / 3, one token on the OLMoE shape: 15.5 / 14.8 / 14.9 / 15.3 us per layer;
+    // together with the gate/up rows, which is where the compiler puts every load it is free to move: 15.0)
+    gate_up_tile<WT, 1, NIT, true, false, decltype(fetch_down), 1>(gate, up, e, a, la, rs, hidden, inter, nullptr, QAct(), s_act, tile, fetch_down);
     __syncthreads();
     MUMMU_PHASE(4);
 
@@ -157,7 +165,7 @@ __global__ __launch_bounds__(256) void decode_layer_kernel(const uint8_t *__rest
     {
         const int blk = (int)threadIdx.x >> 2, piece = (int)threadIdx.x & 3;
         const bool own = blk >= tile * blocks_per_tile && blk < (tile + 1) * blocks_per_tile;
-        bool have = blk >= n_blocks || own;
+        bool have = blk >= n_blocks || own;   // (threads from 256 on: blk >= kActBlocksMax >= n_blocks)
         const unsigned want = act_piece_tag(epoch, rx.salt, pos0 + threadIdx.x);
         const unsigned long long t_begin = wall_clock64();
         bool complete = __all(have);
@@ -177,7 +185,7 @@ __global__ __launch_bounds__(256) void decode_layer_kernel(const uint8_t *__rest
             __builtin_amdgcn_s_sleep(1);
         }
         const unsigned long long missing = __ballot(!have);
-        if (lane == 0) s_missing[wave] = missing;
+        if (lane == 0 && wave < 4) s_missing[wave] = missing;
     }
     __syncthreads();
     MUMMU_PHASE(15);
@@ -225,9 +233,9 @@ __global__ __launch_bounds__(256) void decode_layer_kernel(const uint8_t *__rest
 // ------------------------------------------------------------------------------------------
 static int decode_layer_down_iters(const ExpertBanks &b) {
     const RowSplit rs = row_split(b.hidden), rsd = row_split(b.inter);
-    const int rpb = 4 * 4 * rs.rows_per_it;
+    const int rpb = kDlWaves * 4 * rs.rows_per_it;
     const int tiles = (b.inter + rpb - 1) / rpb;
-    const int per_it = 4 * rsd.rows_per_it * tiles;  // down rows the grid covers per iteration
+    const int per_it = kDlWaves * rsd.rows_per_it * tiles;  // down rows the grid covers per iteration
     return (b.hidden + per_it - 1) / per_it;
 }
 
@@ -248,8 +256,8 @@ template <int WT, int DT, int NITD>
 static hipError_t launch_decode_layer_t(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
                                         int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
     const RowSplit rs = row_split(b.hidden);
-    const int rpb = 4 * 4 * rs.rows_per_it;
-    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(256);
+    const int rpb = kDlWaves * 4 * rs.rows_per_it;
+    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(64 * kDlWaves);
     const size_t lds = sizeof(float) * (size_t)rpb + 2 * (size_t)b.hidden + 8 * (size_t)(b.hidden / 16) + 2 * (size_t)b.inter +
                        8 * (size_t)(b.inter / 16);
     if (b.n_experts <= 64)

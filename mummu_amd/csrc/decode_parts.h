@@ -12,19 +12,21 @@ namespace mummu {
 
 struct NoHook {
     __device__ __forceinline__ void operator()() const {}
+    __device__ __forceinline__ void operator()(float) const {}
 };
 
 // The gate/up products of one (token, expert) assignment `a` for tile `tile` of output rows, given the
 // lane's share `la` of the token's 16-bit activations: NIT iterations of rows_per_it rows per wave, then
 // silu(gate) * up per row, written as f32 (act) or staged in LDS (s_act, rows_per_block floats) and - with STORE -
 // re-quantized to 16-bit blocks for the down product (ACTQ).  Without STORE the rows are left in s_act and the caller
-// goes on after a barrier of its own.  `all_issued` runs once the loads of every row have been asked for: the place
-// for loads that should queue up behind them.
-template <int WT, int UPL, int NIT, bool ACTQ, bool STORE = true, typename Hook = NoHook>
-__device__ __forceinline__ void gate_up_tile(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, int e, int a,
+// goes on after a barrier of its own.  `hook` runs behind the dots of iteration HOOK_AT and is handed one of their
+// results: loads whose address it makes depend on that value cannot be asked for before the rows of that iteration have
+// arrived (the compiler hoists every independent load to the top of the function, whatever fences lie between).
+template <int WT, int UPL, int NIT, bool ACTQ, bool STORE = true, typename Hook = NoHook, int HOOK_AT = NIT - 1>
+__device__ __forceinline__ void gate_up_tile(const uint8_t *gate, const uint8_t *up /* (restrict or not is the kernel's choice) */, int e, int a,
                                              const LaneAct<UPL> &la, const RowSplit &rs, int hidden, int inter,
                                              float *__restrict__ act, const QAct &actq, float *s_act, int tile,
-                                             Hook all_issued = Hook()) {
+                                             Hook hook = Hook()) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
     const int rows_per_wave = NIT * rs.rows_per_it;
@@ -49,19 +51,16 @@ __device__ __forceinline__ void gate_up_tile(const uint8_t *__restrict__ gate, c
     constexpr int AHEAD = NIT < 2 ? NIT : 2;
 #pragma unroll
     for (int i = 0; i < AHEAD; i++) fetch(i);
-    if (AHEAD == NIT) all_issued();
     MUMMU_CODE_FENCE();
     MUMMU_PHASE(1);
     float part[2 * NIT];
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
-        if (i + AHEAD < NIT) {
-            fetch(i + AHEAD);
-            if (i + AHEAD == NIT - 1) all_issued();
-        }
+        if (i + AHEAD < NIT) fetch(i + AHEAD);
         MUMMU_CODE_FENCE();
         part[2 * i] = dot_row<WT, UPL>(rg[i], unit0, la);
         part[2 * i + 1] = dot_row<WT, UPL>(ru[i], unit0, la);
+        if (i == HOOK_AT) hook(part[2 * i + 1]);
         MUMMU_CODE_FENCE();
     }
     MUMMU_PHASE(2);

@@ -116,7 +116,7 @@ __device__ inline bool xcd_tile(const int32_t *__restrict__ n_tiles, int slabs, 
 // then 8 codes and their block's d; the codes go to LDS as they are, and the wave that owns a column turns its 8
 // codes of an instruction into two operands, hi + lo = d * code exactly, and multiplies both: twice the matrix
 // work of an f16 bank at half the bytes, and the weights lose nothing (x and the activations between the two
-// products are halfs, as for every bank of this kernel).  Needs |d| * 127 inside the half range.
+// products are halfs, as for every bank of this kernel).  Needs |d| * 128 inside the half range.
 template <bool GATE_UP, int MT, int WT>
 __global__ __launch_bounds__(256) void grouped_gemm_f16_kernel(
     const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, const _Float16 *__restrict__ act_in,
@@ -1671,7 +1671,7 @@ hipError_t launch_q8_scale_max(const uint8_t *bank, size_t n_blocks, uint32_t *m
 }
 
 // Q8_0 banks through the f16 kernel (every weight as two halfs): all three banks Q8_0 and, checked when the layer
-// was loaded, every |d| * 127 inside the half range
+// was loaded, every |d| * 128 inside the half range
 bool grouped_gemm_q8_f16(const ExpertBanks &b) {
     return b.q8_half_ok && b.gate_type == T_Q8_0 && b.up_type == T_Q8_0 && b.down_type == T_Q8_0 && b.hidden % 64 == 0 &&
            b.inter % 64 == 0;

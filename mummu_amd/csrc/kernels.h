@@ -49,7 +49,7 @@ struct ExpertBanks {
     const uint8_t *gate, *up, *down;  // device, GGUF order
     int gate_type, up_type, down_type;
     int hidden, inter, n_experts;
-    bool q8_half_ok = false;          // Q8_0 banks whose every |d| * 127 is inside the half range (launch_q8_scale_max)
+    bool q8_half_ok = false;          // Q8_0 banks whose every |d| * 128 is inside the half range (launch_q8_scale_max)
 };
 
 

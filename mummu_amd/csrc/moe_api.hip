@@ -38,7 +38,7 @@ struct Layer {
     unsigned long long *hits = nullptr;
     size_t bytes = 0;
     bool loaded = false;
-    bool q8_half_ok = false;     // all three banks Q8_0 and every |d| * 127 a finite half: the f16 kernel may take them
+    bool q8_half_ok = false;     // all three banks Q8_0 and every |d| * 128 a finite half: the f16 kernel may take them
     // optional shared expert (always active) and its per-token sigmoid gate vector
     uint8_t *sh_gate = nullptr, *sh_up = nullptr, *sh_down = nullptr;
     int sh_gate_type = 0, sh_up_type = 0, sh_down_type = 0, sh_inter = 0;
@@ -115,10 +115,11 @@ struct mummu_moe {
     bool xcd_round_robin = false;
     int router_exchange = 1;
     unsigned spin_ticks = 5000;
+    unsigned long long fallbacks_seen = 0;   // the fallback counter at mummu_moe_check's last look
     // the one-launch decode form (decode_layer_kernel): the table its workgroups pass the experts' hidden rows through,
     // and a counter that tells launches apart which read the same epoch (the nodes of one captured graph)
     void *aslots = nullptr;
-    int layer_fusion = 1;
+    int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
     // off by default), whose otherwise idle waves do it: the one-launch form then costs one launch per step.  The per-slot
@@ -324,11 +325,24 @@ int reset_flags(mummu_moe *h) {
 
 int flags_to_status(mummu_moe *h, const int32_t *f);
 
+constexpr unsigned long long kFallbacksBeforeGivingUp = 64;
+
 // Synchronise and translate the device error flags.
 int check_flags(mummu_moe *h, hipStream_t s) {
     HIPCHK(h, hipStreamSynchronize(s));
     int32_t f[4];
     HIPCHK(h, hipMemcpy(f, h->flags, sizeof(f), hipMemcpyDeviceToHost));
+    if (h->router_exchange == 1 && h->xstate != nullptr) {
+        // Workgroups of the fused decode forms that gave up waiting for the others since the last look: each of them sat
+        // out its bound (spin_ticks, tens of microseconds against a step of 15) before it computed what it missed - the
+        // device is shared, or it does not place workgroups the way the probe saw.  The result is right either way, but
+        // the three-launch form is the faster one then: fall back to it for the rest of this handle's life.  (A caller
+        // that set the form explicitly - mummu_moe_set_router_exchange with 0 or 2 - keeps what it asked for.)
+        unsigned long long fb = 0;
+        HIPCHK(h, hipMemcpy(&fb, h->xstate + 1, sizeof(fb), hipMemcpyDeviceToHost));
+        if (fb - h->fallbacks_seen >= kFallbacksBeforeGivingUp) h->router_exchange = 0;
+        h->fallbacks_seen = fb;
+    }
     return flags_to_status(h, f);
 }
 
@@ -505,6 +519,9 @@ HalfPlan half_plan(const mummu_moe *h, const ExpertBanks &b, int64_t n, int k) {
     const bool small32 = na * (size_t)(b.hidden > b.inter ? b.hidden : b.inter) * 2 < (1ull << 32);
     p.hf = h->gemm_q4k_f16 && small32 && grouped_gemm_q4k_f16(b);
     p.hf_down = p.hf && grouped_gemm_q4k_f16_down(b);
+    // x as pairs of halfs borrows h->y (the down product's output, written only after the gate/up launch has read x) and
+    // the scale / sum arrays of the 16-bit form (unused on this path): run_experts keeps the order quantize -> gate/up ->
+    // down on one stream, and nothing else may hold h->y across the gate/up launch
     if (p.hf) p.xh = HAct{(_Float16 *)h->y, (_Float16 *)h->y + (size_t)n * b.hidden, h->xq.scale, (float *)h->xq.sum};
     return p;
 }
@@ -668,6 +685,9 @@ int decode_one_launch(mummu_moe *h, const Layer &L, const DecodeScratch &ws, con
     // next one.  It writes the set of buffers the pending step does not occupy.
     const float *xe = x + (size_t)n * (size_t)b.hidden;
     const bool chain = may_defer && h->deferred_combine && b.hidden % 256 == 0 && residual == nullptr && norm_gamma == nullptr;
+    // (followed by a launch of its own for the sum the form is slower than two launches - 19.5 against 17.3 us per layer on
+    // the OLMoE shape - so outside a chain it is taken only on request)
+    if (!chain && h->layer_fusion < 2) return MUMMU_OK;
     PendingSum ps;
     if (h->pending.active) {
         const float *po = h->pending.out, *pe = po + (size_t)h->pending.n * (size_t)b.hidden;
@@ -900,7 +920,8 @@ int probe_xcd_round_robin(mummu_moe *h) {
     hipError_t e = hipSuccess;
     for (int rep = 0; rep < 2 && e == hipSuccess; rep++) {
         launch_kernel(xcd_probe_kernel, dim3(8, kProbe / 8), dim3(256), 0, h->stream, d);
-        e = hipMemcpyAsync(got.data(), d, sizeof(int) * kProbe, hipMemcpyDeviceToHost, h->stream);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipMemcpyAsync(got.data(), d, sizeof(int) * kProbe, hipMemcpyDeviceToHost, h->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
         for (int i = 0; i < kProbe && e == hipSuccess; i++) rr = rr && got[i] == got[i & 7];
     }
@@ -1050,7 +1071,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
             return bail(fail(h, MUMMU_ERR_DEVICE, "hipMalloc(hidden-row exchange) failed"));
         if ((rc = probe_xcd_round_robin(h))) return bail(rc);
         if (const char *e = getenv("MUMMU_ROUTER_EXCHANGE")) h->router_exchange = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
-        if (const char *e = getenv("MUMMU_LAYER_FUSION")) h->layer_fusion = atoi(e) != 0;
+        if (const char *e = getenv("MUMMU_LAYER_FUSION")) h->layer_fusion = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
         if (const char *e = getenv("MUMMU_DEFERRED_COMBINE")) h->deferred_combine = atoi(e) != 0;
     }
     {
@@ -1143,7 +1164,7 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
     L.up_type = up_type;
     L.down_type = down_type;
     if (gate_type == T_Q8_0 && up_type == T_Q8_0 && down_type == T_Q8_0) {
-        // the f16 kernel multiplies d * code as halfs: only banks whose largest |d| * 127 is a finite half (d <= 512)
+        // the f16 kernel multiplies d * code as halfs: only banks whose largest |d| * 128 is a finite half (|d| < 512: a code may be -128)
         uint32_t *max_bits = nullptr, got = 0;
         HIPCHK(h, hipMalloc((void **)&max_bits, sizeof(uint32_t)));
         hipError_t e = hipMemsetAsync(max_bits, 0, sizeof(uint32_t), h->stream);
@@ -1154,7 +1175,7 @@ int mummu_moe_load_layer(mummu_moe *h, int layer, const void *router, int router
         if (e == hipSuccess) e = hipMemcpy(&got, max_bits, sizeof(uint32_t), hipMemcpyDeviceToHost);
         (void)hipFree(max_bits);
         HIPCHK(h, e);
-        L.q8_half_ok = got <= 0x6000u;   // half bits of 512.0
+        L.q8_half_ok = got < 0x6000u;   // half bits of 512.0: 512 * -128 = -65536 rounds to -inf
     }
     L.bytes = rb + gb + ub + db + (rms_gamma ? sizeof(float) * (size_t)H : 0);
     L.loaded = true;
@@ -1721,7 +1742,7 @@ int mummu_moe_set_layer_fusion(mummu_moe *h, int enable) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     Entry entry(h);
     if (entry.rc) return entry.rc;
-    h->layer_fusion = enable != 0;
+    h->layer_fusion = enable < 0 ? 0 : (enable > 2 ? 2 : enable);
     return MUMMU_OK;
 }
 
@@ -1749,6 +1770,7 @@ int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_t *fallbac
         unsigned long long v = 0, zero = 0;
         HIPCHK(h, hipMemcpy(&v, h->xstate + 1, sizeof(v), hipMemcpyDeviceToHost));
         HIPCHK(h, hipMemcpy(h->xstate + 1, &zero, sizeof(zero), hipMemcpyHostToDevice));
+        h->fallbacks_seen = 0;
         *fallbacks = v;
     }
     return MUMMU_OK;

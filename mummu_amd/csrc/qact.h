@@ -117,6 +117,9 @@ struct HAct {
 };
 
 // The scale for a largest magnitude m = f * 2^ex, f in [0.5, 1): x / scale = x * 2^(10 - ex).
+// A non-finite m (exponent 255) gives hi = inf and lo = inf - inf = NaN for an infinite element: a row that holds an
+// infinity comes out NaN where the reference's f32 product gives an infinity (non-finite rows are outside what the
+// parity tests pin).
 __device__ inline void hact_scale_of(float m, float &inv, float &scale) {
     int ex = (int)((__float_as_uint(m) >> 23) & 255u) - 126;
     ex = ex < -116 ? -116 : ex;

@@ -276,7 +276,9 @@ __device__ __forceinline__ void route_token(float (&l)[JN], int t, int n_experts
             const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
             denom = fs > floor_v ? fs : floor_v;
         }
-        if (my_slot >= 0) {
+        // (a lane past n_experts never wins a round while a real candidate is left: its -1 loses to every probability,
+        // which is a finite non-negative float here - non-finite logits were refused above; the bound is kept all the same)
+        if (my_slot >= 0 && lane < n_experts) {
             float wv = p[0];
             if (flavour != 0 || norm) wv = __fdiv_rn(wv, denom);
             ids[orow * k + my_slot] = lane;

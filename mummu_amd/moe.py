@@ -311,8 +311,9 @@ class SparseMoe:
 
     def set_layer_fusion(self, enable):
         """Whether a decode step on block-quantized banks with top-8 routing runs its experts in ONE launch (router,
-        routing, gate/up and the down product; on by default), else in the two-launch form."""
-        self._check(self._lib.mummu_moe_set_layer_fusion(self._h, int(bool(enable))))
+        routing, gate/up and the down product): 0 / False never, 1 / True (default) in chains of deferred sums only,
+        2 wherever the kernel serves."""
+        self._check(self._lib.mummu_moe_set_layer_fusion(self._h, int(enable)))
 
     def set_deferred_combine(self, enable):
         """With the one-launch decode form: leave the sum over a token's eight weighted rows to the launch of the next

@@ -66,7 +66,7 @@ def test_half_form_matches_the_f64_reference(monkeypatch, H, I, E, k, n):
 
 
 def test_a_bank_with_a_scale_outside_the_half_range_keeps_the_int8_form(monkeypatch):
-    # one block of the up bank with d = 1000: d * 127 is no finite half, so the layer is not eligible and both
+    # one block of the up bank with d = 1000: d * 128 is no finite half, so the layer is not eligible and both
     # settings of the switch run the same kernels
     H, I, E, k, n = 512, 256, 8, 2, 200
     x = normal((n, H), 91)
@@ -79,6 +79,23 @@ def test_a_bank_with_a_scale_outside_the_half_range_keeps_the_int8_form(monkeypa
     # 16-bit block-scaled activations of the int8 form are known to lose small elements in)
     got, _ = run(monkeypatch, True, H, I, E, k, x, (gate, up, down), seed=93)
     got8, _ = run(monkeypatch, False, H, I, E, k, x, (gate, up, down), seed=93)
+    assert np.all(np.isfinite(got))
+    assert np.array_equal(got.view(np.uint32), got8.view(np.uint32))
+
+
+def test_a_scale_of_512_with_a_code_of_minus_128_keeps_the_int8_form(monkeypatch):
+    # d = 512 and a code of -128 (the reference's encoder never writes one, a file may hold it): d * code = -65536 is
+    # no finite half, so |d| must stay BELOW 512 for the half form and this layer keeps the integer one
+    H, I, E, k, n = 512, 256, 8, 2, 200
+    x = normal((n, H), 94)
+    gate, up, down = banks_of(H, I, E, 95)
+    up = up.copy()
+    bits = int(np.array([512.0], dtype=np.float16).view(np.uint16)[0])
+    blk = 34 * 77
+    up[blk], up[blk + 1] = bits & 0xFF, bits >> 8
+    up[blk + 2] = 0x80  # code -128
+    got, _ = run(monkeypatch, True, H, I, E, k, x, (gate, up, down), seed=96)
+    got8, _ = run(monkeypatch, False, H, I, E, k, x, (gate, up, down), seed=96)
     assert np.all(np.isfinite(got))
     assert np.array_equal(got.view(np.uint32), got8.view(np.uint32))
 

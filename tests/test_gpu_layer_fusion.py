@@ -54,7 +54,7 @@ def test_one_launch_gives_the_bits_of_two_and_three(H, I, E, k, gt, dt, rt, flav
         for n in (1, 3, 8):
             x = g.standard_normal((n, H), dtype=np.float32)
             m.set_router_exchange(2)
-            m.set_layer_fusion(True)
+            m.set_layer_fusion(2)
             m.kernel_timing(True)
             one = m.forward(x, k, flavour == 1)
             r1 = m.last_routing(n, k)
@@ -92,7 +92,7 @@ def test_stack_with_the_norm_inside_the_one_launch_form():
         for n in (1, 5):
             x = (3.0 * g.standard_normal((n, H), dtype=np.float32)).astype(np.float32)
             m.set_router_exchange(2)
-            m.set_layer_fusion(True)
+            m.set_layer_fusion(2)
             one, ids1 = m.stack_forward(x, k, False, return_ids=True)
             m.set_router_exchange(False)
             three, ids3 = m.stack_forward(x, k, False, return_ids=True)
@@ -111,6 +111,7 @@ def test_graph_replays_of_the_one_launch_form():
         m.set_router_exchange(False)
         want = [m.forward(x, k, False) for x in xs]
         m.set_router_exchange(True)
+        m.set_layer_fusion(2)
         xd = [M.DeviceBuffer.from_array(x) for x in xs]
         od = [M.DeviceBuffer(H * 4) for _ in xs]
         m.graph_begin()
@@ -145,7 +146,7 @@ def test_shared_expert_beside_the_one_launch_form():
         for n in (1, 4):
             x = g.standard_normal((n, H), dtype=np.float32)
             m.set_router_exchange(2)
-            m.set_layer_fusion(True)
+            m.set_layer_fusion(2)
             one = m.forward(x, k, False)
             m.set_router_exchange(False)
             three = m.forward(x, k, False)

@@ -43,6 +43,60 @@ def test_noalloc_forward_gives_the_bits_of_forward_device_on_two_calls_in_a_row(
             assert np.array_equal(bits(want), bits(m.forward(x, k, False)))
 
 
+def test_noalloc_forward_with_the_logit_table_at_every_offset_under_graph_capture_and_on_two_handles():
+    # The static array is carved per call: with the two-launch form forced at every size, the router's logit table lands
+    # behind buffers whose size follows the token count and top_k, on bytes that earlier calls used for activations.
+    # Calls captured into a graph (what the entry point is for) and two handles taking turns on one stream share it too.
+    H, I, E = 1024, 512, 32
+    g = np.random.Generator(np.random.PCG64(911))
+    handles = []
+    for j in range(2):
+        gate = synth.random_bank_fast(M.Q4_K, [H, I, E], 920 + 3 * j)
+        up = synth.random_bank_fast(M.Q4_K, [H, I, E], 921 + 3 * j)
+        down = synth.random_bank_fast(M.Q4_K, [I, H, E], 922 + 3 * j)
+        router = (g.standard_normal((E, H), dtype=np.float32) * np.float32(0.05)).astype(np.float16)
+        m = M.SparseMoe(M.SparseMoeConfig(H, I, E, 8), max_tokens=8)
+        m.load_layer(0, router, M.F16, gate, M.Q4_K, up, M.Q4_K, down, M.Q4_K)
+        handles.append(m)
+    try:
+        a, b = handles
+        for m in handles:
+            m.set_router_exchange(2)
+        for n, k in ((8, 8), (3, 4), (1, 8), (5, 2), (1, 4)):
+            x = g.standard_normal((n, H), dtype=np.float32)
+            xd = M.DeviceBuffer.from_array(x)
+            for m in (a, b, a):  # taking turns: each call finds the other handle's data in the array
+                got_d = M.DeviceBuffer(x.nbytes)
+                got_d.upload(np.full((n, H), np.nan, np.float32))
+                m.forward_device_noalloc(0, xd, n, k, False, got_d)
+                m.check()
+                assert np.array_equal(bits(got_d.download(np.float32, (n, H))), bits(m.forward(x, k, False))), (n, k)
+        assert a.router_exchange_state()[1] == 0 and b.router_exchange_state()[1] == 0
+        # captured: three calls of different sizes in one graph, replayed with fresh inputs
+        shapes = ((1, 8), (4, 8), (2, 4))
+        xs = [g.standard_normal((n, H), dtype=np.float32) for n, _ in shapes]
+        xd = [M.DeviceBuffer.from_array(x) for x in xs]
+        od = [M.DeviceBuffer(x.nbytes) for x in xs]
+        a.graph_begin()
+        for (n, k), x, o in zip(shapes, xd, od):
+            a.forward_device_noalloc(0, x, n, k, False, o)
+        graph = a.graph_end()
+        for rep in range(3):
+            for o, x in zip(od, xs):
+                o.upload(np.full(x.shape, np.nan, np.float32))
+            graph.launch()
+            a.check()
+            for (n, k), x, o in zip(shapes, xs, od):
+                assert np.array_equal(bits(o.download(np.float32, (n, H))), bits(a.forward(x, k, False))), (rep, n, k)
+            xs = [g.standard_normal((n, H), dtype=np.float32) for n, _ in shapes]
+            for d, x in zip(xd, xs):
+                d.upload(x)
+        graph.close()
+    finally:
+        for m in handles:
+            m.close()
+
+
 def test_noalloc_forward_refuses_what_it_cannot_hold():
     H, I, E, k = 256, 64, 8, 2
     rng = synth.SplitMix64(5)
