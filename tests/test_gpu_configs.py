@@ -210,37 +210,46 @@ def run_c4(L, n, seed, layer_tol=None):
     return got, gids, cur, np.stack(oids), np.stack(margins)
 
 
-def check_stack(got, gids, want, oids, margins, tol):
+def check_stack(got, gids, want, oids, margins, tol, max_flips, max_margin):
     # A layer routes the GPU's own residual stream, which differs from the oracle's by the
     # expert products' rounding: a token whose closest pair among its top k+1 probabilities is
     # nearer than that noise may legitimately swap two slots or pick the other expert.  Such
     # tokens must be rare and near-tied; every other token must route identically in every layer.
-    # `tol` bounds max|got - want| over a row in units of the row's rms: over 2048 elements the
-    # maximum of an error with relative rms r is about 4.5 r, so 2e-3 per element is 9e-3 here.
+    # `tol` bounds max|got - want| over a row in units of the row's rms (over 2048 elements the
+    # maximum of an error with relative rms r is about 4.5 r).  The three bounds are set about 1.5x
+    # above what this configuration measures (printed below; run with -s to see them), so that a
+    # regression of the arithmetic shows here long before it reaches the 2e-3 bar of a single layer.
     L, n, _ = gids.shape
     same = np.array([[np.array_equal(gids[l, t], oids[l, t]) for t in range(n)] for l in range(L)])
     assert same[0].all(), "layer 0 sees the same input: routing must be exact"
     flipped = ~same
-    assert flipped.sum() <= max(1, int(0.02 * L * n)), f"{flipped.sum()} of {L * n} (layer, token) routings differ"
     first = np.argmax(flipped, axis=0)  # first layer at which each flipped token departs
-    for t in np.nonzero(flipped.any(axis=0))[0]:
-        assert margins[first[t], t] < 5e-3, f"token {t} flipped at layer {first[t]} with margin {margins[first[t], t]:.3e}"
+    departed = np.nonzero(flipped.any(axis=0))[0]
+    worst_margin = max((float(margins[first[t], t]) for t in departed), default=0.0)
     same_set = np.array([[sorted(gids[l, t]) == sorted(oids[l, t]) for t in range(n)] for l in range(L)]).all(axis=0)
-    assert same_set.mean() >= 0.95
     scale = np.sqrt((want.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
-    err = (np.abs(got - want) / scale)[same_set].max()
-    assert err <= tol, f"residual stream off by {err:.3e}"
+    err = float((np.abs(got - want) / scale)[same_set].max())
+    print(f"\nstack of {L} layers x {n} tokens: {int(flipped.sum())} of {L * n} (layer, token) routings differ from the oracle's, "
+          f"{departed.size} tokens depart (largest margin at the departure {worst_margin:.3e}), {int((~same_set).sum())} tokens end "
+          f"on another expert set, residual stream off by {err:.3e} of the row rms")
+    assert flipped.sum() <= max_flips, f"{flipped.sum()} of {L * n} (layer, token) routings differ (bound {max_flips})"
+    assert worst_margin <= max_margin, f"a token departed with margin {worst_margin:.3e} (bound {max_margin:.1e})"
+    assert same_set.mean() >= 0.95
+    assert err <= tol, f"residual stream off by {err:.3e} (bound {tol:.1e})"
 
 
 def test_c4_sixteen_layer_q8_0_stack_decode():
-    check_stack(*run_c4(16, 1, 400), tol=2e-3)  # integer GEMV with 16-bit activations: far inside
+    # integer GEMV with 16-bit activations; measured: no routing differs, residual stream off by 8.5e-4 of the row rms
+    check_stack(*run_c4(16, 1, 400), tol=1.3e-3, max_flips=0, max_margin=0.0)
 
 
 def test_c4_sixteen_layer_q8_0_stack_prefill_256_tokens():
     # the configuration as stated: 16 layers, 256 tokens.  Layer by layer on identical inputs every element is
-    # inside 2e-3 by the reference's measure; the residual stream after 16 layers, where each layer's rounding
-    # feeds the next, is held per row (see check_stack for the unit)
-    check_stack(*run_c4(16, 256, 500, layer_tol=2e-3), tol=9e-3)
+    # inside 2e-3 by the reference's measure (layer_tol); the residual stream after 16 layers, where each layer's
+    # rounding feeds the next, is held per row (see check_stack for the unit).  Measured: 21 of 4096 routings differ
+    # (14 tokens depart, the least tied of them at a margin of 4.9e-4, 3 end on another expert set), residual stream
+    # off by 2.03e-3 of the row rms
+    check_stack(*run_c4(16, 256, 500, layer_tol=2e-3), tol=3e-3, max_flips=32, max_margin=8e-4)
 
 
 @pytest.mark.parametrize("H,I,E,k,gt", [(2048, 256, 64, 8, M.Q4_K), (512, 128, 8, 2, M.Q8_0), (1280, 128, 16, 4, M.Q5_0),

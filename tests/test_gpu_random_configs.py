@@ -81,7 +81,9 @@ def test_a_random_configuration_matches_the_oracle(seed):
     assert hits.tolist() == np.bincount(oids.reshape(-1), minlength=E).tolist(), what
     assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), what
     want, mag = orc.moe_ref_f64(banks, oids, ow, x)
-    exact_float = gt in (M.F32, M.BF16) and dt in (M.F32, M.BF16) and n < batched_from
+    # float banks on the decode kernels multiply exact f32 values of the weights (F32, BF16 and F16 alike) by the f32
+    # activations; from batched_from on the 16-bit types take the f16 matrix units, where x is rounded to halfs
+    exact_float = gt in (M.F32, M.BF16, M.F16) and dt in (M.F32, M.BF16, M.F16) and n < batched_from
     tol = 1e-5 if exact_float else 2e-3
     # (outputs 100 times smaller than the batch's typical magnitude - a token whose hidden row is all but zero - are
     # held to the tolerance against that floor, not against their own magnitude)
