@@ -126,8 +126,8 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
     const int subd = lane >> rsd.group_log2, unit0d = lane & (rsd.group - 1);
     const int down_rows_wg = kDlWaves * NITD * rsd.rows_per_it;
     const int drow0 = tile * down_rows_wg + wave * NITD * rsd.rows_per_it;
-    const size_t drow_bytes = type_row_bytes(DT, inter);
-    const uint8_t *de = down + (size_t)e * (size_t)hidden * drow_bytes;
+    const uint32_t drow_bytes = (uint32_t)type_row_bytes(DT, inter);
+    const uint8_t *de = down + (size_t)uniform_index(e) * (size_t)hidden * drow_bytes;
     RawRow<DT, 1> rd[NITD];
     auto fetch_down = [&](float after) {
         // (an offset of zero that the compiler cannot see through: the loads below wait for the value it is made of)
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
         for (int i = 0; i < NITD; i++) {
             const int row = drow0 + i * rsd.rows_per_it + subd;
             const bool ok = row < hidden;
-            load_row<DT, 1>(de + (size_t)(ok ? row : 0) * drow_bytes + zero, unit0d, rsd.units, ok, rd[i]);
+            load_row<DT, 1>(de, (uint32_t)(ok ? row : 0) * drow_bytes + zero, unit0d, rsd.units, ok, rd[i]);
         }
     };
     // (asked for behind the dots of iteration 0 / 1 / 2 / 3, one token on the OLMoE shape: 15.5 / 14.8 / 14.9 / 15.3 us per layer;

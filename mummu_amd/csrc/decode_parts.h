@@ -33,9 +33,9 @@ __device__ __forceinline__ void gate_up_tile(const uint8_t *gate, const uint8_t 
     const int rows_per_block = rows_per_wave * (blockDim.x >> 6);
     const int block_row0 = tile * rows_per_block;
     const int row0 = block_row0 + wave * rows_per_wave;
-    const size_t row_bytes = type_row_bytes(WT, hidden);
-    const uint8_t *ge = gate + (size_t)e * (size_t)inter * row_bytes;
-    const uint8_t *ue = up + (size_t)e * (size_t)inter * row_bytes;
+    const uint32_t row_bytes = (uint32_t)type_row_bytes(WT, hidden);
+    const uint8_t *ge = gate + (size_t)uniform_index(e) * (size_t)inter * row_bytes;  // (e is the same in every lane)
+    const uint8_t *ue = up + (size_t)uniform_index(e) * (size_t)inter * row_bytes;
 
     // Software pipeline over the wave's NIT row iterations: the loads of iterations i+1 and i+2
     // are in flight while iteration i is multiplied, so the integer dots run under the stream
@@ -45,8 +45,9 @@ __device__ __forceinline__ void gate_up_tile(const uint8_t *gate, const uint8_t 
     auto fetch = [&](int i) {
         const int row = row0 + i * rs.rows_per_it + sub;
         const bool ok = row < inter;
-        load_row<WT, UPL>(ge + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rg[i]);
-        load_row<WT, UPL>(ue + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, ru[i]);
+        const uint32_t row_off = (uint32_t)(ok ? row : 0) * row_bytes;
+        load_row<WT, UPL>(ge, row_off, unit0, rs.units, ok, rg[i]);
+        load_row<WT, UPL>(ue, row_off, unit0, rs.units, ok, ru[i]);
     };
     constexpr int AHEAD = NIT < 2 ? NIT : 2;
 #pragma unroll

@@ -253,8 +253,8 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_q_kernel(const uint8_t *
     const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
     const int rows_per_wave = NIT * rs.rows_per_it;
     const int row0 = (blockIdx.y * kGemvWaves + wave) * rows_per_wave;
-    const size_t row_bytes = type_row_bytes(WT, inter);
-    const uint8_t *de = down + (size_t)e * (size_t)hidden * row_bytes;
+    const uint32_t row_bytes = (uint32_t)type_row_bytes(WT, inter);
+    const uint8_t *de = down + (size_t)uniform_index(e) * (size_t)hidden * row_bytes;  // (e is the same in every lane)
     float *yrow = y + (size_t)a * (size_t)hidden;
 
     RawRow<WT, UPL> rd[NIT];
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_q_kernel(const uint8_t *
     for (int i = 0; i < NIT; i++) {
         const int row = row0 + i * rs.rows_per_it + sub;
         const bool ok = row < hidden;
-        load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i]);
+        load_row<WT, UPL>(de, (uint32_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i]);
     }
     LaneAct<UPL> la;
     load_lane_act<WT, UPL>(actq, (size_t)a, inter, unit0, rs.units, la);
@@ -379,10 +379,10 @@ __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
     LaneAct<UPL> la[KPW];
     auto fetch = [&](int step) {
         const int i = step / NIT, it = step % NIT;
-        const uint8_t *de = down + (size_t)(on_p[i] ? e_p[i] : 0) * (size_t)hidden * row_bytes;
+        const uint8_t *de = down + (size_t)uniform_index(on_p[i] ? e_p[i] : 0) * (size_t)hidden * row_bytes;
         const int row = row0 + it * rs.rows_per_it + sub;
         const bool ok = on_p[i] && row < hidden;
-        load_row<WT, UPL>(de + (size_t)(ok ? row : 0) * row_bytes, unit0, rs.units, ok, rd[i][it]);
+        load_row<WT, UPL>(de, (uint32_t)(ok ? row : 0) * (uint32_t)row_bytes, unit0, rs.units, ok, rd[i][it]);
     };
     constexpr int STEPS = KPW * NIT;
     constexpr int AHEAD = STEPS < 2 ? STEPS : 2;

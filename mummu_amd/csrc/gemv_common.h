@@ -130,8 +130,16 @@ struct RawRow<T_Q6_K, UPL> {
 
 constexpr bool is_legacy32(int t) { return t == T_Q4_0 || t == T_Q4_1 || t == T_Q5_0 || t == T_Q5_1; }
 
+// An index every lane of the wave holds the same value of, told to the compiler (a value read from LDS or passed
+// between lanes is uniform in fact, not by construction): addresses made of it and of kernel arguments stay in
+// scalar registers.
+__device__ __forceinline__ int uniform_index(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// The lane's share of the weight row that starts row_off bytes into the matrix at `base` (the same pointer in every
+// lane - see uniform_index - so that a load is a scalar base plus a 32-bit lane offset: the matrix of one expert stays
+// below 4 GB).
 template <int WT, int UPL>
-__device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int units, bool ok, RawRow<WT, UPL> &r) {
+__device__ inline void load_row(const uint8_t *base, uint32_t row_off, int unit0, int units, bool ok, RawRow<WT, UPL> &r) {
     // Every lane loads unconditionally (a lane without a unit re-reads the row's last unit, a
     // lane of a row past the matrix reads the valid row the caller passes instead): straight-line
     // loads keep the wait counts exact, so rows still in flight are not waited for early.  What
@@ -142,18 +150,18 @@ __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int
         const bool on = ok && u < units;
         const int uc = u < units ? u : units - 1;
         if constexpr (WT == T_Q4_K) {
-            const uint8_t *blk = rowp + (size_t)(uc >> 3) * 144;
+            const uint8_t *blk = base + (row_off + (uint32_t)(uc >> 3) * 144u);
             r.hdr[i] = *(const uint4 *)blk;
             r.q[i] = *(const uint4 *)(blk + 16 + (uc & 7) * 16);
             r.hdr[i].x = on ? r.hdr[i].x : 0u;  // d = dmin = 0
         } else if constexpr (WT == T_Q5_K) {
-            const uint8_t *blk = rowp + (size_t)(uc >> 3) * 176;  // 176 = 11 * 16: every piece is 16-byte aligned
+            const uint8_t *blk = base + (row_off + (uint32_t)(uc >> 3) * 176u);  // 176 = 11 * 16: every piece is 16-byte aligned
             r.hdr[i] = *(const uint4 *)blk;
             r.qh[i] = *(const uint4 *)(blk + 16 + (uc & 1) * 16);
             r.q[i] = *(const uint4 *)(blk + 48 + (uc & 7) * 16);
             r.hdr[i].x = on ? r.hdr[i].x : 0u;
         } else if constexpr (WT == T_Q6_K) {
-            const uint8_t *blk = rowp + (size_t)(uc >> 3) * 210;  // 2-byte aligned only
+            const uint8_t *blk = base + (row_off + (uint32_t)(uc >> 3) * 210u);  // 2-byte aligned only
             const int up = uc & 7;
 #pragma unroll
             for (int w = 0; w < 4; w++) {
@@ -168,7 +176,7 @@ __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int
         } else if constexpr (is_legacy32(WT)) {
             constexpr bool has_m = WT == T_Q4_1 || WT == T_Q5_1;
             constexpr bool has_h = WT == T_Q5_0 || WT == T_Q5_1;
-            const uint8_t *blk = rowp + (size_t)uc * block_bytes(WT);
+            const uint8_t *blk = base + (row_off + (uint32_t)uc * (uint32_t)block_bytes(WT));
             uint16_t db, mb = 0;
             __builtin_memcpy(&db, blk, 2);
             if constexpr (has_m) __builtin_memcpy(&mb, blk + 2, 2);
@@ -182,7 +190,7 @@ __device__ inline void load_row(const uint8_t *__restrict__ rowp, int unit0, int
 #pragma unroll
             for (int w = 0; w < 4; w++) __builtin_memcpy(&r.q[i][w], p + 4 * w, 4);
         } else {
-            const uint8_t *blk = rowp + (size_t)uc * 34;
+            const uint8_t *blk = base + (row_off + (uint32_t)uc * 34u);
             uint16_t db;
             __builtin_memcpy(&db, blk, 2);
             r.d[i] = on ? (uint32_t)db : 0u;
@@ -204,6 +212,11 @@ __device__ inline void k4_scale_min_pair(uint32_t y, uint32_t z, uint32_t w, int
     sc = c < 2 ? lo_sc : hi_sc;
     mn = c < 2 ? lo_mn : hi_mn;
 }
+
+// a . b over four signed bytes with nothing to add to: the first link of an accumulation chain.  (Written out for the
+// first word of each chain below: with the chains started from variables that hold 0 the same unrolled loop compiles
+// to a schedule that measures 7 % slower at four tokens per step.)
+__device__ __forceinline__ int sdot4_first(int a, int b) { return __builtin_amdgcn_sdot4(a, b, 0, false); }
 
 // The lane's partial of <row, activation> (formulas in the file comment).  A lane that loaded
 // nothing holds zero scales and contributes exactly 0.
@@ -228,6 +241,13 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
             for (int w = 0; w < 4; w++) {
                 int lo = (int)(q[w] & 0x0F0F0F0Fu);
                 int hi = (int)((q[w] >> 4) & 0x0F0F0F0Fu);
+                if (w == 0) {
+                    lh = sdot4_first(lo, a.xh[i][0]);
+                    ll = sdot4_first(lo, a.xl[i][0]);
+                    hh = sdot4_first(hi, a.xh[i][4]);
+                    hl = sdot4_first(hi, a.xl[i][4]);
+                    continue;
+                }
                 lh = __builtin_amdgcn_sdot4(lo, a.xh[i][w], lh, false);
                 ll = __builtin_amdgcn_sdot4(lo, a.xl[i][w], ll, false);
                 hh = __builtin_amdgcn_sdot4(hi, a.xh[i][4 + w], hh, false);
@@ -298,6 +318,13 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
             int h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
             for (int w = 0; w < 4; w++) {
+                if (w == 0) {
+                    h0 = sdot4_first((int)c0[0], a.xh[i][0]);
+                    l0 = sdot4_first((int)c0[0], a.xl[i][0]);
+                    h1 = sdot4_first((int)c1[0], a.xh[i][4]);
+                    l1 = sdot4_first((int)c1[0], a.xl[i][4]);
+                    continue;
+                }
                 h0 = __builtin_amdgcn_sdot4((int)c0[w], a.xh[i][w], h0, false);
                 l0 = __builtin_amdgcn_sdot4((int)c0[w], a.xl[i][w], l0, false);
                 h1 = __builtin_amdgcn_sdot4((int)c1[w], a.xh[i][4 + w], h1, false);
@@ -313,6 +340,13 @@ __device__ inline float dot_row(const RawRow<WT, UPL> &r, int unit0, const LaneA
             int h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
             for (int w = 0; w < 4; w++) {
+                if (w == 0) {
+                    h0 = sdot4_first((int)r.q[i][0], a.xh[i][0]);
+                    l0 = sdot4_first((int)r.q[i][0], a.xl[i][0]);
+                    h1 = sdot4_first((int)r.q[i][4], a.xh[i][4]);
+                    l1 = sdot4_first((int)r.q[i][4], a.xl[i][4]);
+                    continue;
+                }
                 h0 = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xh[i][w], h0, false);
                 l0 = __builtin_amdgcn_sdot4((int)r.q[i][w], a.xl[i][w], l0, false);
                 h1 = __builtin_amdgcn_sdot4((int)r.q[i][4 + w], a.xh[i][4 + w], h1, false);
