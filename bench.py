@@ -15,8 +15,10 @@ if that is shorter) - the serving-loop form; they start where the warm-up steps 
 `steady` adds the median and p10 / p90 of the per-layer time over >= 200 event-timed replays.
 
 Prints ONE JSON line (the contract the round driver reads), including
-  roofline      the dominant kernel against the 8 TB/s HBM peak, its duration
-                measured live with HIP events on the library's stream,
+  roofline      the dominant kernel against the 8 TB/s HBM peak: its duration is the median of the
+                event-timed graph replays per layer, less the layer's other launches (their eager
+                event-bound averages); `avg_launch_us_eager` is the kernel's own event-bound average in
+                eager launches, and `layer_frac` the whole layer's algorithmic bytes over the layer time,
   cpu_baseline  the CPU oracle (a C restatement of the reference's routed CPU path) timed on
                 this host on a bounded sample of the same workload.
 
