@@ -94,6 +94,7 @@ SIGNATURES = {
     "mummu_moe_router_exchange_state": (_I, [_P, C.POINTER(C.c_int), C.POINTER(C.c_uint64)]),
     "mummu_moe_set_layer_fusion": (_I, [_P, _I]),
     "mummu_moe_set_deferred_combine": (_I, [_P, _I]),
+    "mummu_moe_set_tile_order": (_I, [_P, _I]),
     "mummu_moe_flush": (_I, [_P]),
     "mummu_moe_check": (_I, [_P, _P]),
     "mummu_moe_last_routing": (_I, [_P, _I64, _I, _P, _P]),

@@ -61,13 +61,33 @@ static hipError_t with_bank_type(int type, F &&f) {
 #undef MUMMU_TYPE_CASE
 }
 
+// Several tokens per step, on request (ExpertBanks::tile_order): tokens that routed to the same expert read the same
+// weight rows, and the eight XCDs each have an L2 of their own, so the second read only hits if both workgroups sit
+// on one XCD at about the same time.  Workgroups go to the XCDs round-robin by linear index; with grid = (kXcds,
+// slots * tokens, ceil(tiles / kXcds)) the XCD is the row tile modulo 8 and every (token, slot) pair of a tile follows
+// its neighbour onto that XCD: whoever shares an expert shares the lines while they are in that L2 (or on their way
+// into it).  The launches then fetch the bytes of the distinct experts once (1.01x against 1.5x at eight tokens of
+// top-8 over 64 experts) in the same time at eight tokens and 1 - 6 % more at two to four (an XCD no longer walks
+// through one expert's matrix from end to end): it is for callers to whom the memory traffic matters.  A variant of
+// the kernels compiled for it, so that the plain order keeps its code as it is.
+constexpr int kXcds = 8;
+
+// The grid of that order for `pairs` = tokens (x slots) per row tile, or false: the plain grid (not asked for, one
+// token, or an extent past the limit of a grid).  x = row tile modulo 8, y = the (token, slot) pair, z = row tile / 8.
+static bool tile_order_grid(bool wanted, int tokens, int pairs, int tiles, dim3 &grid) {
+    const int z = (tiles + kXcds - 1) / kXcds;
+    if (!wanted || tokens <= 1 || pairs > 65535 || z > 65535) return false;
+    grid = dim3(kXcds, (unsigned)pairs, (unsigned)z);
+    return true;
+}
+
 // ------------------------------------------------------------------------------------------
 // gate/up, quantized banks: NIT iterations of rows_per_it rows per wave; the workgroup's
 // rows_per_block = waves*NIT*rows_per_it output rows are a whole number of 16-element
 // activation blocks, quantized for the down projection in the epilogue.
 // ------------------------------------------------------------------------------------------
 // RJN > 0: the kernel routes by itself, RJN experts per lane of the routing wave (see RouteInline).
-template <int WT, int UPL, int NIT, bool ACTQ, int RJN = 0>
+template <int WT, int UPL, int NIT, bool ACTQ, int RJN = 0, bool ORDERED = false>
 __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restrict__ gate,
                                                          const uint8_t *__restrict__ up, QAct xq,
                                                          const int32_t *__restrict__ ids, int k, int fixed_expert,
@@ -82,8 +102,17 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
     __shared__ float s_w[64];
     MUMMU_PHASE(0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.z;  // grid = (slot, row tile, token)
-    const int a = t * gridDim.x + blockIdx.x;
+    // grid = (slot, row tile, token), or ORDERED: (row tile modulo 8, token * k + slot, row tile / 8)
+    int slot = blockIdx.x, tile = blockIdx.y, t = blockIdx.z, slots = gridDim.x;
+    if constexpr (ORDERED) {
+        slots = k;
+        slot = blockIdx.y % k;
+        t = blockIdx.y / k;
+        tile = blockIdx.z * kXcds + blockIdx.x;
+        const int rows_per_block = NIT * (64 >> row_split(hidden).group_log2) * (blockDim.x >> 6);
+        if (tile * rows_per_block >= inter) return;  // (the eight columns cover a whole number of tiles or a few more)
+    }
+    const int a = t * slots + slot;
     const RowSplit rs = row_split(hidden);
     const int unit0 = lane & (rs.group - 1);
     LaneAct<UPL> la;  // the token's activations do not depend on the routing: fetch them first
@@ -96,7 +125,7 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
             for (int j = 0; j < JN; j++) l[j] = lane + 64 * j < n_experts ? route.logits[(size_t)t * n_experts + lane + 64 * j] : 0.0f;
             route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, s_ids, s_w, nullptr, flags, s_route, 0);
             wave_lds_sync();
-            if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
+            if (slot == 0 && tile == 0 && lane < k) {
                 const int id = s_ids[lane];
                 route.ids[(size_t)t * k + lane] = id;
                 route.weights[(size_t)t * k + lane] = s_w[lane];
@@ -107,12 +136,12 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
         __syncthreads();
         MUMMU_PHASE(7);
     }
-    const int e = ROUTE ? s_ids[blockIdx.x] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
+    const int e = ROUTE ? s_ids[slot] : (fixed_expert >= 0 ? fixed_expert : ids[a]);
     if ((unsigned)e >= (unsigned)n_experts) {
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
     }
-    gate_up_tile<WT, UPL, NIT, ACTQ>(gate, up, e, a, la, rs, hidden, inter, act, actq, s_act, blockIdx.y);
+    gate_up_tile<WT, UPL, NIT, ACTQ>(gate, up, e, a, la, rs, hidden, inter, act, actq, s_act, tile);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -328,22 +357,28 @@ __global__ __launch_bounds__(64 * kGemvWaves) void down_f_kernel(const uint8_t *
 // in ascending-id order, KPW each; their row sums meet in LDS and are combined in that same
 // order, multiply and add rounded separately.
 // ------------------------------------------------------------------------------------------
-template <int WT, int UPL, int NIT, int KPW, int kDcWaves = 4>
+template <int WT, int UPL, int NIT, int KPW, int kDcWaves = 4, bool ORDERED = false>
 __global__ __launch_bounds__(64 * kDcWaves) void down_combine_q_kernel(
     const uint8_t *down /* not __restrict__: the code fences below must order its loads */, QAct actq, const int32_t *__restrict__ ids, const float *__restrict__ weights,
     int k, int hidden, int inter, int n_experts, const float *__restrict__ residual, float *__restrict__ out,
     unsigned long long *epoch_bump) {
     constexpr int KMAX = kDcWaves * KPW;
     // the launch before this one (gate_up_fused_kernel) has finished with the epoch: move it on for the next
-    if (epoch_bump != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *epoch_bump = *epoch_bump + 1ULL;
+    if (epoch_bump != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && (!ORDERED || blockIdx.z == 0) && threadIdx.x == 0) *epoch_bump = *epoch_bump + 1ULL;
     extern __shared__ float s_mem[];  // [KMAX][rows_per_block] row sums, then [KMAX] weights
     MUMMU_PHASE(0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.x;
+    // grid = (token, row tile), or ORDERED: (row tile modulo 8, token, row tile / 8)
+    int t = blockIdx.x, tile = blockIdx.y;
+    if constexpr (ORDERED) {
+        t = blockIdx.y;
+        tile = blockIdx.z * kXcds + blockIdx.x;
+    }
     const RowSplit rs = row_split(inter);
     const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
     const int rows_per_block = NIT * rs.rows_per_it;
-    const int row0 = blockIdx.y * rows_per_block;
+    const int row0 = tile * rows_per_block;
+    if (ORDERED && row0 >= hidden) return;  // (the eight columns cover a whole number of tiles or a few more)
     float *s_y = s_mem;
     float *s_w = s_mem + KMAX * rows_per_block;
     const size_t row_bytes = type_row_bytes(WT, inter);
@@ -452,9 +487,14 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         int waves = 4;                                                                                          \
         while (waves * (NIT)*rs.rows_per_it < 16) waves *= 2; /* whole 16-element activation blocks */          \
         const int rpb = waves * (NIT)*rs.rows_per_it;                                                           \
-        dim3 grid(slots, (b.inter + rpb - 1) / rpb, n_assign / slots), block(64 * waves);                                      \
+        const int tiles = (b.inter + rpb - 1) / rpb, tokens = n_assign / slots;                                 \
+        dim3 grid(slots, tiles, tokens), block(64 * waves);                                                     \
+        const bool ordered = tile_order_grid(b.tile_order && fixed_expert < 0 && actq_out, tokens, slots * tokens, tiles, grid); \
         const size_t lds = sizeof(float) * (size_t)rpb;                                                         \
-        if (actq_out)                                                                                           \
+        if (ordered)                                                                                            \
+            launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true, 0, true>, grid, block, lds, s,                              \
+                b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags, RouteInline());      \
+        else if (actq_out)                                                                                      \
             launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true>, grid, block, lds, s,                                       \
                 b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags, RouteInline());      \
         else                                                                                                    \
@@ -635,11 +675,19 @@ static hipError_t launch_gate_up_routed_t(const ExpertBanks &b, QAct xq, const R
     int waves = 4;
     while (waves * NIT * rs.rows_per_it < 16) waves *= 2;
     const int rpb = waves * NIT * rs.rows_per_it;
-    dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(64 * waves);
+    const int tiles = (b.inter + rpb - 1) / rpb;
+    dim3 grid(k, tiles, n_tokens), block(64 * waves);
+    const bool ordered = tile_order_grid(b.tile_order, n_tokens, k * n_tokens, tiles, grid);
     const size_t lds = sizeof(float) * (size_t)rpb;
 #define MUMMU_GUR(JN)                                                                                                    \
-    launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true, JN>, grid, block, lds, s, b.gate, b.up, xq, (const int32_t *)nullptr, \
-                  k, -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route)
+    do {                                                                                                                 \
+        if (ordered)                                                                                                     \
+            launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true, JN, true>, grid, block, lds, s, b.gate, b.up, xq,         \
+                          (const int32_t *)nullptr, k, -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route); \
+        else                                                                                                             \
+            launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true, JN>, grid, block, lds, s, b.gate, b.up, xq,               \
+                          (const int32_t *)nullptr, k, -1, b.hidden, b.inter, b.n_experts, (float *)nullptr, actq, flags, route); \
+    } while (0)
     if (b.n_experts <= 64) MUMMU_GUR(1);
     else if (b.n_experts <= 128) MUMMU_GUR(2);
     else MUMMU_GUR(8);
@@ -760,10 +808,16 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
 #define MUMMU_DC(UPL, NIT, KPW, WAVES)                                                                             \
     do {                                                                                                           \
         const int rpb = (NIT)*rs.rows_per_it;                                                                      \
-        dim3 grid(n, (b.hidden + rpb - 1) / rpb), block(64 * (WAVES));                                             \
+        const int tiles = (b.hidden + rpb - 1) / rpb;                                                              \
+        dim3 grid(n, tiles), block(64 * (WAVES));                                                                  \
+        const bool ordered = tile_order_grid(b.tile_order, n, n, tiles, grid);                                     \
         const size_t lds = sizeof(float) * (size_t)((WAVES) * (KPW)) * (size_t)(rpb + 1);                          \
-        launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW, WAVES>, grid, block, lds, s, b.down, actq, ids, weights, k, \
-                      b.hidden, b.inter, b.n_experts, residual, out, epoch_bump);                                  \
+        if (ordered)                                                                                               \
+            launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW, WAVES, true>, grid, block, lds, s, b.down, actq, ids, weights, k, \
+                          b.hidden, b.inter, b.n_experts, residual, out, epoch_bump);                              \
+        else                                                                                                       \
+            launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW, WAVES>, grid, block, lds, s, b.down, actq, ids, weights, k, \
+                          b.hidden, b.inter, b.n_experts, residual, out, epoch_bump);                              \
     } while (0)
     // one expert per wave up to top_k 8 (eight waves, four row iterations each: measured against two experts per wave
     // in four waves and against one / two / six / eight iterations, 5.4 against 5.8 us at one token and 18.0

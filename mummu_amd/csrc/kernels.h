@@ -50,6 +50,7 @@ struct ExpertBanks {
     int gate_type, up_type, down_type;
     int hidden, inter, n_experts;
     bool q8_half_ok = false;          // Q8_0 banks whose every |d| * 128 is inside the half range (launch_q8_scale_max)
+    bool tile_order = false;          // decode launches of several tokens: workgroups ordered so that tokens sharing an expert meet in one XCD's L2
 };
 
 

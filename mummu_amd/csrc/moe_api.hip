@@ -120,6 +120,7 @@ struct mummu_moe {
     // and a counter that tells launches apart which read the same epoch (the nodes of one captured graph)
     void *aslots = nullptr;
     int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
+    int tile_order = 0;        // decode launches of several tokens fetch a shared expert's rows once (mummu_moe_set_tile_order)
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
     // off by default), whose otherwise idle waves do it: the one-launch form then costs one launch per step.  The per-slot
@@ -477,6 +478,7 @@ ExpertBanks banks_of(const mummu_moe *h, const Layer &L) {
     b.inter = h->cfg.expert_intermediate_size;
     b.n_experts = h->cfg.num_experts;
     b.q8_half_ok = L.q8_half_ok;
+    b.tile_order = h->tile_order != 0;
     return b;
 }
 
@@ -1073,6 +1075,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
         if (const char *e = getenv("MUMMU_ROUTER_EXCHANGE")) h->router_exchange = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
         if (const char *e = getenv("MUMMU_LAYER_FUSION")) h->layer_fusion = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
         if (const char *e = getenv("MUMMU_DEFERRED_COMBINE")) h->deferred_combine = atoi(e) != 0;
+        if (const char *e = getenv("MUMMU_TILE_ORDER")) h->tile_order = atoi(e) != 0;
     }
     {
         // resolve the static scratch's address on this device now, outside any stream capture
@@ -1751,6 +1754,14 @@ int mummu_moe_set_deferred_combine(mummu_moe *h, int enable) {
     Entry entry(h);
     if (entry.rc) return entry.rc;
     h->deferred_combine = enable != 0;
+    return MUMMU_OK;
+}
+
+int mummu_moe_set_tile_order(mummu_moe *h, int enable) {
+    if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
+    Entry entry(h);
+    if (entry.rc) return entry.rc;
+    h->tile_order = enable != 0;
     return MUMMU_OK;
 }
 

@@ -320,6 +320,11 @@ class SparseMoe:
         forward_device call (off by default).  out of a call is complete after the next call, flush() or check()."""
         self._check(self._lib.mummu_moe_set_deferred_combine(self._h, int(bool(enable))))
 
+    def set_tile_order(self, enable):
+        """Decode steps of several tokens fetch the rows of an expert that several tokens share once (off by default:
+        a third less HBM traffic at eight tokens in the same time, 1 - 6 % more time at two to four).  Same bits either way."""
+        self._check(self._lib.mummu_moe_set_tile_order(self._h, int(bool(enable))))
+
     def flush(self):
         """Enqueues the sum a deferred decode step left pending; does not synchronise."""
         self._check(self._lib.mummu_moe_flush(self._h))
