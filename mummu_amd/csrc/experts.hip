@@ -501,7 +501,8 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
             launch_kernel(gate_up_q_kernel<WT, UPL, NIT, false>, grid, block, lds, s,                                      \
                 b.gate, b.up, xq, ids, k, fixed_expert, b.hidden, b.inter, b.n_experts, act, actq, flags, RouteInline());      \
     } while (0)
-        if (upl == 1) MUMMU_GUQ(1, 4);
+        if (upl == 1 && n_assign / slots >= 8 && fixed_expert < 0 && b.inter % 32 == 0) MUMMU_GUQ(1, 8);  // (as launch_gate_up_routed)
+        else if (upl == 1) MUMMU_GUQ(1, 4);
         else if (upl == 2) MUMMU_GUQ(2, 2);
         else if (upl <= 4) MUMMU_GUQ(4, 1);
         else return hipErrorInvalidValue;
@@ -703,6 +704,9 @@ hipError_t launch_gate_up_routed(const ExpertBanks &b, QAct xq, const RouteInlin
     return with_bank_type(b.gate_type, [&](auto tag) {
         constexpr int WT = decltype(tag)::value;
         if constexpr (is_quant_type(WT)) {
+            // (eight row iterations per wave from eight tokens on: the same routing and activation loads serve twice the
+            // rows - 29.3 against 30.0 us at 8 tokens of the OLMoE shape, but 12.7 against 11.8 at 2)
+            if (!wide && n_tokens >= 8 && b.inter % 32 == 0) return launch_gate_up_routed_t<WT, 1, 8>(b, xq, route, n_tokens, k, actq, flags, s);
             return wide ? launch_gate_up_routed_t<WT, 2, 2>(b, xq, route, n_tokens, k, actq, flags, s)
                         : launch_gate_up_routed_t<WT, 1, 4>(b, xq, route, n_tokens, k, actq, flags, s);
         } else {
@@ -824,6 +828,7 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
     // against 23.0 us at eight), two per wave beyond
     if (upl == 1) {
         if (k <= 4) MUMMU_DC(1, 4, 1, 4);
+        else if (k <= 8 && n >= 3) MUMMU_DC(1, 8, 1, 8);  // (several tokens: 9.5 against 11.0 us at 4 tokens, 16.2 against 17.9 at 8; 6.1 against 5.4 at one)
         else if (k <= 8) MUMMU_DC(1, 4, 1, 8);
         else if (k <= 10) MUMMU_DC(1, 2, 2, 5);  // (ten waves of one expert: 8.7 against 7.7 us at one token, top-10 of 512)
         else if (k <= 12) MUMMU_DC(1, 2, 2, 6);
