@@ -261,11 +261,15 @@ MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_
  * along: mummu_moe_set_deferred_combine.  No counterpart in the reference.  Same bits as the other forms; the same
  * spin_ticks bounds its waits, and a workgroup that gives up computes the hidden blocks it misses itself (counted by
  * _state's fallbacks).  enable = 0: never; 1 (default): in chains of deferred sums only; 2: wherever the kernel serves
- * (every decode call of up to 8 tokens when mummu_moe_set_router_exchange says 2).  Environment: MUMMU_LAYER_FUSION. */
+ * (every decode call of up to 8 tokens when mummu_moe_set_router_exchange says 2).  Environment: MUMMU_LAYER_FUSION.
+ * With at most 64 experts the launch starts every slot's rows on the expert whose logit has the slot's rank and confirms
+ * that pick against the routing proper while the rows are on their way; a slot the routing names differently (two
+ * logits whose probabilities round to the same float) is done again inside the launch: the same routing and the same
+ * bits (MUMMU_EARLY_IDS=0 at mummu_moe_create: route first). */
 MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
 /* enable = 1 (default 0): a mummu_moe_forward_device call that can take the one-launch form no longer enqueues the sum over
  * each token's eight weighted rows; the launch of the NEXT such call on the same stream does it on the side (a wave per
- * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (14.9 us
+ * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (14.4 us
  * per layer on the OLMoE shape).  out_dev of a call is then complete once the next call's work, or mummu_moe_flush, has
  * run on the stream; every other entry point of the handle, mummu_graph_begin / _end and mummu_moe_check enqueue a
  * pending sum first, so a captured graph always ends with its last step's sum and a caller that reads out_dev after

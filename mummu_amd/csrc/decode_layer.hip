@@ -12,6 +12,13 @@
 // one exchange inside an L2 instead of a launch, and its weight stream hides behind the wait for the slowest
 // workgroup.  Nothing crosses XCDs inside the launch: every slot leaves its own row of down sums in y.
 //
+// EARLY (at most 64 experts): the workgroups do not wait for the routing.  Wave 0 stops at the eight largest LOGITS,
+// the workgroup starts its rows on the expert of its slot's rank, and wave 0 confirms the pick behind its first row
+// loads - the softmax, then a check that rounds on the probabilities would choose the same experts in the same order
+// (route_token_checked8), with the rounds themselves only where the check fails.  A slot whose expert the routing then
+// names differently (probabilities that tie or cross where the logits do not: the tie goes to the lower id) does its
+// rows again for that expert, in every workgroup of the slot alike.  Same bits as routing first.
+//
 // Every wait is bounded (spin_ticks of the 100 MHz clock).  A workgroup that does not find a block - workgroups
 // placed otherwise than assumed, not all resident at once, or a tiny bound set by a test - computes that block's
 // gate/up rows itself with the same code: the same bits, only slower.
@@ -79,7 +86,7 @@ __device__ __forceinline__ void quantize_tile_to_lds(const float *s_act, int row
 
 constexpr int kDlWaves = 4;  // waves per workgroup (eight, in half as many workgroups, measured the same: 14.9 us per layer)
 
-template <int WT, int DT, int NITD, int RJN>
+template <int WT, int DT, int NITD, int RJN, bool EARLY>
 // (the three banks are not __restrict__: the code fences between the row loads must order them - gate/up rows first,
 // the down rows behind them - and the compiler moves loads of restrict pointers across such a fence as it likes)
 __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8_t *gate, const uint8_t *up, const uint8_t *down,
@@ -110,11 +117,13 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
         if (ps.n > 0 && wave == 1)
             pending_sum_wave(ps, hidden, (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x, gridDim.x * gridDim.y * gridDim.z);
     };
-    const unsigned long long epoch =
-        decode_route_prologue<RJN>(k, hidden, n_experts, flags, route, rx, sh, s_xhi, s_xlo, s_xscale, s_xsum, side_work);
+    RouteCarry<RJN> carry;
+    const unsigned long long epoch = decode_route_prologue<RJN, decltype(side_work), EARLY>(k, hidden, n_experts, flags, route, rx, sh, s_xhi, s_xlo,
+                                                                                            s_xscale, s_xsum, side_work, &carry);
     LaneAct<1> la;
     load_lane_act_lds<WT>(s_xhi, s_xlo, s_xscale, s_xsum, unit0, rs.units, la);
-    const int e = sh.ids[slot];
+    // EARLY: the slot's expert by the rank of its logit, the routing proper still to come (route_rest, below)
+    int e = EARLY ? sh.early_ids[slot] : sh.ids[slot];
     if ((unsigned)e >= (unsigned)n_experts) {  // (the same for every workgroup of the slot: nobody waits for this one)
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
@@ -142,8 +151,30 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
     };
     // (asked for behind the dots of iteration 0 / 1 / 2 / 3, one token on the OLMoE shape: 15.5 / 14.8 / 14.9 / 15.3 us per layer;
     // together with the gate/up rows, which is where the compiler puts every load it is free to move: 15.0)
-    gate_up_tile<WT, 1, NIT, true, false, decltype(fetch_down), 1>(gate, up, e, a, la, rs, hidden, inter, nullptr, QAct(), s_act, tile, fetch_down);
-    __syncthreads();
+    if constexpr (EARLY) {
+        // wave 0 routes while the first rows of its share are on their way
+        auto route_rest = [&]() {
+            if (wave == 0) decode_route_finish<RJN, true>(carry.l, k, n_experts, flags, route, rx, sh);
+        };
+        gate_up_tile<WT, 1, NIT, true, false, decltype(fetch_down), 1, decltype(route_rest)>(gate, up, e, a, la, rs, hidden, inter, nullptr, QAct(),
+                                                                                             s_act, tile, fetch_down, route_rest);
+        __syncthreads();
+        if (sh.ids[slot] != e) {
+            // the routing gives this slot another expert than its logit's rank did (the same finding in every workgroup of
+            // the slot): the rows again, for that one
+            e = sh.ids[slot];
+            if ((unsigned)e >= (unsigned)n_experts) {
+                if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
+                return;
+            }
+            de = down + (size_t)uniform_index(e) * (size_t)hidden * drow_bytes;
+            gate_up_tile<WT, 1, NIT, true, false, decltype(fetch_down), 1>(gate, up, e, a, la, rs, hidden, inter, nullptr, QAct(), s_act, tile, fetch_down);
+            __syncthreads();
+        }
+    } else {
+        gate_up_tile<WT, 1, NIT, true, false, decltype(fetch_down), 1>(gate, up, e, a, la, rs, hidden, inter, nullptr, QAct(), s_act, tile, fetch_down);
+        __syncthreads();
+    }
     MUMMU_PHASE(4);
 
     // this tile's blocks: into the LDS copy of the slot's hidden row, and out to the XCD's table
@@ -252,7 +283,7 @@ bool decode_layer_supported(const ExpertBanks &b, int k, int n_tokens, const Rou
     return decode_layer_down_iters(b) <= 8;
 }
 
-template <int WT, int DT, int NITD>
+template <int WT, int DT, int NITD, bool EARLY>
 static hipError_t launch_decode_layer_t(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
                                         int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
     const RowSplit rs = row_split(b.hidden);
@@ -261,44 +292,51 @@ static hipError_t launch_decode_layer_t(const ExpertBanks &b, const RouterExchan
     const size_t lds = sizeof(float) * (size_t)rpb + 2 * (size_t)b.hidden + 8 * (size_t)(b.hidden / 16) + 2 * (size_t)b.inter +
                        8 * (size_t)(b.inter / 16);
     if (b.n_experts <= 64)
-        launch_kernel(decode_layer_kernel<WT, DT, NITD, 1>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter, b.n_experts,
-                      flags, route, rx, lx, ps);
-    else
-        launch_kernel(decode_layer_kernel<WT, DT, NITD, 2>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter, b.n_experts,
-                      flags, route, rx, lx, ps);
+        launch_kernel(decode_layer_kernel<WT, DT, NITD, 1, EARLY>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter,
+                      b.n_experts, flags, route, rx, lx, ps);
+    else  // (two experts per routing lane: the early pick is written for one)
+        launch_kernel(decode_layer_kernel<WT, DT, NITD, 2, false>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter,
+                      b.n_experts, flags, route, rx, lx, ps);
     return hipGetLastError();
 }
 
-template <int WT, int DT>
+template <int WT, int DT, bool EARLY>
 static hipError_t launch_decode_layer_d(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
                                         int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
-    return decode_layer_down_iters(b) <= 4 ? launch_decode_layer_t<WT, DT, 4>(b, rx, lx, route, n_tokens, k, flags, s, ps)
-                                           : launch_decode_layer_t<WT, DT, 8>(b, rx, lx, route, n_tokens, k, flags, s, ps);
+    return decode_layer_down_iters(b) <= 4 ? launch_decode_layer_t<WT, DT, 4, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps)
+                                           : launch_decode_layer_t<WT, DT, 8, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps);
 }
 
-template <int WT>
+template <int WT, bool EARLY>
 static hipError_t launch_decode_layer_w(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
                                         int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
     switch (b.down_type) {
-    case T_Q4_K: return launch_decode_layer_d<WT, T_Q4_K>(b, rx, lx, route, n_tokens, k, flags, s, ps);
-    case T_Q8_0: return launch_decode_layer_d<WT, T_Q8_0>(b, rx, lx, route, n_tokens, k, flags, s, ps);
-    case T_Q6_K: return launch_decode_layer_d<WT, T_Q6_K>(b, rx, lx, route, n_tokens, k, flags, s, ps);
+    case T_Q4_K: return launch_decode_layer_d<WT, T_Q4_K, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps);
+    case T_Q8_0: return launch_decode_layer_d<WT, T_Q8_0, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps);
+    case T_Q6_K: return launch_decode_layer_d<WT, T_Q6_K, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <bool EARLY>
+static hipError_t launch_decode_layer_e(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
+                                        int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
+    switch (b.gate_type) {
+    case T_Q4_K: return launch_decode_layer_w<T_Q4_K, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps);
+    case T_Q8_0: return launch_decode_layer_w<T_Q8_0, EARLY>(b, rx, lx, route, n_tokens, k, flags, s, ps);
     default: return hipErrorInvalidValue;
     }
 }
 
 hipError_t launch_decode_layer(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
-                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
+                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps, bool early_ids) {
     if (n_tokens <= 0) return hipSuccess;
     if (!decode_layer_supported(b, k, n_tokens, rx, lx)) return hipErrorInvalidValue;
     if (ps.n > 0 && (b.hidden % 256 != 0 || ps.y == nullptr || ps.ids == nullptr || ps.weights == nullptr || ps.out == nullptr ||
                      (((uintptr_t)ps.y | (uintptr_t)ps.residual | (uintptr_t)ps.out) & 15) != 0))
         return hipErrorInvalidValue;
-    switch (b.gate_type) {
-    case T_Q4_K: return launch_decode_layer_w<T_Q4_K>(b, rx, lx, route, n_tokens, k, flags, s, ps);
-    case T_Q8_0: return launch_decode_layer_w<T_Q8_0>(b, rx, lx, route, n_tokens, k, flags, s, ps);
-    default: return hipErrorInvalidValue;
-    }
+    return early_ids ? launch_decode_layer_e<true>(b, rx, lx, route, n_tokens, k, flags, s, ps)
+                     : launch_decode_layer_e<false>(b, rx, lx, route, n_tokens, k, flags, s, ps);
 }
 
 }  // namespace mummu

@@ -8,6 +8,8 @@
 #include "gemv_common.h"
 #include "route_common.h"
 
+#include <type_traits>
+
 namespace mummu {
 
 struct NoHook {
@@ -22,11 +24,12 @@ struct NoHook {
 // goes on after a barrier of its own.  `hook` runs behind the dots of iteration HOOK_AT and is handed one of their
 // results: loads whose address it makes depend on that value cannot be asked for before the rows of that iteration have
 // arrived (the compiler hoists every independent load to the top of the function, whatever fences lie between).
-template <int WT, int UPL, int NIT, bool ACTQ, bool STORE = true, typename Hook = NoHook, int HOOK_AT = NIT - 1>
+// `first` runs once the rows of the first iterations have been asked for, in front of every dot.
+template <int WT, int UPL, int NIT, bool ACTQ, bool STORE = true, typename Hook = NoHook, int HOOK_AT = NIT - 1, typename First = NoHook>
 __device__ __forceinline__ void gate_up_tile(const uint8_t *gate, const uint8_t *up /* (restrict or not is the kernel's choice) */, int e, int a,
                                              const LaneAct<UPL> &la, const RowSplit &rs, int hidden, int inter,
                                              float *__restrict__ act, const QAct &actq, float *s_act, int tile,
-                                             Hook hook = Hook()) {
+                                             Hook hook = Hook(), First first = First()) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane >> rs.group_log2, unit0 = lane & (rs.group - 1);
     const int rows_per_wave = NIT * rs.rows_per_it;
@@ -54,6 +57,10 @@ __device__ __forceinline__ void gate_up_tile(const uint8_t *gate, const uint8_t 
     for (int i = 0; i < AHEAD; i++) fetch(i);
     MUMMU_CODE_FENCE();
     MUMMU_PHASE(1);
+    if constexpr (!std::is_same<First, NoHook>::value) {
+        first();
+        MUMMU_CODE_FENCE();
+    }
     float part[2 * NIT];
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
@@ -273,7 +280,118 @@ struct DecodeShared {
     RouteScratch<JN> route;
     int ids[64];
     float w[64];
+    int early_ids[8];  // (EARLY prologue: the eight largest logits, slot order, before the routing proper has run)
 };
+
+// What wave 0 of a workgroup carries from the first half of the routing (the logits are in) to the second.
+template <int JN>
+struct RouteCarry {
+    float l[JN];
+};
+
+// A finite float as an integer that orders the same way (-0 below +0).
+__device__ __forceinline__ int float_order_key(float v) {
+    const int b = __float_as_int(v);
+    return b ^ ((b >> 31) & 0x7FFFFFFF);
+}
+
+// route_token for one expert per lane and k = 8 when the eight winners are believed known (early[0..8), slot order: the
+// eight largest logits): the softmax as route_token computes it, then a CHECK that the rounds on the probabilities would
+// pick exactly these experts in exactly this order - every slot's probability above the next one's, or equal to it with
+// the lower id, and nobody outside as good as the last - instead of the rounds themselves (eight dependent wave
+// maxima), and the renormaliser summed in slot order as the rounds would have.  True: ids / weights written, the bits
+// of route_token.  False (probabilities that tie or cross where the logits do not, a logit that is not finite):
+// nothing written, the caller runs route_token.
+__device__ __forceinline__ bool route_token_checked8(float l, int n_experts, int flavour, int norm, const int *early, int32_t *ids,
+                                                     float *weights, RouteScratch<1> &sc) {
+    const int lane = threadIdx.x & 63;
+    const bool real = lane < n_experts;
+    if (__any(real && !(fabsf(l) <= 3.402823466e38f))) return false;
+    const float mx = wave_max(real ? l : -__builtin_inff());
+    float p = real ? det_expf(__fsub_rn(l, mx)) : 0.0f;
+    sc.p[lane] = p;
+    wave_lds_sync();
+    const float4 *bp = (const float4 *)sc.p;
+    if (flavour == 0) {
+        float total = 0.0f;
+#pragma unroll 16
+        for (int c = 0; c < 16; c++) {
+            const float4 v = bp[c];
+            total = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(total, v.x), v.y), v.z), v.w);
+        }
+        p = __fdiv_rn(p, total);
+    } else {
+        double total = 0.0;
+#pragma unroll 16
+        for (int c = 0; c < 16; c++) {
+            const float4 v = bp[c];
+            total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
+        }
+        p = __fmul_rn(p, (float)__ddiv_rn(1.0, total));
+    }
+    int eid[8];
+    float ps[8];
+    int my_slot = -1;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        eid[s] = __builtin_amdgcn_readfirstlane(early[s]);
+        ps[s] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), eid[s]));
+        my_slot = lane == eid[s] ? s : my_slot;
+    }
+    bool ok = true;
+#pragma unroll
+    for (int s = 0; s < 7; s++) ok = ok && (ps[s] > ps[s + 1] || (ps[s] == ps[s + 1] && eid[s] < eid[s + 1]));
+    const bool beats_last = real && my_slot < 0 && (p > ps[7] || (p == ps[7] && lane < eid[7]));
+    if (!ok || __any(beats_last)) return false;
+    float sum32 = 0.0f;
+    double sum64 = 0.0;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        sum32 = __fadd_rn(sum32, ps[s]);
+        sum64 = __dadd_rn(sum64, (double)ps[s]);
+    }
+    float denom = 1.0f;
+    if (flavour == 0) {
+        if (norm) denom = sum32;
+    } else {
+        const float fs = (float)sum64;
+        const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
+        denom = fs > floor_v ? fs : floor_v;
+    }
+    if (my_slot >= 0) {
+        float wv = p;
+        if (flavour != 0 || norm) wv = __fdiv_rn(wv, denom);
+        ids[my_slot] = lane;
+        weights[my_slot] = wv;
+    }
+    return true;
+}
+
+// Second half of wave 0's routing in the prologue below: the token's logits l -> sh.ids / sh.w in slot order, and, from
+// one workgroup per token, the routing, the logits and the hit counters in global memory.  CHECKED: sh.early_ids holds
+// the prologue's early pick, which is confirmed where it can be instead of the rounds being run.
+template <int JN, bool CHECKED = false>
+__device__ __forceinline__ void decode_route_finish(float (&l)[JN], int k, int n_experts, int32_t *__restrict__ flags,
+                                                    const RouteInline &route, const RouterExchange &rx, DecodeShared<JN> &sh) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.z;
+    if (rx.logits_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
+#pragma unroll
+        for (int j = 0; j < JN; j++)
+            if (lane + 64 * j < n_experts) rx.logits_out[(size_t)t * n_experts + lane + 64 * j] = l[j];
+    }
+    bool routed = false;
+    if constexpr (CHECKED && JN == 1) routed = route_token_checked8(l[0], n_experts, route.flavour, route.norm, sh.early_ids, sh.ids, sh.w, sh.route);
+    if (!routed) route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, sh.ids, sh.w, nullptr, flags, sh.route, 0);
+    wave_lds_sync();
+    if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
+        const int id = sh.ids[lane];
+        route.ids[(size_t)t * k + lane] = id;
+        route.weights[(size_t)t * k + lane] = sh.w[lane];
+        if (route.hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&route.hits[id], 1ULL);
+    }
+    MUMMU_PHASE(11);
+}
 
 // ------------------------------------------------------------------------------------------
 // Prologue of the decode kernels that route by themselves (grid = (slot, row tile, token), four waves per
@@ -293,11 +411,20 @@ struct DecodeShared {
 // routing in slot order and the LDS row is complete.  `idle` is called by waves 1.. of the workgroup while wave 0
 // routes (they have nothing else to do until the barrier).
 // ------------------------------------------------------------------------------------------
-template <int JN, typename Idle = NoHook>
+//
+// EARLY (one expert per routing lane, k = 8): wave 0 stops once it has the logits and the eight LARGEST OF THEM in
+// sh.early_ids - the experts the routing will pick wherever the probabilities order like the logits, which softmax all
+// but guarantees - and the workgroup goes on with those; wave 0 runs the routing proper later, through
+// decode_route_finish, behind its first row loads (the softmax, the rounds on probabilities and the renormalisation are
+// some 350 dependent instructions that no expert byte had been asked for until now).  The caller compares sh.ids with
+// what it started on and starts over where they differ (two logits whose probabilities round to the same float, or
+// cross: a tie goes to the lower id, not to the larger logit).
+template <int JN, typename Idle = NoHook, bool EARLY = false>
 __device__ __forceinline__ unsigned long long decode_route_prologue(int k, int hidden, int n_experts, int32_t *__restrict__ flags,
                                                                     const RouteInline &route, const RouterExchange &rx,
                                                                     DecodeShared<JN> &sh, int8_t *s_xhi, int8_t *s_xlo,
-                                                                    float *s_xscale, int *s_xsum, Idle idle = Idle()) {
+                                                                    float *s_xscale, int *s_xsum, Idle idle = Idle(),
+                                                                    RouteCarry<JN> *carry = nullptr) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.z;
 
@@ -443,20 +570,23 @@ __device__ __forceinline__ unsigned long long decode_route_prologue(int k, int h
                 }
             }
         }
-        if (rx.logits_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
+        if constexpr (EARLY) {
+            static_assert(JN == 1, "one expert per routing lane");
+            int cand = lane < n_experts ? float_order_key(l[0]) : (int)0x80000000;
 #pragma unroll
-            for (int j = 0; j < JN; j++)
-                if (lane + 64 * j < n_experts) rx.logits_out[(size_t)t * n_experts + lane + 64 * j] = l[j];
+            for (int s = 0; s < 8; s++) {
+                const int best = wave_max_i32(cand);
+                const int win = (int)__builtin_ctzll(__ballot(cand == best));  // lowest expert id holding the maximum
+                if (lane == win) {
+                    sh.early_ids[s] = lane;
+                    cand = (int)0x80000000;
+                }
+            }
+            carry->l[0] = l[0];
+            MUMMU_PHASE(11);
+        } else {
+            decode_route_finish<JN>(l, k, n_experts, flags, route, rx, sh);
         }
-        route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, sh.ids, sh.w, nullptr, flags, sh.route, 0);
-        wave_lds_sync();
-        if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
-            const int id = sh.ids[lane];
-            route.ids[(size_t)t * k + lane] = id;
-            route.weights[(size_t)t * k + lane] = sh.w[lane];
-            if (route.hits && (unsigned)id < (unsigned)n_experts) atomicAdd(&route.hits[id], 1ULL);
-        }
-        MUMMU_PHASE(11);
     } else {
         idle();
     }

@@ -123,7 +123,8 @@ struct PendingSum {
 inline size_t layer_exchange_bytes() { return (size_t)kExchangeXcds * kExchangeTokens * 8 * (size_t)kActBlocksMax * 64; }
 bool decode_layer_supported(const ExpertBanks &b, int k, int n_tokens, const RouterExchange &rx, const LayerExchange &lx);
 hipError_t launch_decode_layer(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
-                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &pending = PendingSum());
+                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &pending = PendingSum(),
+                               bool early_ids = true);
 // The same pair for float banks (F32 / F16 / BF16 gate/up and down, at most 512 experts, top_k <= 16):
 // gate/up with the routing inside writes act [n*k, inter] f32, then down + combine in one launch.
 bool float_decode_fused(const ExpertBanks &b, int k);

@@ -120,6 +120,7 @@ struct mummu_moe {
     // and a counter that tells launches apart which read the same epoch (the nodes of one captured graph)
     void *aslots = nullptr;
     int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
+    int early_ids = 1;         // the one-launch form starts its rows on the eight largest logits and confirms them (MUMMU_EARLY_IDS=0: routes first)
     int tile_order = 0;        // decode launches of several tokens fetch a shared expert's rows once (mummu_moe_set_tile_order)
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
@@ -712,7 +713,7 @@ int decode_one_launch(mummu_moe *h, const Layer &L, const DecodeScratch &ws, con
     lx.y = db.y;
     route.ids = db.ids;
     route.weights = db.weights;
-    LAUNCH(h, K_DECODE_LAYER, s, launch_decode_layer(b, rx, lx, route, n, k, h->flags, s, ps));
+    LAUNCH(h, K_DECODE_LAYER, s, launch_decode_layer(b, rx, lx, route, n, k, h->flags, s, ps, h->early_ids != 0));
     h->pending.active = false;
     h->routing_buf = buf;
     if (chain) {
@@ -1076,6 +1077,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
         if (const char *e = getenv("MUMMU_LAYER_FUSION")) h->layer_fusion = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
         if (const char *e = getenv("MUMMU_DEFERRED_COMBINE")) h->deferred_combine = atoi(e) != 0;
         if (const char *e = getenv("MUMMU_TILE_ORDER")) h->tile_order = atoi(e) != 0;
+        if (const char *e = getenv("MUMMU_EARLY_IDS")) h->early_ids = atoi(e) != 0;
     }
     {
         // resolve the static scratch's address on this device now, outside any stream capture
