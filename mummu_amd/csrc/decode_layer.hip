@@ -329,13 +329,13 @@ static hipError_t launch_decode_layer_e(const ExpertBanks &b, const RouterExchan
 }
 
 hipError_t launch_decode_layer(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
-                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps, bool early_ids) {
+                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &ps) {
     if (n_tokens <= 0) return hipSuccess;
     if (!decode_layer_supported(b, k, n_tokens, rx, lx)) return hipErrorInvalidValue;
     if (ps.n > 0 && (b.hidden % 256 != 0 || ps.y == nullptr || ps.ids == nullptr || ps.weights == nullptr || ps.out == nullptr ||
                      (((uintptr_t)ps.y | (uintptr_t)ps.residual | (uintptr_t)ps.out) & 15) != 0))
         return hipErrorInvalidValue;
-    return early_ids ? launch_decode_layer_e<true>(b, rx, lx, route, n_tokens, k, flags, s, ps)
+    return b.early_ids ? launch_decode_layer_e<true>(b, rx, lx, route, n_tokens, k, flags, s, ps)
                      : launch_decode_layer_e<false>(b, rx, lx, route, n_tokens, k, flags, s, ps);
 }
 

@@ -152,14 +152,16 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
 // leave the token's 16-bit row in LDS) is followed by the workgroup's tile of gate/up rows.  The epoch of the
 // exchange is incremented by the launch after this one (down_combine).
 // hidden <= 2048 and a multiple of 64; (slots * row tiles) a multiple of 8.
+// EARLY (k = 8, one expert per routing lane): the rows start on the expert whose logit has the slot's rank; wave 0 confirms
+// the pick behind its first row loads and a slot the routing names differently is done again (see decode_route_prologue).
 // ------------------------------------------------------------------------------------------
-template <int WT, int NIT, int RJN>
+template <int WT, int NIT, int RJN, bool EARLY>
 __global__ __launch_bounds__(256) void gate_up_fused_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up, int k,
                                                             int hidden, int inter, int n_experts, QAct actq,
                                                             int32_t *__restrict__ flags, RouteInline route, RouterExchange rx) {
     extern __shared__ float s_dyn[];  // [rows_per_block] gate/up results, then the token's 16-bit row
     __shared__ __attribute__((aligned(16))) DecodeShared<RJN> sh;
-    const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.z;  // grid = (slot, row tile, token)
     const int a = t * gridDim.x + blockIdx.x;
     const RowSplit rs = row_split(hidden);
@@ -171,16 +173,34 @@ __global__ __launch_bounds__(256) void gate_up_fused_kernel(const uint8_t *__res
     float *s_xscale = (float *)(s_xlo + hidden);
     int *s_xsum = (int *)(s_xscale + hidden / 16);
     MUMMU_PHASE(0);
-    decode_route_prologue<RJN>(k, hidden, n_experts, flags, route, rx, sh, s_xhi, s_xlo, s_xscale, s_xsum);
+    RouteCarry<RJN> carry;
+    decode_route_prologue<RJN, NoHook, EARLY>(k, hidden, n_experts, flags, route, rx, sh, s_xhi, s_xlo, s_xscale, s_xsum, NoHook(), &carry);
     LaneAct<1> la;
     load_lane_act_lds<WT>(s_xhi, s_xlo, s_xscale, s_xsum, unit0, rs.units, la);
     MUMMU_PHASE(14);
-    const int e = sh.ids[blockIdx.x];
+    int e = EARLY ? sh.early_ids[blockIdx.x] : sh.ids[blockIdx.x];
     if ((unsigned)e >= (unsigned)n_experts) {
         if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
         return;
     }
-    gate_up_tile<WT, 1, NIT, true>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act, blockIdx.y);
+    if constexpr (EARLY) {
+        auto route_rest = [&]() {
+            if (wave == 0) decode_route_finish<RJN, true>(carry.l, k, n_experts, flags, route, rx, sh);
+        };
+        gate_up_tile<WT, 1, NIT, true, true, NoHook, NIT - 1, decltype(route_rest)>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act,
+                                                                                    blockIdx.y, NoHook(), route_rest);
+        __syncthreads();
+        if (sh.ids[blockIdx.x] != e) {  // (the same finding in every workgroup of the slot: its rows again, for the expert the routing names)
+            e = sh.ids[blockIdx.x];
+            if ((unsigned)e >= (unsigned)n_experts) {
+                if (threadIdx.x == 0) atomicAdd(&flags[FLAG_BAD_ID], 1);
+                return;
+            }
+            gate_up_tile<WT, 1, NIT, true>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act, blockIdx.y);
+        }
+    } else {
+        gate_up_tile<WT, 1, NIT, true>(gate, up, e, a, la, rs, hidden, inter, nullptr, actq, s_act, blockIdx.y);
+    }
 }
 
 // gate/up, float banks.  RJN > 0: the kernel routes by itself (see RouteInline), RJN experts per lane
@@ -736,11 +756,12 @@ static hipError_t launch_gate_up_fused_t(const ExpertBanks &b, const RouterExcha
     const int rpb = 4 * NIT * rs.rows_per_it;
     dim3 grid(k, (b.inter + rpb - 1) / rpb, n_tokens), block(256);
     const size_t lds = sizeof(float) * (size_t)rpb + 2 * (size_t)b.hidden + 8 * (size_t)(b.hidden / 16);
-#define MUMMU_GUX(JN) \
-    launch_kernel(gate_up_fused_kernel<WT, NIT, JN>, grid, block, lds, s, b.gate, b.up, k, b.hidden, b.inter, b.n_experts, actq, flags, route, rx)
-    if (b.n_experts <= 64) MUMMU_GUX(1);
-    else if (b.n_experts <= 128) MUMMU_GUX(2);
-    else MUMMU_GUX(8);
+#define MUMMU_GUX(JN, EARLY) \
+    launch_kernel(gate_up_fused_kernel<WT, NIT, JN, EARLY>, grid, block, lds, s, b.gate, b.up, k, b.hidden, b.inter, b.n_experts, actq, flags, route, rx)
+    if (b.n_experts <= 64 && k == 8 && b.early_ids) MUMMU_GUX(1, true);
+    else if (b.n_experts <= 64) MUMMU_GUX(1, false);
+    else if (b.n_experts <= 128) MUMMU_GUX(2, false);
+    else MUMMU_GUX(8, false);
 #undef MUMMU_GUX
     return hipGetLastError();
 }

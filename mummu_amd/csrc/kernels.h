@@ -51,6 +51,7 @@ struct ExpertBanks {
     int hidden, inter, n_experts;
     bool q8_half_ok = false;          // Q8_0 banks whose every |d| * 128 is inside the half range (launch_q8_scale_max)
     bool tile_order = false;          // decode launches of several tokens: workgroups ordered so that tokens sharing an expert meet in one XCD's L2
+    bool early_ids = true;            // the decode launches that route by themselves (top-8, at most 64 experts) start their rows on the eight largest logits and confirm them
 };
 
 
@@ -123,8 +124,7 @@ struct PendingSum {
 inline size_t layer_exchange_bytes() { return (size_t)kExchangeXcds * kExchangeTokens * 8 * (size_t)kActBlocksMax * 64; }
 bool decode_layer_supported(const ExpertBanks &b, int k, int n_tokens, const RouterExchange &rx, const LayerExchange &lx);
 hipError_t launch_decode_layer(const ExpertBanks &b, const RouterExchange &rx, const LayerExchange &lx, const RouteInline &route,
-                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &pending = PendingSum(),
-                               bool early_ids = true);
+                               int n_tokens, int k, int32_t *flags, hipStream_t s, const PendingSum &pending = PendingSum());
 // The same pair for float banks (F32 / F16 / BF16 gate/up and down, at most 512 experts, top_k <= 16):
 // gate/up with the routing inside writes act [n*k, inter] f32, then down + combine in one launch.
 bool float_decode_fused(const ExpertBanks &b, int k);

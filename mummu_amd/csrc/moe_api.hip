@@ -120,7 +120,7 @@ struct mummu_moe {
     // and a counter that tells launches apart which read the same epoch (the nodes of one captured graph)
     void *aslots = nullptr;
     int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
-    int early_ids = 1;         // the one-launch form starts its rows on the eight largest logits and confirms them (MUMMU_EARLY_IDS=0: routes first)
+    int early_ids = 1;         // the fused decode launches start their rows on the eight largest logits and confirm them (MUMMU_EARLY_IDS=0: route first)
     int tile_order = 0;        // decode launches of several tokens fetch a shared expert's rows once (mummu_moe_set_tile_order)
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
@@ -480,6 +480,7 @@ ExpertBanks banks_of(const mummu_moe *h, const Layer &L) {
     b.n_experts = h->cfg.num_experts;
     b.q8_half_ok = L.q8_half_ok;
     b.tile_order = h->tile_order != 0;
+    b.early_ids = h->early_ids != 0;
     return b;
 }
 
@@ -713,7 +714,7 @@ int decode_one_launch(mummu_moe *h, const Layer &L, const DecodeScratch &ws, con
     lx.y = db.y;
     route.ids = db.ids;
     route.weights = db.weights;
-    LAUNCH(h, K_DECODE_LAYER, s, launch_decode_layer(b, rx, lx, route, n, k, h->flags, s, ps, h->early_ids != 0));
+    LAUNCH(h, K_DECODE_LAYER, s, launch_decode_layer(b, rx, lx, route, n, k, h->flags, s, ps));
     h->pending.active = false;
     h->routing_buf = buf;
     if (chain) {

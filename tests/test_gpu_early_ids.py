@@ -1,4 +1,4 @@
-"""The one-launch decode form starts a slot's rows on the expert whose LOGIT has the slot's rank and confirms that pick
+"""The fused decode launches (one launch per layer, or router + gate/up in one) start a slot's rows on the expert whose LOGIT has the slot's rank and confirms that pick
 against the routing proper (softmax -> top-8 on probabilities, the lower id on a tie: experts.rs:557-573,
 nn/moe.rs:2143-2144) while the rows are on their way.  Logits built so that the two orders differ - two different
 logits whose probabilities round to the same float, inside the top eight and across its boundary - must take the
@@ -87,6 +87,12 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
                 assert np.array_equal(ids1, ids3), name
                 assert np.array_equal(bits(w1), bits(w3)), name
                 assert np.array_equal(bits(got), bits(want)), name
+                m.set_layer_fusion(0)             # two launches: the fused gate/up kernel makes the same early pick
+                got2 = m.forward(x, K, norm)
+                ids2, w2 = m.last_routing(1, K)
+                m.set_layer_fusion(2)
+                assert np.array_equal(ids2, ids3) and np.array_equal(bits(w2), bits(w3)), name
+                assert np.array_equal(bits(got2), bits(want)), name
                 # and in a chain of deferred sums, where the weights reach the output through the next launch
                 m.set_deferred_combine(True)
                 a, o1, o2 = M.DeviceBuffer.from_array(x), M.DeviceBuffer(H * 4), M.DeviceBuffer(H * 4)
@@ -119,7 +125,11 @@ def test_random_tokens_route_alike_with_and_without_the_early_pick():
             m.set_layer_fusion(2)
             got = m.forward(x, K, True)
             ids1, w1 = m.last_routing(1, K)
+            m.set_layer_fusion(0)
+            got2 = m.forward(x, K, True)
+            ids2, w2 = m.last_routing(1, K)
             m.set_layer_fusion(1)
+            assert np.array_equal(ids2, ids3) and np.array_equal(bits(w2), bits(w3)) and np.array_equal(bits(got2), bits(want)), rep
             assert np.array_equal(ids1, ids3), rep
             assert np.array_equal(bits(w1), bits(w3)), rep
             assert np.array_equal(bits(got), bits(want)), rep
