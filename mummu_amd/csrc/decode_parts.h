@@ -295,6 +295,22 @@ __device__ __forceinline__ int float_order_key(float v) {
     return b ^ ((b >> 31) & 0x7FFFFFFF);
 }
 
+// The eight largest of a wave's logits (lane = expert, n_experts <= 64), larger first, the lower id on equal values:
+// early[s] = the expert of rank s.  What the routing picks wherever the probabilities order like the logits.
+__device__ __forceinline__ void early_top8(float l, int n_experts, int *early) {
+    const int lane = threadIdx.x & 63;
+    int cand = lane < n_experts ? float_order_key(l) : (int)0x80000000;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        const int best = wave_max_i32(cand);
+        const int win = (int)__builtin_ctzll(__ballot(cand == best));  // lowest expert id holding the maximum
+        if (lane == win) {
+            early[s] = lane;
+            cand = (int)0x80000000;
+        }
+    }
+}
+
 // route_token for one expert per lane and k = 8 when the eight winners are believed known (early[0..8), slot order: the
 // eight largest logits): the softmax as route_token computes it, then a CHECK that the rounds on the probabilities would
 // pick exactly these experts in exactly this order - every slot's probability above the next one's, or equal to it with
@@ -572,16 +588,7 @@ __device__ __forceinline__ unsigned long long decode_route_prologue(int k, int h
         }
         if constexpr (EARLY) {
             static_assert(JN == 1, "one expert per routing lane");
-            int cand = lane < n_experts ? float_order_key(l[0]) : (int)0x80000000;
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const int best = wave_max_i32(cand);
-                const int win = (int)__builtin_ctzll(__ballot(cand == best));  // lowest expert id holding the maximum
-                if (lane == win) {
-                    sh.early_ids[s] = lane;
-                    cand = (int)0x80000000;
-                }
-            }
+            early_top8(l[0], n_experts, sh.early_ids);
             carry->l[0] = l[0];
             MUMMU_PHASE(11);
         } else {

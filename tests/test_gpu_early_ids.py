@@ -1,8 +1,10 @@
-"""The fused decode launches (one launch per layer, or router + gate/up in one) start a slot's rows on the expert whose LOGIT has the slot's rank and confirms that pick
+"""The decode launches that route by themselves (gate/up with the routing inside, router + gate/up in one launch, the
+whole layer in one launch) start a slot's rows on the expert whose LOGIT has the slot's rank and confirm that pick
 against the routing proper (softmax -> top-8 on probabilities, the lower id on a tie: experts.rs:557-573,
-nn/moe.rs:2143-2144) while the rows are on their way.  Logits built so that the two orders differ - two different
-logits whose probabilities round to the same float, inside the top eight and across its boundary - must take the
-slot's second pass and still give the routing and the output bits of the three-launch form, which routes first."""
+nn/moe.rs:2143-2144) while the rows are on their way.  Logits built so that the two orders differ - different logits
+whose probabilities round to the same float, inside the top eight and across its last place - must take the slot's
+second pass and still give the routing and the output bits of a handle that routes first (MUMMU_EARLY_IDS=0), in the
+three-, two- and one-launch forms, one token at a time and as a decode batch."""
 import numpy as np
 import pytest
 
@@ -54,6 +56,40 @@ def cases():
     return out
 
 
+def make(flavour, gt, router, rt, seed, early):
+    """A one-layer handle; early = False: created with MUMMU_EARLY_IDS=0, every launch routes first."""
+    import os
+    old = os.environ.get("MUMMU_EARLY_IDS")
+    os.environ["MUMMU_EARLY_IDS"] = "1" if early else "0"
+    try:
+        m = M.SparseMoe(M.SparseMoeConfig(H, I, E, K), num_layers=1, max_tokens=8, rms_norm_eps=1e-5, router_flavour=flavour)
+    finally:
+        if old is None:
+            del os.environ["MUMMU_EARLY_IDS"]
+        else:
+            os.environ["MUMMU_EARLY_IDS"] = old
+    gate = synth.random_bank_fast(gt, [H, I, E], seed + 1)
+    up = synth.random_bank_fast(gt, [H, I, E], seed + 2)
+    down = synth.random_bank_fast(gt, [I, H, E], seed + 3)
+    m.load_layer(0, router, rt, gate, gt, up, gt, down, gt)
+    return m
+
+
+def forms(m, x, norm):
+    """(name, output, ids, weights) of a call in the three-, two- and one-launch forms."""
+    n = x.shape[0]
+    out = []
+    for name, exchange, fusion in (("three launches", False, 1), ("two launches", 2, 0), ("one launch", 2, 2)):
+        m.set_router_exchange(exchange)
+        m.set_layer_fusion(fusion)
+        y = m.forward(x, K, norm)
+        ids, w = m.last_routing(n, K)
+        out.append((name, y, ids, w))
+    m.set_router_exchange(True)
+    m.set_layer_fusion(1)
+    return out
+
+
 @pytest.mark.parametrize("flavour", [0, 1])
 def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
     g = np.random.Generator(np.random.PCG64(9900 + flavour))
@@ -61,38 +97,33 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
     # precondition: the crafted logits really separate the two orders (but for the plain ties)
     for name, l in table.items():
         assert (logit_order(l) != softmax_order(l)) == (name != "all equal"), name
-    m = M.SparseMoe(M.SparseMoeConfig(H, I, E, K), num_layers=1, max_tokens=8, rms_norm_eps=1e-5, router_flavour=flavour)
-    gate = synth.random_bank_fast(M.Q4_K, [H, I, E], 9901)
-    up = synth.random_bank_fast(M.Q4_K, [H, I, E], 9902)
-    down = synth.random_bank_fast(M.Q4_K, [I, H, E], 9903)
     # an F32 router whose column j holds case j's logits: the one-hot token e_j gets exactly them
     router = (g.standard_normal((E, H), dtype=np.float32) * np.float32(0.05)).astype(np.float32)
     names = list(table)
     for j, name in enumerate(names):
         router[:, 100 + j] = table[name]
-    m.load_layer(0, router, M.F32, gate, M.Q4_K, up, M.Q4_K, down, M.Q4_K)
-    with m:
-        for j, name in enumerate(names):
-            x = np.zeros((1, H), np.float32)
-            x[0, 100 + j] = 1.0
+    ref = make(flavour, M.Q4_K, router, M.F32, 9900, early=False)
+    m = make(flavour, M.Q4_K, router, M.F32, 9900, early=True)
+    with ref, m:
+        xs = np.zeros((len(names), H), np.float32)
+        for j in range(len(names)):
+            xs[j, 100 + j] = 1.0
+        # one token at a time, then all of them as one decode batch (the multi-token launches)
+        batches = [(name, xs[j:j + 1]) for j, name in enumerate(names)] + [("batch", xs), ("batch twice", np.concatenate([xs, xs[::-1]]))]
+        for name, x in batches:
+            n = x.shape[0]
             for norm in (False, True):
-                m.set_router_exchange(False)      # three launches: routes first
-                want = m.forward(x, K, norm)
-                ids3, w3 = m.last_routing(1, K)
-                assert list(ids3[0]) == softmax_order(table[name]), name
-                m.set_router_exchange(True)
-                m.set_layer_fusion(2)             # one launch, its sum as a launch of its own
-                got = m.forward(x, K, norm)
-                ids1, w1 = m.last_routing(1, K)
-                assert np.array_equal(ids1, ids3), name
-                assert np.array_equal(bits(w1), bits(w3)), name
-                assert np.array_equal(bits(got), bits(want)), name
-                m.set_layer_fusion(0)             # two launches: the fused gate/up kernel makes the same early pick
-                got2 = m.forward(x, K, norm)
-                ids2, w2 = m.last_routing(1, K)
-                m.set_layer_fusion(2)
-                assert np.array_equal(ids2, ids3) and np.array_equal(bits(w2), bits(w3)), name
-                assert np.array_equal(bits(got2), bits(want)), name
+                ref.set_router_exchange(False)
+                want = ref.forward(x, K, norm)
+                ids0, w0 = ref.last_routing(n, K)
+                if n == 1:
+                    assert list(ids0[0]) == softmax_order(table[name]), name
+                for form, y, ids, w in forms(m, x, norm):
+                    assert np.array_equal(ids, ids0), (name, form)
+                    assert np.array_equal(bits(w), bits(w0)), (name, form)
+                    assert np.array_equal(bits(y), bits(want)), (name, form)
+                if n > 1:
+                    continue
                 # and in a chain of deferred sums, where the weights reach the output through the next launch
                 m.set_deferred_combine(True)
                 a, o1, o2 = M.DeviceBuffer.from_array(x), M.DeviceBuffer(H * 4), M.DeviceBuffer(H * 4)
@@ -102,35 +133,24 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
                 assert np.array_equal(bits(o1.download(np.float32, (1, H))), bits(want)), name
                 assert np.array_equal(bits(o2.download(np.float32, (1, H))), bits(want)), name
                 m.set_deferred_combine(False)
-                m.set_layer_fusion(1)
         assert m.router_exchange_state()[1] == 0
 
 
 def test_random_tokens_route_alike_with_and_without_the_early_pick():
     g = np.random.Generator(np.random.PCG64(9950))
-    m = M.SparseMoe(M.SparseMoeConfig(H, I, E, K), num_layers=1, max_tokens=8, rms_norm_eps=1e-5)
-    gate = synth.random_bank_fast(M.Q8_0, [H, I, E], 9951)
-    up = synth.random_bank_fast(M.Q8_0, [H, I, E], 9952)
-    down = synth.random_bank_fast(M.Q8_0, [I, H, E], 9953)
     # a coarse router (few distinct values) makes equal and near-equal logits common
     router = (np.round(g.standard_normal((E, H)) * 2.0) / 64.0).astype(np.float16)
-    m.load_layer(0, router, M.F16, gate, M.Q8_0, up, M.Q8_0, down, M.Q8_0)
-    with m:
+    ref = make(0, M.Q8_0, router, M.F16, 9950, early=False)
+    m = make(0, M.Q8_0, router, M.F16, 9950, early=True)
+    with ref, m:
         for rep in range(24):
-            x = np.round(g.standard_normal((1, H)) * 2.0).astype(np.float32)
-            m.set_router_exchange(False)
-            want = m.forward(x, K, True)
-            ids3, w3 = m.last_routing(1, K)
-            m.set_router_exchange(True)
-            m.set_layer_fusion(2)
-            got = m.forward(x, K, True)
-            ids1, w1 = m.last_routing(1, K)
-            m.set_layer_fusion(0)
-            got2 = m.forward(x, K, True)
-            ids2, w2 = m.last_routing(1, K)
-            m.set_layer_fusion(1)
-            assert np.array_equal(ids2, ids3) and np.array_equal(bits(w2), bits(w3)) and np.array_equal(bits(got2), bits(want)), rep
-            assert np.array_equal(ids1, ids3), rep
-            assert np.array_equal(bits(w1), bits(w3)), rep
-            assert np.array_equal(bits(got), bits(want)), rep
+            n = 1 + rep % 8
+            x = np.round(g.standard_normal((n, H)) * 2.0).astype(np.float32)
+            ref.set_router_exchange(False)
+            want = ref.forward(x, K, True)
+            ids0, w0 = ref.last_routing(n, K)
+            for form, y, ids, w in forms(m, x, True):
+                assert np.array_equal(ids, ids0), (rep, form)
+                assert np.array_equal(bits(w), bits(w0)), (rep, form)
+                assert np.array_equal(bits(y), bits(want)), (rep, form)
         assert m.router_exchange_state()[1] == 0
