@@ -257,7 +257,7 @@ MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_
  * land on the eight XCDs, and the workgroups of a slot pass the expert's hidden row to one another through their XCD's L2
  * the way the router logits travel, so the down product starts inside the launch that made its input.  What is left is
  * the sum over a token's eight weighted rows, which crosses XCDs.  As a launch of its own that sum costs more than the
- * form saves (19.5 against 17.3 us per layer on the OLMoE shape), so the form pays where a later launch can take the sum
+ * form saves (18.3 against 16.1 us per layer on the OLMoE shape), so the form pays where a later launch can take the sum
  * along: mummu_moe_set_deferred_combine.  No counterpart in the reference.  Same bits as the other forms; the same
  * spin_ticks bounds its waits, and a workgroup that gives up computes the hidden blocks it misses itself (counted by
  * _state's fallbacks).  enable = 0: never; 1 (default): in chains of deferred sums only; 2: wherever the kernel serves

@@ -689,7 +689,7 @@ int decode_one_launch(mummu_moe *h, const Layer &L, const DecodeScratch &ws, con
     // next one.  It writes the set of buffers the pending step does not occupy.
     const float *xe = x + (size_t)n * (size_t)b.hidden;
     const bool chain = may_defer && h->deferred_combine && b.hidden % 256 == 0 && residual == nullptr && norm_gamma == nullptr;
-    // (followed by a launch of its own for the sum the form is slower than two launches - 19.5 against 17.3 us per layer on
+    // (followed by a launch of its own for the sum the form is slower than two launches - 18.3 against 16.1 us per layer on
     // the OLMoE shape - so outside a chain it is taken only on request)
     if (!chain && h->layer_fusion < 2) return MUMMU_OK;
     PendingSum ps;
