@@ -262,8 +262,9 @@ MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_
  * spin_ticks bounds its waits, and a workgroup that gives up computes the hidden blocks it misses itself (counted by
  * _state's fallbacks).  enable = 0: never; 1 (default): in chains of deferred sums only; 2: wherever the kernel serves
  * (every decode call of up to 8 tokens when mummu_moe_set_router_exchange says 2).  Environment: MUMMU_LAYER_FUSION.
- * With at most 64 experts the launch starts every slot's rows on the expert whose logit has the slot's rank and confirms
- * that pick against the routing proper while the rows are on their way; a slot the routing names differently (two
+ * With at most 128 experts the launch (and the router + gate/up launch of the two-launch form) starts every slot's rows
+ * on the expert whose logit has the slot's rank and confirms that pick against the routing proper while the rows are on
+ * their way; a slot the routing names differently (two
  * logits whose probabilities round to the same float) is done again inside the launch: the same routing and the same
  * bits (MUMMU_EARLY_IDS=0 at mummu_moe_create: route first). */
 MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);

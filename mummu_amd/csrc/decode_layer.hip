@@ -12,7 +12,7 @@
 // one exchange inside an L2 instead of a launch, and its weight stream hides behind the wait for the slowest
 // workgroup.  Nothing crosses XCDs inside the launch: every slot leaves its own row of down sums in y.
 //
-// EARLY (at most 64 experts): the workgroups do not wait for the routing.  Wave 0 stops at the eight largest LOGITS,
+// EARLY: the workgroups do not wait for the routing.  Wave 0 stops at the eight largest LOGITS,
 // the workgroup starts its rows on the expert of its slot's rank, and wave 0 confirms the pick behind its first row
 // loads - the softmax, then a check that rounds on the probabilities would choose the same experts in the same order
 // (route_token_checked8), with the rounds themselves only where the check fails.  A slot whose expert the routing then
@@ -294,8 +294,8 @@ static hipError_t launch_decode_layer_t(const ExpertBanks &b, const RouterExchan
     if (b.n_experts <= 64)
         launch_kernel(decode_layer_kernel<WT, DT, NITD, 1, EARLY>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter,
                       b.n_experts, flags, route, rx, lx, ps);
-    else  // (two experts per routing lane: the early pick is written for one)
-        launch_kernel(decode_layer_kernel<WT, DT, NITD, 2, false>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter,
+    else
+        launch_kernel(decode_layer_kernel<WT, DT, NITD, 2, EARLY>, grid, block, lds, s, b.gate, b.up, b.down, k, b.hidden, b.inter,
                       b.n_experts, flags, route, rx, lx, ps);
     return hipGetLastError();
 }

@@ -295,69 +295,125 @@ __device__ __forceinline__ int float_order_key(float v) {
     return b ^ ((b >> 31) & 0x7FFFFFFF);
 }
 
-// The eight largest of a wave's logits (lane = expert, n_experts <= 64), larger first, the lower id on equal values:
-// early[s] = the expert of rank s.  What the routing picks wherever the probabilities order like the logits.
-__device__ __forceinline__ void early_top8(float l, int n_experts, int *early) {
+// The eight largest of a wave's logits (lane holds experts lane, lane + 64, ...: n_experts <= 64 * JN), larger first,
+// the lower id on equal values: early[s] = the expert of rank s.  What the routing picks wherever the probabilities
+// order like the logits.
+template <int JN>
+__device__ __forceinline__ void early_top8(const float (&l)[JN], int n_experts, int *early) {
     const int lane = threadIdx.x & 63;
-    int cand = lane < n_experts ? float_order_key(l) : (int)0x80000000;
+    int cand[JN];
+#pragma unroll
+    for (int j = 0; j < JN; j++) cand[j] = lane + 64 * j < n_experts ? float_order_key(l[j]) : (int)0x80000000;
 #pragma unroll
     for (int s = 0; s < 8; s++) {
-        const int best = wave_max_i32(cand);
-        const int win = (int)__builtin_ctzll(__ballot(cand == best));  // lowest expert id holding the maximum
-        if (lane == win) {
-            early[s] = lane;
-            cand = (int)0x80000000;
+        int mine = cand[0];
+#pragma unroll
+        for (int j = 1; j < JN; j++) mine = cand[j] > mine ? cand[j] : mine;
+        const int best = wave_max_i32(mine);
+        // lowest expert id holding the maximum: the first lane of the lowest j that has one
+        int win = -1;
+#pragma unroll
+        for (int j = JN - 1; j >= 0; j--) {
+            const unsigned long long m = __ballot(cand[j] == best);
+            win = m != 0ull ? (int)__builtin_ctzll(m) + 64 * j : win;
+        }
+#pragma unroll
+        for (int j = 0; j < JN; j++) {
+            if (lane + 64 * j == win) {
+                early[s] = win;
+                cand[j] = (int)0x80000000;
+            }
         }
     }
 }
 
-// route_token for one expert per lane and k = 8 when the eight winners are believed known (early[0..8), slot order: the
-// eight largest logits): the softmax as route_token computes it, then a CHECK that the rounds on the probabilities would
-// pick exactly these experts in exactly this order - every slot's probability above the next one's, or equal to it with
-// the lower id, and nobody outside as good as the last - instead of the rounds themselves (eight dependent wave
-// maxima), and the renormaliser summed in slot order as the rounds would have.  True: ids / weights written, the bits
-// of route_token.  False (probabilities that tie or cross where the logits do not, a logit that is not finite):
-// nothing written, the caller runs route_token.
-__device__ __forceinline__ bool route_token_checked8(float l, int n_experts, int flavour, int norm, const int *early, int32_t *ids,
-                                                     float *weights, RouteScratch<1> &sc) {
+// route_token for k = 8 when the eight winners are believed known (early[0..8), slot order: the eight largest logits):
+// the softmax as route_token computes it, then a CHECK that the rounds on the probabilities would pick exactly these
+// experts in exactly this order - every slot's probability above the next one's, or equal to it with the lower id, and
+// nobody outside as good as the last - instead of the rounds themselves (eight dependent wave maxima), and the
+// renormaliser summed in slot order as the rounds would have.  True: ids / weights written, the bits of route_token.
+// False (probabilities that tie or cross where the logits do not, a logit that is not finite): nothing written, the
+// caller runs route_token.
+template <int JN>
+__device__ __forceinline__ bool route_token_checked8(const float (&l)[JN], int n_experts, int flavour, int norm, const int *early,
+                                                     int32_t *ids, float *weights, RouteScratch<JN> &sc) {
     const int lane = threadIdx.x & 63;
-    const bool real = lane < n_experts;
-    if (__any(real && !(fabsf(l) <= 3.402823466e38f))) return false;
-    const float mx = wave_max(real ? l : -__builtin_inff());
-    float p = real ? det_expf(__fsub_rn(l, mx)) : 0.0f;
-    sc.p[lane] = p;
+    bool bad = false;
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        if (lane + 64 * j < n_experts) {
+            bad = bad || !(fabsf(l[j]) <= 3.402823466e38f);
+            mx = fmaxf(mx, l[j]);
+        }
+    }
+    if (__any(bad)) return false;
+    mx = wave_max(mx);
+    float p[JN];
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        p[j] = (lane + 64 * j < n_experts) ? det_expf(__fsub_rn(l[j], mx)) : 0.0f;
+        sc.p[lane + 64 * j] = p[j];
+    }
     wave_lds_sync();
+    // (the normaliser: route_token's, line for line)
     const float4 *bp = (const float4 *)sc.p;
+    const int chunks = JN == 1 ? 16 : (n_experts + 3) >> 2;
     if (flavour == 0) {
         float total = 0.0f;
 #pragma unroll 16
-        for (int c = 0; c < 16; c++) {
+        for (int c = 0; c < chunks; c++) {
             const float4 v = bp[c];
             total = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(total, v.x), v.y), v.z), v.w);
         }
-        p = __fdiv_rn(p, total);
+#pragma unroll
+        for (int j = 0; j < JN; j++) p[j] = __fdiv_rn(p[j], total);
     } else {
         double total = 0.0;
+        bool exact = JN > 1;
+#pragma unroll
+        for (int j = 0; j < JN; j++) exact = exact && (p[j] == 0.0f || p[j] >= 0x1p-20f);
+        if (JN > 1 && __all(exact)) {
+#pragma unroll
+            for (int j = 0; j < JN; j++) total = __dadd_rn(total, (double)p[j]);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) total = __dadd_rn(total, __shfl_xor(total, off, 64));
+        } else {
 #pragma unroll 16
-        for (int c = 0; c < 16; c++) {
-            const float4 v = bp[c];
-            total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
+            for (int c = 0; c < chunks; c++) {
+                const float4 v = bp[c];
+                total = __dadd_rn(__dadd_rn(__dadd_rn(__dadd_rn(total, (double)v.x), (double)v.y), (double)v.z), (double)v.w);
+            }
         }
-        p = __fmul_rn(p, (float)__ddiv_rn(1.0, total));
+        const float scale = (float)__ddiv_rn(1.0, total);
+#pragma unroll
+        for (int j = 0; j < JN; j++) p[j] = __fmul_rn(p[j], scale);
     }
     int eid[8];
     float ps[8];
-    int my_slot = -1;
+    int my_slot[JN];
+#pragma unroll
+    for (int j = 0; j < JN; j++) my_slot[j] = -1;
 #pragma unroll
     for (int s = 0; s < 8; s++) {
         eid[s] = __builtin_amdgcn_readfirstlane(early[s]);
-        ps[s] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), eid[s]));
-        my_slot = lane == eid[s] ? s : my_slot;
+        float v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p[0]), eid[s] & 63));
+#pragma unroll
+        for (int j = 1; j < JN; j++) {
+            const float vj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p[j]), eid[s] & 63));
+            v = (eid[s] >> 6) == j ? vj : v;
+        }
+        ps[s] = v;
+#pragma unroll
+        for (int j = 0; j < JN; j++) my_slot[j] = lane + 64 * j == eid[s] ? s : my_slot[j];
     }
     bool ok = true;
 #pragma unroll
     for (int s = 0; s < 7; s++) ok = ok && (ps[s] > ps[s + 1] || (ps[s] == ps[s + 1] && eid[s] < eid[s + 1]));
-    const bool beats_last = real && my_slot < 0 && (p > ps[7] || (p == ps[7] && lane < eid[7]));
+    bool beats_last = false;
+#pragma unroll
+    for (int j = 0; j < JN; j++)
+        beats_last = beats_last || (lane + 64 * j < n_experts && my_slot[j] < 0 && (p[j] > ps[7] || (p[j] == ps[7] && lane + 64 * j < eid[7])));
     if (!ok || __any(beats_last)) return false;
     float sum32 = 0.0f;
     double sum64 = 0.0;
@@ -374,11 +430,14 @@ __device__ __forceinline__ bool route_token_checked8(float l, int n_experts, int
         const float floor_v = 1.0f / 16384.0f;  // experts.rs:74
         denom = fs > floor_v ? fs : floor_v;
     }
-    if (my_slot >= 0) {
-        float wv = p;
-        if (flavour != 0 || norm) wv = __fdiv_rn(wv, denom);
-        ids[my_slot] = lane;
-        weights[my_slot] = wv;
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        if (my_slot[j] >= 0) {
+            float wv = p[j];
+            if (flavour != 0 || norm) wv = __fdiv_rn(wv, denom);
+            ids[my_slot[j]] = lane + 64 * j;
+            weights[my_slot[j]] = wv;
+        }
     }
     return true;
 }
@@ -397,7 +456,7 @@ __device__ __forceinline__ void decode_route_finish(float (&l)[JN], int k, int n
             if (lane + 64 * j < n_experts) rx.logits_out[(size_t)t * n_experts + lane + 64 * j] = l[j];
     }
     bool routed = false;
-    if constexpr (CHECKED && JN == 1) routed = route_token_checked8(l[0], n_experts, route.flavour, route.norm, sh.early_ids, sh.ids, sh.w, sh.route);
+    if constexpr (CHECKED && JN <= 2) routed = route_token_checked8<JN>(l, n_experts, route.flavour, route.norm, sh.early_ids, sh.ids, sh.w, sh.route);
     if (!routed) route_token<JN, false>(l, t, n_experts, k, route.flavour, route.norm, sh.ids, sh.w, nullptr, flags, sh.route, 0);
     wave_lds_sync();
     if (blockIdx.x == 0 && blockIdx.y == 0 && lane < k) {
@@ -587,9 +646,10 @@ __device__ __forceinline__ unsigned long long decode_route_prologue(int k, int h
             }
         }
         if constexpr (EARLY) {
-            static_assert(JN == 1, "one expert per routing lane");
-            early_top8(l[0], n_experts, sh.early_ids);
-            carry->l[0] = l[0];
+            static_assert(JN <= 2, "one or two experts per routing lane");
+            early_top8<JN>(l, n_experts, sh.early_ids);
+#pragma unroll
+            for (int j = 0; j < JN; j++) carry->l[j] = l[j];
             MUMMU_PHASE(11);
         } else {
             decode_route_finish<JN>(l, k, n_experts, flags, route, rx, sh);

@@ -152,7 +152,7 @@ __global__ __launch_bounds__(1024) void gate_up_q_kernel(const uint8_t *__restri
 // leave the token's 16-bit row in LDS) is followed by the workgroup's tile of gate/up rows.  The epoch of the
 // exchange is incremented by the launch after this one (down_combine).
 // hidden <= 2048 and a multiple of 64; (slots * row tiles) a multiple of 8.
-// EARLY (k = 8, one expert per routing lane): the rows start on the expert whose logit has the slot's rank; wave 0 confirms
+// EARLY (k = 8, at most two experts per routing lane): the rows start on the expert whose logit has the slot's rank; wave 0 confirms
 // the pick behind its first row loads and a slot the routing names differently is done again (see decode_route_prologue).
 // ------------------------------------------------------------------------------------------
 template <int WT, int NIT, int RJN, bool EARLY>
@@ -760,6 +760,7 @@ static hipError_t launch_gate_up_fused_t(const ExpertBanks &b, const RouterExcha
     launch_kernel(gate_up_fused_kernel<WT, NIT, JN, EARLY>, grid, block, lds, s, b.gate, b.up, k, b.hidden, b.inter, b.n_experts, actq, flags, route, rx)
     if (b.n_experts <= 64 && k == 8 && b.early_ids) MUMMU_GUX(1, true);
     else if (b.n_experts <= 64) MUMMU_GUX(1, false);
+    else if (b.n_experts <= 128 && k == 8 && b.early_ids) MUMMU_GUX(2, true);
     else if (b.n_experts <= 128) MUMMU_GUX(2, false);
     else MUMMU_GUX(8, false);
 #undef MUMMU_GUX

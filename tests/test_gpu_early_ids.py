@@ -13,7 +13,7 @@ from mummu_amd import synth
 
 pytestmark = pytest.mark.gpu
 
-H, I, E, K = 2048, 256, 64, 8
+H, I, K = 2048, 256, 8
 
 
 def bits(a):
@@ -32,23 +32,24 @@ def softmax_order(l):
     return sorted(range(len(l)), key=lambda e: (-float(p[e]), e))[:8]
 
 
-def cases():
+def cases(E):
+    f = E // 64   # (with 128 experts the same places doubled: both experts of a routing lane take part)
     tiny, tiny2 = np.float32(1e-30), np.float32(2e-30)
     out = {}
     # inside the top eight: expert 40 has the larger logit, expert 10 the same probability and the lower id
     l = np.full(E, -6.0, np.float32)
-    l[[3, 7, 21, 33, 50, 63]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75]
-    l[10], l[40] = tiny, tiny2
+    l[[3 * f, 7 * f, 21 * f, 33 * f, 50 * f, 63 * f]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75]
+    l[10 * f], l[40 * f] = tiny, tiny2
     out["order inside the eight"] = l
     # across the boundary: seven clear winners, then 40 (larger logit) against 10 (same probability, lower id)
     l = np.full(E, -6.0, np.float32)
-    l[[3, 7, 21, 33, 50, 63, 12]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75, 0.5]
-    l[10], l[40] = tiny, tiny2
+    l[[3 * f, 7 * f, 21 * f, 33 * f, 50 * f, 63 * f, 12 * f]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75, 0.5]
+    l[10 * f], l[40 * f] = tiny, tiny2
     out["the eighth place"] = l
     # three of them, two places left
     l = np.full(E, -6.0, np.float32)
-    l[[3, 7, 21, 33, 50, 63]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75]
-    l[9], l[30], l[55] = tiny, np.float32(3e-30), tiny2
+    l[[3 * f, 7 * f, 21 * f, 33 * f, 50 * f, 63 * f]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75]
+    l[9 * f], l[30 * f], l[55 * f] = tiny, np.float32(3e-30), tiny2
     out["three for two places"] = l
     # plain ties (equal logits): both orders agree, no second pass
     l = np.full(E, 0.25, np.float32)
@@ -56,7 +57,7 @@ def cases():
     return out
 
 
-def make(flavour, gt, router, rt, seed, early):
+def make(flavour, gt, router, rt, seed, early, E):
     """A one-layer handle; early = False: created with MUMMU_EARLY_IDS=0, every launch routes first."""
     import os
     old = os.environ.get("MUMMU_EARLY_IDS")
@@ -90,10 +91,10 @@ def forms(m, x, norm):
     return out
 
 
-@pytest.mark.parametrize("flavour", [0, 1])
-def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
-    g = np.random.Generator(np.random.PCG64(9900 + flavour))
-    table = cases()
+@pytest.mark.parametrize("flavour,E", [(0, 64), (1, 64), (0, 128), (1, 128)])
+def test_the_early_pick_is_corrected_where_probabilities_tie(flavour, E):
+    g = np.random.Generator(np.random.PCG64(9900 + flavour + E))
+    table = cases(E)
     # precondition: the crafted logits really separate the two orders (but for the plain ties)
     for name, l in table.items():
         assert (logit_order(l) != softmax_order(l)) == (name != "all equal"), name
@@ -102,8 +103,8 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
     names = list(table)
     for j, name in enumerate(names):
         router[:, 100 + j] = table[name]
-    ref = make(flavour, M.Q4_K, router, M.F32, 9900, early=False)
-    m = make(flavour, M.Q4_K, router, M.F32, 9900, early=True)
+    ref = make(flavour, M.Q4_K, router, M.F32, 9900, False, E)
+    m = make(flavour, M.Q4_K, router, M.F32, 9900, True, E)
     with ref, m:
         xs = np.zeros((len(names), H), np.float32)
         for j in range(len(names)):
@@ -136,12 +137,13 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour):
         assert m.router_exchange_state()[1] == 0
 
 
-def test_random_tokens_route_alike_with_and_without_the_early_pick():
-    g = np.random.Generator(np.random.PCG64(9950))
+@pytest.mark.parametrize("E", [64, 128])
+def test_random_tokens_route_alike_with_and_without_the_early_pick(E):
+    g = np.random.Generator(np.random.PCG64(9950 + E))
     # a coarse router (few distinct values) makes equal and near-equal logits common
     router = (np.round(g.standard_normal((E, H)) * 2.0) / 64.0).astype(np.float16)
-    ref = make(0, M.Q8_0, router, M.F16, 9950, early=False)
-    m = make(0, M.Q8_0, router, M.F16, 9950, early=True)
+    ref = make(0, M.Q8_0, router, M.F16, 9950, False, E)
+    m = make(0, M.Q8_0, router, M.F16, 9950, True, E)
     with ref, m:
         for rep in range(24):
             n = 1 + rep % 8
