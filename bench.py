@@ -177,7 +177,9 @@ def main() -> int:
                          "mummu_moe_set_deferred_combine)")
     ap.add_argument("--tile-order", action="store_true",
                     help="several tokens per step: order the decode workgroups so that tokens sharing an expert fetch its rows "
-                         "once (mummu_moe_set_tile_order: a third less HBM traffic at 8 tokens, up to 6 %% more time)")
+                         "once, from two tokens on (mummu_moe_set_tile_order; by default the library does so from six tokens "
+                         "on, where it is also the faster order)")
+    ap.add_argument("--no-tile-order", action="store_true", help="never order the decode workgroups that way")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--seed", type=int, default=1234)
@@ -240,7 +242,8 @@ def main() -> int:
                       router_flavour=w.get("flavour", 0))
     deferred = not args.no_deferred_combine and not args.stack and not args.shared_inter
     moe.set_deferred_combine(deferred)
-    moe.set_tile_order(args.tile_order)
+    tile_order = True if args.tile_order else (False if args.no_tile_order else None)
+    moe.set_tile_order(tile_order)
     routers = []
     keep_layer0 = None
     for l in range(L):
@@ -436,7 +439,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
                    "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "shared_inter": args.shared_inter,
-                   "deferred_combine": bool(deferred), "tile_order": bool(args.tile_order), "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
+                   "deferred_combine": bool(deferred), "tile_order": "from 6 tokens" if tile_order is None else tile_order, "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
                    "graph_replays_timed": (replays + (1 if left else 0)) if graph is not None else 0,
                    "first_timed_step": first,
                    "cache_cold": bool((per_graph - 1) * layer_bytes * layers_per_step > 256e6) if graph is not None else

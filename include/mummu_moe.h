@@ -278,12 +278,13 @@ MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
  * No counterpart in the reference.  Same bits as mummu_moe_forward_device without it.  Not taken with a shared expert on
  * the layer or inside mummu_moe_stack_forward*.  Environment: MUMMU_DEFERRED_COMBINE=1. */
 MUMMU_API int mummu_moe_set_deferred_combine(mummu_moe *h, int enable);
-/* enable = 1 (default 0): decode steps of several tokens on block-quantized banks order their workgroups so that the
- * tokens which routed to the same expert read its rows through the same XCD's L2 at the same time.  The launches then
- * fetch every distinct expert once - 1.01x its bytes instead of 1.2x / 1.5x at 4 / 8 tokens of top-8 over 64 experts, where
- * the reference shares a decoded row among the rows of a call (nn/packed_gemv.rs:561-575) - in the same time at 8 tokens
- * and 1 - 6 % more at 2 - 4: for callers to whom HBM traffic matters.  Same bits either way.  Environment:
- * MUMMU_TILE_ORDER=1. */
+/* Decode steps of several tokens on block-quantized banks can order their workgroups so that the tokens which routed to
+ * the same expert read its rows through the same XCD's L2 at the same time.  The launches then fetch every distinct
+ * expert once - 1.01x its bytes instead of 1.2x / 1.5x at 4 / 8 tokens of top-8 over 64 experts, where the reference
+ * shares a decoded row among the rows of a call (nn/packed_gemv.rs:561-575).  From six tokens on that is also the faster
+ * order (49.4 against 49.7 us per layer at 8 tokens of the OLMoE shape, 81.8 against 84.6 at 16), at two to four it
+ * costs 1 - 6 %.  enable = -1 (the default): from six tokens on; 1: from two, for callers to whom the HBM traffic
+ * matters more than the time; 0: never.  Same bits in every case.  Environment: MUMMU_TILE_ORDER. */
 MUMMU_API int mummu_moe_set_tile_order(mummu_moe *h, int enable);
 /* Enqueues the sum a deferred step left pending (nothing to do otherwise); does not synchronise. */
 MUMMU_API int mummu_moe_flush(mummu_moe *h);

@@ -61,15 +61,15 @@ static hipError_t with_bank_type(int type, F &&f) {
 #undef MUMMU_TYPE_CASE
 }
 
-// Several tokens per step, on request (ExpertBanks::tile_order): tokens that routed to the same expert read the same
+// Several tokens per step (ExpertBanks::tile_order_from and up): tokens that routed to the same expert read the same
 // weight rows, and the eight XCDs each have an L2 of their own, so the second read only hits if both workgroups sit
 // on one XCD at about the same time.  Workgroups go to the XCDs round-robin by linear index; with grid = (kXcds,
 // slots * tokens, ceil(tiles / kXcds)) the XCD is the row tile modulo 8 and every (token, slot) pair of a tile follows
 // its neighbour onto that XCD: whoever shares an expert shares the lines while they are in that L2 (or on their way
 // into it).  The launches then fetch the bytes of the distinct experts once (1.01x against 1.5x at eight tokens of
-// top-8 over 64 experts) in the same time at eight tokens and 1 - 6 % more at two to four (an XCD no longer walks
-// through one expert's matrix from end to end): it is for callers to whom the memory traffic matters.  A variant of
-// the kernels compiled for it, so that the plain order keeps its code as it is.
+// top-8 over 64 experts); from six tokens on that is the faster order as well (81.8 against 84.6 us per layer at 16
+// tokens), at two to four it takes 1 - 6 % more time (an XCD no longer walks through one expert's matrix from end to
+// end), so by default it starts at six.  A variant of the kernels compiled for it: the plain order keeps its code.
 constexpr int kXcds = 8;
 
 // The grid of that order for `pairs` = tokens (x slots) per row tile, or false: the plain grid (not asked for, one
@@ -509,7 +509,7 @@ static hipError_t launch_gate_up_t(const ExpertBanks &b, const float *x, QAct xq
         const int rpb = waves * (NIT)*rs.rows_per_it;                                                           \
         const int tiles = (b.inter + rpb - 1) / rpb, tokens = n_assign / slots;                                 \
         dim3 grid(slots, tiles, tokens), block(64 * waves);                                                     \
-        const bool ordered = tile_order_grid(b.tile_order && fixed_expert < 0 && actq_out, tokens, slots * tokens, tiles, grid); \
+        const bool ordered = tile_order_grid(tokens >= b.tile_order_from && fixed_expert < 0 && actq_out, tokens, slots * tokens, tiles, grid); \
         const size_t lds = sizeof(float) * (size_t)rpb;                                                         \
         if (ordered)                                                                                            \
             launch_kernel(gate_up_q_kernel<WT, UPL, NIT, true, 0, true>, grid, block, lds, s,                              \
@@ -698,7 +698,7 @@ static hipError_t launch_gate_up_routed_t(const ExpertBanks &b, QAct xq, const R
     const int rpb = waves * NIT * rs.rows_per_it;
     const int tiles = (b.inter + rpb - 1) / rpb;
     dim3 grid(k, tiles, n_tokens), block(64 * waves);
-    const bool ordered = tile_order_grid(b.tile_order, n_tokens, k * n_tokens, tiles, grid);
+    const bool ordered = tile_order_grid(n_tokens >= b.tile_order_from, n_tokens, k * n_tokens, tiles, grid);
     const size_t lds = sizeof(float) * (size_t)rpb;
 #define MUMMU_GUR(JN)                                                                                                    \
     do {                                                                                                                 \
@@ -836,7 +836,7 @@ static hipError_t launch_down_combine_t(const ExpertBanks &b, QAct actq, const i
         const int rpb = (NIT)*rs.rows_per_it;                                                                      \
         const int tiles = (b.hidden + rpb - 1) / rpb;                                                              \
         dim3 grid(n, tiles), block(64 * (WAVES));                                                                  \
-        const bool ordered = tile_order_grid(b.tile_order, n, n, tiles, grid);                                     \
+        const bool ordered = tile_order_grid(n >= b.tile_order_from, n, n, tiles, grid);                                    \
         const size_t lds = sizeof(float) * (size_t)((WAVES) * (KPW)) * (size_t)(rpb + 1);                          \
         if (ordered)                                                                                               \
             launch_kernel(down_combine_q_kernel<WT, UPL, NIT, KPW, WAVES, true>, grid, block, lds, s, b.down, actq, ids, weights, k, \

@@ -50,7 +50,7 @@ struct ExpertBanks {
     int gate_type, up_type, down_type;
     int hidden, inter, n_experts;
     bool q8_half_ok = false;          // Q8_0 banks whose every |d| * 128 is inside the half range (launch_q8_scale_max)
-    bool tile_order = false;          // decode launches of several tokens: workgroups ordered so that tokens sharing an expert meet in one XCD's L2
+    int tile_order_from = 6;          // decode launches of this many tokens or more: workgroups ordered so that tokens sharing an expert meet in one XCD's L2
     bool early_ids = true;            // the decode launches that route by themselves (top-8, at most 64 experts) start their rows on the eight largest logits and confirm them
 };
 

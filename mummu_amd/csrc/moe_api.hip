@@ -121,7 +121,7 @@ struct mummu_moe {
     void *aslots = nullptr;
     int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
     int early_ids = 1;         // the fused decode launches start their rows on the eight largest logits and confirm them (MUMMU_EARLY_IDS=0: route first)
-    int tile_order = 0;        // decode launches of several tokens fetch a shared expert's rows once (mummu_moe_set_tile_order)
+    int tile_order = -1;       // decode launches of several tokens fetch a shared expert's rows once: -1 from six tokens on, 0 never, 1 from two (mummu_moe_set_tile_order)
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
     // off by default), whose otherwise idle waves do it: the one-launch form then costs one launch per step.  The per-slot
@@ -479,7 +479,7 @@ ExpertBanks banks_of(const mummu_moe *h, const Layer &L) {
     b.inter = h->cfg.expert_intermediate_size;
     b.n_experts = h->cfg.num_experts;
     b.q8_half_ok = L.q8_half_ok;
-    b.tile_order = h->tile_order != 0;
+    b.tile_order_from = h->tile_order < 0 ? 6 : (h->tile_order == 0 ? 0x7fffffff : 2);
     b.early_ids = h->early_ids != 0;
     return b;
 }
@@ -1077,7 +1077,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
         if (const char *e = getenv("MUMMU_ROUTER_EXCHANGE")) h->router_exchange = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
         if (const char *e = getenv("MUMMU_LAYER_FUSION")) h->layer_fusion = atoi(e) < 0 ? 0 : (atoi(e) > 2 ? 2 : atoi(e));
         if (const char *e = getenv("MUMMU_DEFERRED_COMBINE")) h->deferred_combine = atoi(e) != 0;
-        if (const char *e = getenv("MUMMU_TILE_ORDER")) h->tile_order = atoi(e) != 0;
+        if (const char *e = getenv("MUMMU_TILE_ORDER")) h->tile_order = atoi(e) < 0 ? -1 : (atoi(e) != 0);
         if (const char *e = getenv("MUMMU_EARLY_IDS")) h->early_ids = atoi(e) != 0;
     }
     {
@@ -1764,7 +1764,7 @@ int mummu_moe_set_tile_order(mummu_moe *h, int enable) {
     if (!h) return fail(nullptr, MUMMU_ERR_ARG, "null handle");
     Entry entry(h);
     if (entry.rc) return entry.rc;
-    h->tile_order = enable != 0;
+    h->tile_order = enable < 0 ? -1 : (enable != 0);
     return MUMMU_OK;
 }
 

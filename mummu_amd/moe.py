@@ -321,9 +321,10 @@ class SparseMoe:
         self._check(self._lib.mummu_moe_set_deferred_combine(self._h, int(bool(enable))))
 
     def set_tile_order(self, enable):
-        """Decode steps of several tokens fetch the rows of an expert that several tokens share once (off by default:
-        a third less HBM traffic at eight tokens in the same time, 1 - 6 % more time at two to four).  Same bits either way."""
-        self._check(self._lib.mummu_moe_set_tile_order(self._h, int(bool(enable))))
+        """Decode steps of several tokens fetch the rows of an expert that several tokens share once: None = from six
+        tokens on (the default: there it is also the faster order), True = from two (a third less HBM traffic, 1 - 6 %
+        more time at two to four tokens), False = never.  Same bits in every case."""
+        self._check(self._lib.mummu_moe_set_tile_order(self._h, -1 if enable is None else int(bool(enable))))
 
     def flush(self):
         """Enqueues the sum a deferred decode step left pending; does not synchronise."""
