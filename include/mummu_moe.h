@@ -266,11 +266,13 @@ MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_
  * on the expert whose logit has the slot's rank and confirms that pick against the routing proper while the rows are on
  * their way; a slot the routing names differently (two
  * logits whose probabilities round to the same float) is done again inside the launch: the same routing and the same
- * bits (MUMMU_EARLY_IDS=0 at mummu_moe_create: route first). */
+ * bits (MUMMU_EARLY_IDS=0 at mummu_moe_create: route first).  At its end the launch also reads the router of the layer after
+ * its own (the first after the last: the layer a decode loop calls next) into the L2s, so that the next launch starts on
+ * warm rows: 2 MB of extra reads per launch for 0.4 us (MUMMU_WARM_NEXT=0: not). */
 MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
 /* enable = 1 (default 0): a mummu_moe_forward_device call that can take the one-launch form no longer enqueues the sum over
  * each token's eight weighted rows; the launch of the NEXT such call on the same stream does it on the side (a wave per
- * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (14.4 us
+ * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (13.9 us
  * per layer on the OLMoE shape).  out_dev of a call is then complete once the next call's work, or mummu_moe_flush, has
  * run on the stream; every other entry point of the handle, mummu_graph_begin / _end and mummu_moe_check enqueue a
  * pending sum first, so a captured graph always ends with its last step's sum and a caller that reads out_dev after

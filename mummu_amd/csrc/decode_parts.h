@@ -274,6 +274,20 @@ __device__ __forceinline__ void pending_sum_wave(const PendingSum &ps, int hidde
     }
 }
 
+// Reads `warm` (bytes: a multiple of 16) into the L2 of the XCD this workgroup runs on: the workgroups of the XCD take a slice each, the last wave of
+// each asks for it, nobody uses the data.  The loads come back whenever they do, so their destination is a register set
+// the caller keeps reserved to the end of the kernel (`sink`, handed to warm_wait there): nothing else may have been given
+// those registers by then.
+__device__ __forceinline__ void warm_next(const void *warm, unsigned bytes, u32x4 &sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (warm == nullptr || wave != (int)(blockDim.x >> 6) - 1) return;
+    const unsigned per_xcd = (gridDim.x * gridDim.y) >> 3, mine = (blockIdx.y * gridDim.x + blockIdx.x) >> 3;
+    const unsigned pieces = bytes >> 4, each = (pieces + per_xcd - 1) / per_xcd;
+    for (unsigned i = mine * each + (unsigned)lane; i < (mine + 1) * each && i < pieces; i += 64)
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"((const u32x4 *)warm + i) : "memory");
+}
+__device__ __forceinline__ void warm_wait(u32x4 &sink) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory"); }
+
 // LDS a decode workgroup keeps of its token: the 16-bit row of the block's input and the routing.
 template <int JN>
 struct DecodeShared {

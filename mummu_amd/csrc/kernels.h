@@ -110,6 +110,10 @@ struct LayerExchange {
     void *act_slots = nullptr;               // layer_exchange_bytes() bytes, 256-byte aligned
     float *y = nullptr;                      // [n * k, hidden] out
     unsigned long long *fallbacks = nullptr; // nullable: += 1 per workgroup that computed blocks of other workgroups itself
+    // nullable: warm_bytes (a multiple of 16) that the NEXT launch will want first - the router of the layer a decode loop
+    // calls next - which this launch reads into every XCD's L2 once its own rows have all been asked for
+    const void *warm = nullptr;
+    unsigned warm_bytes = 0;
 };
 // A weighted sum over the eight slots of an earlier launch's tokens that this launch performs on the side (waves that
 // would otherwise wait for the routing): out = (residual +) the sum in ascending expert id, as launch_combine.

@@ -121,6 +121,7 @@ struct mummu_moe {
     void *aslots = nullptr;
     int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
     int early_ids = 1;         // the fused decode launches start their rows on the eight largest logits and confirm them (MUMMU_EARLY_IDS=0: route first)
+    int warm_next = 1;         // the one-launch decode form reads the next layer's router into the L2s at its end (MUMMU_WARM_NEXT=0: not)
     int tile_order = -1;       // decode launches of several tokens fetch a shared expert's rows once: -1 from six tokens on, 0 never, 1 from two (mummu_moe_set_tile_order)
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
@@ -677,6 +678,15 @@ int decode_one_launch(mummu_moe *h, const Layer &L, const DecodeScratch &ws, con
     lx.act_slots = ws.aslots;
     lx.y = ws.y;
     lx.fallbacks = ws.xstate + 1;
+    // the layer a decode loop calls next is, as a rule, the one after this one (and the first after the last)
+    const size_t li = (size_t)(&L - h->layers.data()), nl = h->layers.size();
+    if (h->warm_next && nl > 1 && li < nl) {
+        const Layer &N = h->layers[(li + 1) % nl];
+        if (N.router != nullptr) {
+            lx.warm = N.router;
+            lx.warm_bytes = (unsigned)((size_t)h->cfg.num_experts * (size_t)h->cfg.hidden_size * (N.router_type == T_F32 ? 4 : 2)) & ~15u;
+        }
+    }
     RouterExchange rx = router_exchange_of(h, L, ws, x, norm_gamma, xnorm_out);
     if (!decode_layer_supported(b, k, n, rx, lx)) return MUMMU_OK;
     RouteInline route;
@@ -1079,6 +1089,7 @@ int mummu_moe_create(const mummu_moe_config *cfg, mummu_moe **out) {
         if (const char *e = getenv("MUMMU_DEFERRED_COMBINE")) h->deferred_combine = atoi(e) != 0;
         if (const char *e = getenv("MUMMU_TILE_ORDER")) h->tile_order = atoi(e) < 0 ? -1 : (atoi(e) != 0);
         if (const char *e = getenv("MUMMU_EARLY_IDS")) h->early_ids = atoi(e) != 0;
+        if (const char *e = getenv("MUMMU_WARM_NEXT")) h->warm_next = atoi(e) != 0;
     }
     {
         // resolve the static scratch's address on this device now, outside any stream capture
