@@ -7,7 +7,10 @@ headline metric is quoted on.  A "step" is one forward of one MoE layer over one
 tokens, inputs and weights already resident in HBM.  Steps rotate over `--layers` distinct
 layer banks (16 x 226.5 MB) and over a pool of distinct tokens, so that no step finds its
 expert weights in the 256 MB Infinity Cache from an earlier step: a layer is revisited only
-after the other 15 have streamed >= 425 MB through the cache.
+after the other 15 have streamed >= 425 MB through the cache.  What a step does find warm is its
+256 KB router: the library's one-launch decode form reads the router of the layer after its own into
+the L2s while it ends (what a decode loop that walks the layers in order calls next, and what these
+steps do); MUMMU_WARM_NEXT=0 in the environment measures without that (`config.warm_next_router`).
 
 The timed steps are replays of a HIP graph that holds one rotation (or the whole timed region,
 if that is shorter) - the serving-loop form; they start where the warm-up steps stopped, so no
@@ -439,7 +442,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: hidden {H}, {E} experts, top-{k}, inter {I}, {w['bank']} experts{' (' + w['down'] + ' down)' if 'down' in w else ''}, "
                                f"f16 router, norm_topk_prob={str(norm).lower()}, {n} token(s)/step, rotating over {L} layer banks",
                    "tokens_per_step": n, "layers": L, "stack": bool(args.stack), "shared_inter": args.shared_inter,
-                   "deferred_combine": bool(deferred), "tile_order": "from 6 tokens" if tile_order is None else tile_order, "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
+                   "deferred_combine": bool(deferred), "tile_order": "from 6 tokens" if tile_order is None else tile_order, "warm_next_router": os.environ.get("MUMMU_WARM_NEXT", "1") != "0", "hip_graph": graph is not None, "steps_per_graph_launch": per_graph if graph is not None else None,
                    "graph_replays_timed": (replays + (1 if left else 0)) if graph is not None else 0,
                    "first_timed_step": first,
                    "cache_cold": bool((per_graph - 1) * layer_bytes * layers_per_step > 256e6) if graph is not None else
