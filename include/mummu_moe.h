@@ -272,7 +272,7 @@ MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_
 MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
 /* enable = 1 (default 0): a mummu_moe_forward_device call that can take the one-launch form no longer enqueues the sum over
  * each token's eight weighted rows; the launch of the NEXT such call on the same stream does it on the side (a wave per
- * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (13.9 us
+ * workgroup that would otherwise wait for the routing), so a sequence of decode steps costs one launch per step (13.7 us
  * per layer on the OLMoE shape).  out_dev of a call is then complete once the next call's work, or mummu_moe_flush, has
  * run on the stream; every other entry point of the handle, mummu_graph_begin / _end and mummu_moe_check enqueue a
  * pending sum first, so a captured graph always ends with its last step's sum and a caller that reads out_dev after

@@ -57,6 +57,24 @@ def cases(E):
     return out
 
 
+def near_ties(E):
+    """Logits a few units in the last place apart, the larger one at the higher id: the early pick, which tells experts
+    apart by id below 2^7 units in the last place, may take them in the other order than the routing does - or not;
+    either way the routing's answer has to come out."""
+    f = E // 64
+    out = {}
+    for name, places, gap in (("one ulp inside", [3, 7, 21, 33, 50, 63], 1), ("forty ulps at the eighth place", [3, 7, 21, 33, 50, 63, 12], 40)):
+        l = np.full(E, -6.0, np.float32)
+        l[[p * f for p in places]] = [2.0, 1.75, 1.5, 1.25, 1.0, 0.75, 0.5][:len(places)]
+        lo = np.float32(0.3)
+        hi = lo
+        for _ in range(gap):
+            hi = np.nextafter(hi, np.float32(1.0))
+        l[10 * f], l[40 * f] = lo, hi
+        out[name] = l
+    return out
+
+
 def make(flavour, gt, router, rt, seed, early, E):
     """A one-layer handle; early = False: created with MUMMU_EARLY_IDS=0, every launch routes first."""
     import os
@@ -100,6 +118,8 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour, E):
         assert (logit_order(l) != softmax_order(l)) == (name != "all equal"), name
     # an F32 router whose column j holds case j's logits: the one-hot token e_j gets exactly them
     router = (g.standard_normal((E, H), dtype=np.float32) * np.float32(0.05)).astype(np.float32)
+    extra = near_ties(E)
+    table = dict(table, **extra)
     names = list(table)
     for j, name in enumerate(names):
         router[:, 100 + j] = table[name]
@@ -110,14 +130,14 @@ def test_the_early_pick_is_corrected_where_probabilities_tie(flavour, E):
         for j in range(len(names)):
             xs[j, 100 + j] = 1.0
         # one token at a time, then all of them as one decode batch (the multi-token launches)
-        batches = [(name, xs[j:j + 1]) for j, name in enumerate(names)] + [("batch", xs), ("batch twice", np.concatenate([xs, xs[::-1]]))]
+        batches = [(name, xs[j:j + 1]) for j, name in enumerate(names)] + [("batch", xs), ("batch of eight", np.concatenate([xs[:4], xs[::-1][:4]]))]
         for name, x in batches:
             n = x.shape[0]
             for norm in (False, True):
                 ref.set_router_exchange(False)
                 want = ref.forward(x, K, norm)
                 ids0, w0 = ref.last_routing(n, K)
-                if n == 1:
+                if n == 1 and name not in extra:
                     assert list(ids0[0]) == softmax_order(table[name]), name
                 for form, y, ids, w in forms(m, x, norm):
                     assert np.array_equal(ids, ids0), (name, form)
