@@ -8,8 +8,8 @@ tokens, inputs and weights already resident in HBM.  Steps rotate over `--layers
 layer banks (16 x 226.5 MB) and over a pool of distinct tokens, so that no step finds its
 expert weights in the 256 MB Infinity Cache from an earlier step: a layer is revisited only
 after the other 15 have streamed >= 425 MB through the cache.  What a step does find warm is its
-256 KB router: the library's one-launch decode form reads the router of the layer after its own into
-the L2s while it ends (what a decode loop that walks the layers in order calls next, and what these
+256 KB router: the library's one-launch decode form reads the router of the layer after its own ahead
+while it ends (what a decode loop that walks the layers in order calls next, and what these
 steps do); MUMMU_WARM_NEXT=0 in the environment measures without that (`config.warm_next_router`).
 
 The timed steps are replays of a HIP graph that holds one rotation (or the whole timed region,

@@ -267,8 +267,8 @@ MUMMU_API int mummu_moe_router_exchange_state(mummu_moe *h, int *usable, uint64_
  * their way; a slot the routing names differently (two
  * logits whose probabilities round to the same float) is done again inside the launch: the same routing and the same
  * bits (MUMMU_EARLY_IDS=0 at mummu_moe_create: route first).  At its end the launch also reads the router of the layer after
- * its own (the first after the last: the layer a decode loop calls next) into the L2s, so that the next launch starts on
- * warm rows: 2 MB of extra reads per launch for 0.3 us of 14 (MUMMU_WARM_NEXT=0: not). */
+ * its own (the first after the last: the layer a decode loop calls next) ahead, every XCD its copy, so that the next launch starts
+ * on warm rows: 2 MB of extra reads per launch for 0.3 us of 14 (MUMMU_WARM_NEXT=0: not). */
 MUMMU_API int mummu_moe_set_layer_fusion(mummu_moe *h, int enable);
 /* enable = 1 (default 0): a mummu_moe_forward_device call that can take the one-launch form no longer enqueues the sum over
  * each token's eight weighted rows; the launch of the NEXT such call on the same stream does it on the side (a wave per

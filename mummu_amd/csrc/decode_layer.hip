@@ -191,7 +191,7 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
                 act_piece_from_lds(s_ahi, s_alo, s_ascale, s_asum, blk, piece, act_piece_tag(epoch, rx.salt, pos0 + (unsigned)(blk * 4 + piece)));
     }
     MUMMU_PHASE(14);
-    // (the rows this launch is still waiting for have all been asked for: the next launch's router goes into the L2 behind them)
+    // (the rows this launch is still waiting for have all been asked for: the next launch's router is read ahead behind them)
     u32x4 warm_sink = {0u, 0u, 0u, 0u};
     warm_next(lx.warm, lx.warm_bytes, warm_sink);
 

@@ -274,7 +274,8 @@ __device__ __forceinline__ void pending_sum_wave(const PendingSum &ps, int hidde
     }
 }
 
-// Reads `warm` (bytes: a multiple of 16) into the L2 of the XCD this workgroup runs on: the workgroups of the XCD take a slice each, the last wave of
+// Reads `warm` (bytes: a multiple of 16) ahead of the launch that will want it, through the L2 of the XCD this workgroup runs on
+// (every XCD all of it, as that launch will: read by one XCD only, half of the gain is left): the workgroups of the XCD take a slice each, the last wave of
 // each asks for it, nobody uses the data.  The loads come back whenever they do, so their destination is a register set
 // the caller keeps reserved to the end of the kernel (`sink`, handed to warm_wait there): nothing else may have been given
 // those registers by then.

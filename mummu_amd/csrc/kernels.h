@@ -111,7 +111,7 @@ struct LayerExchange {
     float *y = nullptr;                      // [n * k, hidden] out
     unsigned long long *fallbacks = nullptr; // nullable: += 1 per workgroup that computed blocks of other workgroups itself
     // nullable: warm_bytes (a multiple of 16) that the NEXT launch will want first - the router of the layer a decode loop
-    // calls next - which this launch reads into every XCD's L2 once its own rows have all been asked for
+    // calls next - which this launch reads ahead, through every XCD's L2, once its own rows have all been asked for
     const void *warm = nullptr;
     unsigned warm_bytes = 0;
 };

@@ -121,7 +121,7 @@ struct mummu_moe {
     void *aslots = nullptr;
     int layer_fusion = 1;      // 0: never the one-launch form; 1: where its sum can be left to the next step; 2: wherever it serves
     int early_ids = 1;         // the fused decode launches start their rows on the eight largest logits and confirm them (MUMMU_EARLY_IDS=0: route first)
-    int warm_next = 1;         // the one-launch decode form reads the next layer's router into the L2s at its end (MUMMU_WARM_NEXT=0: not)
+    int warm_next = 1;         // the one-launch decode form reads the next layer's router ahead at its end (MUMMU_WARM_NEXT=0: not)
     int tile_order = -1;       // decode launches of several tokens fetch a shared expert's rows once: -1 from six tokens on, 0 never, 1 from two (mummu_moe_set_tile_order)
     unsigned launch_salt = 0;
     // The weighted sum over a token's eight slots can be left to the launch of the NEXT device-pointer call (deferred_combine,
