@@ -192,8 +192,7 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
     }
     MUMMU_PHASE(14);
     // (the rows this launch is still waiting for have all been asked for: the next launch's router is read ahead behind them)
-    u32x4 warm_sink = {0u, 0u, 0u, 0u};
-    warm_next(lx.warm, lx.warm_bytes, warm_sink);
+    warm_next(lx.warm, lx.warm_bytes);
 
     // the other blocks of the row: thread i looks for piece i & 3 of block i >> 2
     {
@@ -259,7 +258,6 @@ __global__ __launch_bounds__(64 * kDlWaves) void decode_layer_kernel(const uint8
             }
         }
     });
-    warm_wait(warm_sink);
     MUMMU_PHASE(5);  // (the end of the kernel: overwrites the mark gate_up_tile left at its own end)
 }
 

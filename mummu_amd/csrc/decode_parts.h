@@ -275,19 +275,52 @@ __device__ __forceinline__ void pending_sum_wave(const PendingSum &ps, int hidde
 }
 
 // Reads `warm` (bytes: a multiple of 16) ahead of the launch that will want it, through the L2 of the XCD this workgroup runs on
-// (every XCD all of it, as that launch will: read by one XCD only, half of the gain is left): the workgroups of the XCD take a slice each, the last wave of
-// each asks for it, nobody uses the data.  The loads come back whenever they do, so their destination is a register set
-// the caller keeps reserved to the end of the kernel (`sink`, handed to warm_wait there): nothing else may have been given
-// those registers by then.
-__device__ __forceinline__ void warm_next(const void *warm, unsigned bytes, u32x4 &sink) {
+// (every XCD all of it, as that launch will: read by one XCD only, half of the gain is left): the workgroups of the XCD take a
+// slice each, the last wave of each asks for it (shared among all the waves it measured as no read-ahead at all), nobody
+// uses the data.  The loads of a pass - four, eight or twelve 16-byte pieces per lane, whichever covers the slice - and the
+// wait for them are ONE assembly statement: the compiler never sees a register with a load still on its way into it (it
+// would be free to give that register to something else).  The wave that waits here has nothing better to do: the hidden
+// row it is about to look for is more than a load's latency away.
+__device__ __forceinline__ void warm_next(const void *warm, unsigned bytes) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (warm == nullptr || wave != (int)(blockDim.x >> 6) - 1) return;
     const unsigned per_xcd = (gridDim.x * gridDim.y) >> 3, mine = (blockIdx.y * gridDim.x + blockIdx.x) >> 3;
     const unsigned pieces = bytes >> 4, each = (pieces + per_xcd - 1) / per_xcd;
-    for (unsigned i = mine * each + (unsigned)lane; i < (mine + 1) * each && i < pieces; i += 64)
-        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"((const u32x4 *)warm + i) : "memory");
+    const unsigned first = mine * each, end = (mine + 1) * each < pieces ? (mine + 1) * each : pieces;
+    if (first >= end) return;
+    const u32x4 *base = (const u32x4 *)warm;
+    auto at = [&](unsigned i) { return base + (i < end ? i : end - 1); };  // (a piece past the slice's end stands in for its last)
+    u32x4 sink;
+    for (unsigned i0 = first; i0 < end;) {   // (uniform over the wave)
+        const unsigned i = i0 + (unsigned)lane, left = end - i0;
+        if (left <= 256u) {
+            asm volatile("global_load_dwordx4 %0, %1, off\n\tglobal_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %0, %3, off\n\t"
+                         "global_load_dwordx4 %0, %4, off\n\ts_waitcnt vmcnt(0)"
+                         : "=&v"(sink) : "v"(at(i)), "v"(at(i + 64)), "v"(at(i + 128)), "v"(at(i + 192)) : "memory");
+            i0 += 256;
+        } else if (left <= 512u) {
+            asm volatile("global_load_dwordx4 %0, %1, off\n\tglobal_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %0, %3, off\n\t"
+                         "global_load_dwordx4 %0, %4, off\n\tglobal_load_dwordx4 %0, %5, off\n\tglobal_load_dwordx4 %0, %6, off\n\t"
+                         "global_load_dwordx4 %0, %7, off\n\tglobal_load_dwordx4 %0, %8, off\n\ts_waitcnt vmcnt(0)"
+                         : "=&v"(sink)
+                         : "v"(at(i)), "v"(at(i + 64)), "v"(at(i + 128)), "v"(at(i + 192)), "v"(at(i + 256)), "v"(at(i + 320)), "v"(at(i + 384)),
+                           "v"(at(i + 448))
+                         : "memory");
+            i0 += 512;
+        } else {
+            asm volatile("global_load_dwordx4 %0, %1, off\n\tglobal_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %0, %3, off\n\t"
+                         "global_load_dwordx4 %0, %4, off\n\tglobal_load_dwordx4 %0, %5, off\n\tglobal_load_dwordx4 %0, %6, off\n\t"
+                         "global_load_dwordx4 %0, %7, off\n\tglobal_load_dwordx4 %0, %8, off\n\tglobal_load_dwordx4 %0, %9, off\n\t"
+                         "global_load_dwordx4 %0, %10, off\n\tglobal_load_dwordx4 %0, %11, off\n\tglobal_load_dwordx4 %0, %12, off\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(sink)
+                         : "v"(at(i)), "v"(at(i + 64)), "v"(at(i + 128)), "v"(at(i + 192)), "v"(at(i + 256)), "v"(at(i + 320)), "v"(at(i + 384)),
+                           "v"(at(i + 448)), "v"(at(i + 512)), "v"(at(i + 576)), "v"(at(i + 640)), "v"(at(i + 704))
+                         : "memory");
+            i0 += 768;
+        }
+    }
 }
-__device__ __forceinline__ void warm_wait(u32x4 &sink) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory"); }
 
 // LDS a decode workgroup keeps of its token: the 16-bit row of the block's input and the routing.
 template <int JN>
